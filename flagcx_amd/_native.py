@@ -1,0 +1,84 @@
+"""ctypes bindings of include/flagcx_amd/fx_kernels.h and fx_synth.h."""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+KERNEL_LIB = os.path.join(LIB_DIR, "libflagcx_amd.so")
+PLUGIN_LIB = os.path.join(LIB_DIR, "libflagcx-device-mi355x.so")
+
+# FlagCX enum values (flagcx/include/flagcx.h:21-66)
+SUCCESS, DEVICE_ERROR, SYSTEM_ERROR, INTERNAL_ERROR, INVALID_ARGUMENT = 0, 1, 2, 3, 4
+INVALID_USAGE, IN_PROGRESS, NOT_SUPPORTED = 5, 7, 9
+DT_INT8, DT_UINT8, DT_INT32, DT_UINT32, DT_INT64, DT_UINT64 = 0, 1, 2, 3, 4, 5
+DT_FP16, DT_FP32, DT_FP64, DT_BF16 = 6, 7, 8, 9
+OP_SUM, OP_PROD, OP_MAX, OP_MIN, OP_AVG = 0, 1, 2, 3, 4
+MEMCPY_H2D, MEMCPY_D2H, MEMCPY_D2D = 0, 1, 2
+MEM_HOST, MEM_DEVICE, MEM_MANAGED = 0, 1, 2
+
+DTYPE_SIZE = {DT_INT32: 4, DT_FP32: 4, DT_FP16: 2, DT_BF16: 2}
+# host-side container dtypes: 16-bit floats travel as raw uint16 bit patterns
+NP_DTYPE = {DT_INT32: np.int32, DT_FP32: np.float32, DT_FP16: np.uint16, DT_BF16: np.uint16}
+
+
+class FlagcxError(RuntimeError):
+    def __init__(self, code, what=""):
+        super().__init__(f"flagcxResult_t={code} {what}")
+        self.code = code
+
+
+def check(rc, what=""):
+    if rc != SUCCESS:
+        raise FlagcxError(rc, what)
+    return rc
+
+
+class ReduceTrigger(C.Structure):
+    _fields_ = [("value", C.c_uint64 * 4)]
+
+
+class SliceDesc(C.Structure):
+    _fields_ = [("in_", C.c_void_p * 8), ("out", C.c_void_p), ("count", C.c_uint64)]
+
+
+def _load(path):
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} is missing: build it with `python -m flagcx_amd.build` "
+            "(hipcc, gfx950). There is no CPU fallback.")
+    return C.CDLL(path, mode=C.RTLD_GLOBAL)
+
+
+lib = _load(KERNEL_LIB)
+
+_vp, _sz, _i = C.c_void_p, C.c_size_t, C.c_int
+_SIGS = {
+    "fx_reduce_copy": (_i, [_vp, C.POINTER(_vp), _i, _sz, _i, _i, _i, _vp]),
+    "fx_reduce2": (_i, [_vp, _vp, _vp, _sz, _i, _i, _vp]),
+    "fx_trigger_set": (None, [C.POINTER(ReduceTrigger), C.c_uint64, C.c_uint64, C.c_uint64, _sz, _sz, _i, _i, _i]),
+    "fx_trigger_get": (None, [C.POINTER(ReduceTrigger)] + [C.POINTER(C.c_uint64)] * 5 + [C.POINTER(_i)] * 3),
+    "fx_reduce_triggers": (_i, [C.POINTER(ReduceTrigger), _sz, _vp]),
+    "fx_reduce_slices": (_i, [C.POINTER(SliceDesc), _sz, _i, _i, _i, _vp]),
+    "fx_copy_slices": (_i, [C.POINTER(SliceDesc), _sz, _vp]),
+    "fx_plan_create": (_i, [C.POINTER(_vp), C.POINTER(SliceDesc), _sz, _i, _i, _i]),
+    "fx_plan_launch": (_i, [_vp, _vp]),
+    "fx_plan_destroy": (_i, [_vp]),
+    "fx_pack": (_i, [_vp, _vp, C.POINTER(_sz), C.POINTER(_sz), _i, _i, _vp]),
+    "fx_unpack": (_i, [_vp, _vp, C.POINTER(_sz), C.POINTER(_sz), _i, _i, _vp]),
+    "fx_dtype_size": (_sz, [_i]),
+    "fx_split": (None, [_sz, _sz, _sz, C.POINTER(_sz), C.POINTER(_sz)]),
+    "fx_nredslices": (_sz, [_sz, _i, _sz, _sz, _sz]),
+    "fx_set_xcd_spread": (_i, [_i]),
+    "fx_version": (C.c_char_p, []),
+    "fx_synth_fill": (_i, [_vp, _sz, _i, _i, C.c_double, C.c_double, C.c_uint64, C.c_uint64, _i]),
+}
+for _name, (_res, _args) in _SIGS.items():
+    _f = getattr(lib, _name)
+    _f.restype, _f.argtypes = _res, _args
+
+
+def exported_symbols():
+    """Names this binding expects from libflagcx_amd.so (the C-ABI surface)."""
+    return sorted(_SIGS)

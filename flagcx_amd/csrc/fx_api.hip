@@ -1,0 +1,373 @@
+// C ABI over the gfx950 kernels: argument checking, batching of slice
+// descriptors into launches, and device-resident plans.
+#include <atomic>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "flagcx_amd/fx_kernels.h"
+#include "fx_launch.hpp"
+
+using namespace fx;
+
+namespace {
+
+std::atomic<int> gXcdSpread{-1};
+
+int xcdSpread() {
+  int v = gXcdSpread.load(std::memory_order_relaxed);
+  if (v < 0) {
+    const char *e = getenv("FX_XCD_SPREAD");
+    v = (e && *e) ? (atoi(e) != 0) : 0;
+    gXcdSpread.store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
+// dtype / op screening.  Types FlagCX knows but this path does not carry
+// return flagcxNotSupported so a caller can fall through to another path;
+// values outside the enums are invalid arguments.
+flagcxResult_t screen(int dtype, int op) {
+  if (dtype < 0 || dtype >= flagcxNumTypes) return flagcxInvalidArgument;
+  if (op < 0 || op >= flagcxNumRedOps) return flagcxInvalidArgument;
+  if (dtypeSize(dtype) == 0) return flagcxNotSupported;
+  if (!opSupported(op)) return flagcxNotSupported;  // flagcxAvg
+  return flagcxSuccess;
+}
+
+const KernelSet *setFor(int dtype, int op) {
+  switch (dtype) {
+    case flagcxFloat32: return &kernelSetsF32()[op];
+    case flagcxInt32: return &kernelSetsI32()[op];
+    case flagcxBfloat16: return &kernelSetsBF16()[op];
+    case flagcxFloat16: return &kernelSetsF16()[op];
+    default: return nullptr;
+  }
+}
+
+const KernelSet *copySetFor(int es) { return &kernelSetsCopy()[es == 4 ? 2 : (es == 2 ? 1 : 0)]; }
+
+bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// Validate one slice and return the number of workgroups it needs.
+flagcxResult_t sliceTiles(const fxSliceDesc &s, int k, int es, int U, uint64_t *tiles) {
+  *tiles = 0;
+  if (s.count == 0) return flagcxSuccess;
+  if (!s.out || !aligned(s.out, es)) return flagcxInvalidArgument;
+  for (int p = 0; p < k; p++)
+    if (!s.in[p] || !aligned(s.in[p], es)) return flagcxInvalidArgument;
+  *tiles = tilesFor(s.out, s.count, es, U);
+  return flagcxSuccess;
+}
+
+// Launch n slices through kernel-argument tables of up to kInlineSlices each.
+flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slices, size_t n, int k, hipStream_t s) {
+  const int U = unrollFor(k);
+  InlineSliceTable t;
+  t.n = 0;
+  t.tileStart[0] = 0;
+  for (size_t i = 0; i <= n; i++) {
+    uint64_t tiles = 0;
+    if (i < n) {
+      flagcxResult_t rc = sliceTiles(slices[i], k, ks->elemSize, U, &tiles);
+      if (rc != flagcxSuccess) return rc;
+      if (tiles == 0) continue;
+      if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+    }
+    const bool flush = (i == n) || t.n == (uint32_t)kInlineSlices ||
+                       (uint64_t)t.tileStart[t.n] + tiles > 0x7ffffff0ull;
+    if (flush && t.n > 0) {
+      flagcxResult_t rc = ks->slicesInline[k](t, s);
+      if (rc != flagcxSuccess) return rc;
+      t.n = 0;
+    }
+    if (i == n) break;
+    SliceDescDev &d = t.d[t.n];
+    for (int p = 0; p < kMaxFixedK; p++) d.in[p] = (p < k) ? slices[i].in[p] : nullptr;
+    d.out = slices[i].out;
+    d.count = slices[i].count;
+    t.tileStart[t.n + 1] = t.tileStart[t.n] + (uint32_t)tiles;
+    t.n++;
+  }
+  return flagcxSuccess;
+}
+
+// Largest power-of-two granularity (4, 2 or 1 bytes) shared by all copy slices.
+int copyGranularity(const fxSliceDesc *slices, size_t n) {
+  uintptr_t bits = 0;
+  for (size_t i = 0; i < n; i++) {
+    if (slices[i].count == 0) continue;
+    bits |= (uintptr_t)slices[i].in[0] | (uintptr_t)slices[i].out | (uintptr_t)slices[i].count;
+  }
+  return (bits & 1) ? 1 : ((bits & 2) ? 2 : 4);
+}
+
+}  // namespace
+
+struct fxPlan {
+  const KernelSet *ks;
+  SliceDescDev *dDesc;
+  uint32_t *dTileStart;
+  uint32_t n, grid;
+  int k;
+};
+
+extern "C" {
+#pragma GCC visibility push(default)
+
+const char *fx_version(void) { return "flagcx_amd 0.1 (gfx950)"; }
+
+int fx_set_xcd_spread(int mode) {
+  int prev = xcdSpread();
+  gXcdSpread.store(mode ? 1 : 0, std::memory_order_relaxed);
+  return prev;
+}
+
+size_t fx_dtype_size(int dtype) {
+  switch (dtype) {
+    case flagcxInt8:
+    case flagcxUint8: return 1;
+    case flagcxFloat16:
+    case flagcxBfloat16: return 2;
+    case flagcxInt32:
+    case flagcxUint32:
+    case flagcxFloat32: return 4;
+    case flagcxInt64:
+    case flagcxUint64:
+    case flagcxFloat64: return 8;
+    default: return 0;
+  }
+}
+
+int fx_reduce_copy(void *out, const void *const *in, int k, size_t count, int dtype, int op, int first,
+                   void *stream) {
+  flagcxResult_t rc = screen(dtype, op);
+  if (rc != flagcxSuccess) return rc;
+  if (!in || k < 1 || k > FX_MAX_INPUTS || first < 0 || first >= k) return flagcxInvalidArgument;
+  if (count == 0) return flagcxSuccess;
+  const size_t es = dtypeSize(dtype);
+  if (!out || !aligned(out, es)) return flagcxInvalidArgument;
+  const void *rot[FX_MAX_INPUTS];
+  for (int j = 0; j < k; j++) {
+    const void *p = in[(first + j) % k];
+    if (!p || !aligned(p, es)) return flagcxInvalidArgument;
+    rot[j] = p;
+  }
+  const KernelSet *ks = setFor(dtype, op);
+  return ks->direct[k <= kMaxFixedK ? k : 0](out, rot, k, count, xcdSpread(), (hipStream_t)stream);
+}
+
+int fx_reduce2(void *out, const void *in1, const void *in2, size_t count, int dtype, int op, void *stream) {
+  const void *in[2] = {in1, in2};
+  return fx_reduce_copy(out, in, 2, count, dtype, op, 0, stream);
+}
+
+void fx_trigger_set(fxReduceTrigger *t, uint64_t in1, uint64_t in2, uint64_t out, size_t count, size_t nthreads,
+                    int dtype, int op, int state) {
+  t->value[0] = in1;
+  t->value[1] = in2;
+  t->value[2] = out;
+  t->value[3] = ((uint64_t)count & 0xffffffffull) | (((uint64_t)nthreads & 0xffffull) << 32) |
+                (((uint64_t)dtype & 0xfull) << 48) | (((uint64_t)op & 0xfull) << 52) |
+                (((uint64_t)state & 0x3ull) << 56);
+}
+
+void fx_trigger_get(const fxReduceTrigger *t, uint64_t *in1, uint64_t *in2, uint64_t *out, uint64_t *count,
+                    uint64_t *nthreads, int *dtype, int *op, int *state) {
+  const uint64_t w = t->value[3];
+  if (in1) *in1 = t->value[0];
+  if (in2) *in2 = t->value[1];
+  if (out) *out = t->value[2];
+  if (count) *count = w & 0xffffffffull;
+  if (nthreads) *nthreads = (w >> 32) & 0xffffull;
+  if (dtype) *dtype = (int)((w >> 48) & 0xfull);
+  if (op) *op = (int)((w >> 52) & 0xfull);
+  if (state) *state = (int)((w >> 56) & 0x3ull);
+}
+
+int fx_reduce_slices(const fxSliceDesc *slices, size_t n, int k, int dtype, int op, void *stream) {
+  flagcxResult_t rc = screen(dtype, op);
+  if (rc != flagcxSuccess) return rc;
+  if (k < 1 || k > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
+  if (n == 0) return flagcxSuccess;
+  if (!slices) return flagcxInvalidArgument;
+  return launchSliceBatches(setFor(dtype, op), slices, n, k, (hipStream_t)stream);
+}
+
+int fx_reduce_triggers(const fxReduceTrigger *triggers, size_t n, void *stream) {
+  if (n == 0) return flagcxSuccess;
+  if (!triggers) return flagcxInvalidArgument;
+  std::vector<fxSliceDesc> run;
+  size_t i = 0;
+  while (i < n) {
+    int dtype, op;
+    fx_trigger_get(&triggers[i], nullptr, nullptr, nullptr, nullptr, nullptr, &dtype, &op, nullptr);
+    run.clear();
+    size_t j = i;
+    for (; j < n; j++) {
+      uint64_t a, b, o, c;
+      int dt, rop;
+      fx_trigger_get(&triggers[j], &a, &b, &o, &c, nullptr, &dt, &rop, nullptr);
+      if (dt != dtype || rop != op) break;
+      fxSliceDesc d;
+      memset(&d, 0, sizeof(d));
+      d.in[0] = (const void *)(uintptr_t)a;
+      d.in[1] = (const void *)(uintptr_t)b;
+      d.out = (void *)(uintptr_t)o;
+      d.count = c;
+      run.push_back(d);
+    }
+    int rc = fx_reduce_slices(run.data(), run.size(), 2, dtype, op, stream);
+    if (rc != flagcxSuccess) return rc;
+    i = j;
+  }
+  return flagcxSuccess;
+}
+
+int fx_copy_slices(const fxSliceDesc *slices, size_t n, void *stream) {
+  if (n == 0) return flagcxSuccess;
+  if (!slices) return flagcxInvalidArgument;
+  for (size_t i = 0; i < n; i++)
+    if (slices[i].count && (!slices[i].in[0] || !slices[i].out)) return flagcxInvalidArgument;
+  const int es = copyGranularity(slices, n);
+  std::vector<fxSliceDesc> el(slices, slices + n);
+  for (auto &d : el) d.count /= (uint64_t)es;
+  return launchSliceBatches(copySetFor(es), el.data(), n, 1, (hipStream_t)stream);
+}
+
+int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, int dtype, int op) {
+  if (!plan) return flagcxInvalidArgument;
+  *plan = nullptr;
+  if (n && !slices) return flagcxInvalidArgument;
+  if (n > 0x7fffffffull) return flagcxInvalidArgument;
+  const KernelSet *ks;
+  uint64_t div = 1;
+  if (op == -1) {
+    k = 1;
+    for (size_t i = 0; i < n; i++)
+      if (slices[i].count && (!slices[i].in[0] || !slices[i].out)) return flagcxInvalidArgument;
+    int es = copyGranularity(slices, n);
+    ks = copySetFor(es);
+    div = (uint64_t)es;
+  } else {
+    flagcxResult_t rc = screen(dtype, op);
+    if (rc != flagcxSuccess) return rc;
+    if (k < 1 || k > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
+    ks = setFor(dtype, op);
+  }
+  const int U = unrollFor(k);
+  std::vector<SliceDescDev> desc;
+  std::vector<uint32_t> start(1, 0u);
+  for (size_t i = 0; i < n; i++) {
+    fxSliceDesc s = slices[i];
+    s.count /= div;
+    uint64_t tiles;
+    flagcxResult_t rc = sliceTiles(s, k, ks->elemSize, U, &tiles);
+    if (rc != flagcxSuccess) return rc;
+    if (tiles == 0) continue;
+    if ((uint64_t)start.back() + tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+    SliceDescDev d;
+    for (int p = 0; p < kMaxFixedK; p++) d.in[p] = (p < k) ? s.in[p] : nullptr;
+    d.out = s.out;
+    d.count = s.count;
+    desc.push_back(d);
+    start.push_back(start.back() + (uint32_t)tiles);
+  }
+  fxPlan *pl = new (std::nothrow) fxPlan();
+  if (!pl) return flagcxSystemError;
+  pl->ks = ks;
+  pl->k = k;
+  pl->n = (uint32_t)desc.size();
+  pl->grid = start.back();
+  pl->dDesc = nullptr;
+  pl->dTileStart = nullptr;
+  if (pl->n) {
+    if (hipMalloc((void **)&pl->dDesc, desc.size() * sizeof(SliceDescDev)) != hipSuccess ||
+        hipMalloc((void **)&pl->dTileStart, start.size() * sizeof(uint32_t)) != hipSuccess ||
+        hipMemcpy(pl->dDesc, desc.data(), desc.size() * sizeof(SliceDescDev), hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(pl->dTileStart, start.data(), start.size() * sizeof(uint32_t), hipMemcpyHostToDevice) !=
+            hipSuccess) {
+      fx_plan_destroy(pl);
+      return flagcxUnhandledDeviceError;
+    }
+  }
+  *plan = pl;
+  return flagcxSuccess;
+}
+
+int fx_plan_launch(fxPlan_t plan, void *stream) {
+  if (!plan) return flagcxInvalidArgument;
+  if (plan->n == 0) return flagcxSuccess;
+  return plan->ks->slicesTable[plan->k](plan->dDesc, plan->dTileStart, plan->n, plan->grid, (hipStream_t)stream);
+}
+
+int fx_plan_destroy(fxPlan_t plan) {
+  if (!plan) return flagcxSuccess;
+  if (plan->dDesc) (void)hipFree(plan->dDesc);
+  if (plan->dTileStart) (void)hipFree(plan->dTileStart);
+  delete plan;
+  return flagcxSuccess;
+}
+
+static int packOrUnpack(bool pack, void *a, const void *b, const size_t *counts, const size_t *displs, int npeers,
+                        int dtype, void *stream) {
+  if (npeers < 0) return flagcxInvalidArgument;
+  const size_t es = fx_dtype_size(dtype);
+  if (es == 0) return flagcxInvalidArgument;
+  if (npeers == 0) return flagcxSuccess;
+  if (!counts || !displs) return flagcxInvalidArgument;
+  std::vector<fxSliceDesc> sl;
+  size_t slot = 0;
+  for (int i = 0; i < npeers; i++) {
+    if (counts[i]) {
+      if (!a || !b) return flagcxInvalidArgument;
+      fxSliceDesc d;
+      memset(&d, 0, sizeof(d));
+      if (pack) {  // a = packed, b = sendbuff
+        d.in[0] = (const char *)b + displs[i] * es;
+        d.out = (char *)a + slot * es;
+      } else {     // a = recvbuff, b = packed
+        d.in[0] = (const char *)b + slot * es;
+        d.out = (char *)a + displs[i] * es;
+      }
+      d.count = counts[i] * es;
+      sl.push_back(d);
+    }
+    slot += counts[i];
+  }
+  return fx_copy_slices(sl.data(), sl.size(), stream);
+}
+
+int fx_pack(void *packed, const void *sendbuff, const size_t *sendcounts, const size_t *sdispls, int npeers,
+            int dtype, void *stream) {
+  return packOrUnpack(true, packed, sendbuff, sendcounts, sdispls, npeers, dtype, stream);
+}
+
+int fx_unpack(void *recvbuff, const void *packed, const size_t *recvcounts, const size_t *rdispls, int npeers,
+              int dtype, void *stream) {
+  return packOrUnpack(false, recvbuff, packed, recvcounts, rdispls, npeers, dtype, stream);
+}
+
+void fx_split(size_t total, size_t parts, size_t idx, size_t *cnt, size_t *off) {
+  if (parts == 0) {
+    if (cnt) *cnt = 0;
+    if (off) *off = 0;
+    return;
+  }
+  const size_t base = total / parts, rem = total % parts;
+  if (cnt) *cnt = base + (idx < rem ? 1 : 0);
+  if (off) *off = idx * base + (idx < rem ? idx : rem);
+}
+
+size_t fx_nredslices(size_t count, int nranks, size_t nslices, size_t nredslices, size_t redslicesize) {
+  if (nredslices != 0) return nredslices;
+  if (count == 0 || redslicesize == 0 || nranks < 1 || nslices == 0) return 1;
+  float v = (float)count / nranks / nslices / redslicesize;
+  size_t r = (size_t)ceilf(v);
+  return r ? r : 1;
+}
+
+#pragma GCC visibility pop
+}  // extern "C"

@@ -1,0 +1,120 @@
+// Host-side launch tables for the reduce / copy kernel family.  One
+// translation unit per element type instantiates a KernelSet per reduction
+// op; the C-ABI layer picks the entry for (dtype, op, k) at run time.
+#pragma once
+#include "fx_reduce_body.hpp"
+
+namespace fx {
+
+// Vectors per lane per input: keep roughly 8..16 independent 16-byte loads in
+// flight per lane whatever the input count.
+constexpr int unrollFor(int K) { return K == 0 ? 2 : (K == 1 ? 8 : (K <= 4 ? 4 : 2)); }
+
+struct KernelSet {
+  // index = compile-time input count, 0 = runtime-k kernel
+  flagcxResult_t (*direct[kMaxFixedK + 1])(void *out, const void *const *in, int k, uint64_t count,
+                                           int xcdSpread, hipStream_t s);
+  flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const InlineSliceTable &t, hipStream_t s);
+  flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
+                                                uint32_t grid, hipStream_t s);
+  int elemSize;
+};
+
+// Tiles (workgroups) a segment of `count` elements needs with unroll U.
+inline uint64_t tilesFor(const void *out, uint64_t count, int es, int U) {
+  uint64_t nv = segVectors((uint64_t)(uintptr_t)out & 15u, count, es);
+  return (nv + (uint64_t)U * kBlock - 1) / ((uint64_t)U * kBlock);
+}
+
+template <class R, int K>
+flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t count, int xcdSpread, hipStream_t s) {
+  constexpr int U = unrollFor(K);
+  DirectArgs<K> a;
+  const int kk = (K > 0) ? K : k;
+  for (int p = 0; p < kk; p++) a.in[p] = in[p];
+  a.out = out;
+  a.count = count;
+  a.k = kk;
+  uint64_t ntiles = tilesFor(out, count, R::ES, U);
+  if (ntiles == 0) return flagcxSuccess;
+  if (ntiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+  a.ntiles = (uint32_t)ntiles;
+  a.xcdSpread = (xcdSpread && ntiles >= 64) ? 1 : 0;
+  uint32_t grid = a.xcdSpread ? (uint32_t)((ntiles + 7) / 8 * 8) : (uint32_t)ntiles;
+  hipLaunchKernelGGL((reduceCopyDirect<R, K, U>), dim3(grid), dim3(kBlock), 0, s, a);
+  FX_HIP(hipGetLastError());
+  return flagcxSuccess;
+}
+
+template <class R, int K>
+flagcxResult_t launchSlicesInline(const InlineSliceTable &t, hipStream_t s) {
+  constexpr int U = unrollFor(K);
+  uint32_t grid = t.tileStart[t.n];
+  if (grid == 0) return flagcxSuccess;
+  hipLaunchKernelGGL((reduceSlicesInline<R, K, U>), dim3(grid), dim3(kBlock), 0, s, t);
+  FX_HIP(hipGetLastError());
+  return flagcxSuccess;
+}
+
+template <class R, int K>
+flagcxResult_t launchSlicesTable(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n, uint32_t grid,
+                                 hipStream_t s) {
+  constexpr int U = unrollFor(K);
+  if (grid == 0) return flagcxSuccess;
+  hipLaunchKernelGGL((reduceSlicesTable<R, K, U>), dim3(grid), dim3(kBlock), 0, s, d, tileStart, n);
+  FX_HIP(hipGetLastError());
+  return flagcxSuccess;
+}
+
+template <class R, int K>
+void fillSet(KernelSet &ks) {
+  ks.direct[K] = &launchDirect<R, K>;
+  if (K > 0) {
+    ks.slicesInline[K] = &launchSlicesInline<R, (K > 0 ? K : 1)>;
+    ks.slicesTable[K] = &launchSlicesTable<R, (K > 0 ? K : 1)>;
+  } else {
+    ks.slicesInline[0] = nullptr;
+    ks.slicesTable[0] = nullptr;
+  }
+}
+
+template <class R>
+KernelSet makeSet() {
+  KernelSet ks;
+  fillSet<R, 0>(ks);
+  fillSet<R, 1>(ks);
+  fillSet<R, 2>(ks);
+  fillSet<R, 3>(ks);
+  fillSet<R, 4>(ks);
+  fillSet<R, 5>(ks);
+  fillSet<R, 6>(ks);
+  fillSet<R, 7>(ks);
+  fillSet<R, 8>(ks);
+  ks.elemSize = R::ES;
+  return ks;
+}
+
+// Only k = 1 is meaningful for the byte mover.
+template <int ES>
+KernelSet makeCopySet() {
+  KernelSet ks = {};
+  fillSet<CopyRed<ES>, 1>(ks);
+  ks.elemSize = ES;
+  return ks;
+}
+
+template <int DT>
+const KernelSet *makeSets() {
+  static const KernelSet sets[4] = {makeSet<Red<DT, flagcxSum>>(), makeSet<Red<DT, flagcxProd>>(),
+                                    makeSet<Red<DT, flagcxMax>>(), makeSet<Red<DT, flagcxMin>>()};
+  return sets;
+}
+
+// Defined one per translation unit (fx_reduce_<type>.hip, fx_copy.hip).
+const KernelSet *kernelSetsF32();
+const KernelSet *kernelSetsI32();
+const KernelSet *kernelSetsBF16();
+const KernelSet *kernelSetsF16();
+const KernelSet *kernelSetsCopy();  // index log2(ES): 0 -> 1 byte, 1 -> 2, 2 -> 4
+
+}  // namespace fx

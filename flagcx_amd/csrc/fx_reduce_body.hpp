@@ -1,0 +1,458 @@
+// Device code of the k-way element-wise reduce-copy for gfx950 (wave64).
+//
+// Arithmetic contract (order follows FlagCX's peer loop,
+// flagcx/adaptor/kernel/nvidia/custom_allreduce.cu:345-359):
+//   acc = in[0]; acc = acc (op) in[p] for p = 1..k-1, left to right.
+//   fp32: plain IEEE single arithmetic.  int32: sum/prod wrap modulo 2^32.
+//   bf16/fp16 sum and prod: every input widened to fp32, accumulated in fp32,
+//   rounded to nearest even once.  max = (acc < x) ? x : acc and
+//   min = (x < acc) ? x : acc (the std::max / std::min of
+//   flagcx/service/include/utils.h:707-725: ties and NaN keep the earlier
+//   operand); for 16-bit types the chosen input's own bits are returned.
+//
+// Data movement: one 16-byte vector per lane per input, U vectors per lane in
+// flight per input, all K*U loads issued before the first use.  The index
+// space is anchored at the output pointer rounded down to 16 bytes, so stores
+// are always whole aligned vectors except in the first and last vector of a
+// segment, which fall back to element accesses.  Inputs that share the
+// output's misalignment take the vector-load path; others are gathered
+// element by element (coalesced across lanes, still one pass).
+#pragma once
+#include "fx_common.hpp"
+
+namespace fx {
+
+// ------------------------------------------------------------------ reducers
+
+template <int OP>
+__device__ __forceinline__ float opF32(float a, float b) {
+  if (OP == flagcxSum) return a + b;
+  if (OP == flagcxProd) return a * b;
+  if (OP == flagcxMax) return (a < b) ? b : a;
+  return (b < a) ? b : a;
+}
+
+template <int OP>
+__device__ __forceinline__ uint32_t opI32(uint32_t a, uint32_t b) {
+  if (OP == flagcxSum) return a + b;
+  if (OP == flagcxProd) return a * b;
+  if (OP == flagcxMax) return ((int32_t)a < (int32_t)b) ? b : a;
+  return ((int32_t)b < (int32_t)a) ? b : a;
+}
+
+// fp32 -> bf16 bits in the TOP half of the result (low half is garbage):
+// round to nearest even; NaN keeps its sign/payload with the quiet bit forced.
+__device__ __forceinline__ uint32_t roundBf16Top(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);
+  return ((u & 0x7fffffffu) > 0x7f800000u) ? (u | 0x00400000u) : r;
+}
+
+__device__ __forceinline__ float halfToF32(uint32_t bits16) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+}
+__device__ __forceinline__ uint32_t f32ToHalf(float f) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+template <int DT, int OP>
+struct Red;
+
+template <int OP>
+struct Red<flagcxFloat32, OP> {
+  static constexpr int ES = 4;  // element bytes
+  struct Acc {
+    float a[4];
+  };
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) c.a[i] = __uint_as_float(v[i]);
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) c.a[i] = opF32<OP>(c.a[i], __uint_as_float(v[i]));
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = __float_as_uint(c.a[i]);
+    return r;
+  }
+};
+
+template <int OP>
+struct Red<flagcxInt32, OP> {
+  static constexpr int ES = 4;
+  struct Acc {
+    uint32_t a[4];
+  };
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) c.a[i] = v[i];
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) c.a[i] = opI32<OP>(c.a[i], v[i]);
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = c.a[i];
+    return r;
+  }
+};
+
+// bf16: widening is a shift, so for max/min the accumulator's top half IS the
+// selected input's bit pattern and no rounding is needed.
+template <int OP>
+struct Red<flagcxBfloat16, OP> {
+  static constexpr int ES = 2;
+  struct Acc {
+    float a[8];
+  };
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      c.a[2 * i] = __uint_as_float(v[i] << 16);
+      c.a[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      c.a[2 * i] = opF32<OP>(c.a[2 * i], __uint_as_float(v[i] << 16));
+      c.a[2 * i + 1] = opF32<OP>(c.a[2 * i + 1], __uint_as_float(v[i] & 0xffff0000u));
+    }
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t lo, hi;
+      if (OP == flagcxSum || OP == flagcxProd) {
+        lo = roundBf16Top(c.a[2 * i]);
+        hi = roundBf16Top(c.a[2 * i + 1]);
+      } else {
+        lo = __float_as_uint(c.a[2 * i]);
+        hi = __float_as_uint(c.a[2 * i + 1]);
+      }
+      r[i] = (hi & 0xffff0000u) | (lo >> 16);
+    }
+    return r;
+  }
+};
+
+// fp16: widened with the hardware converter (exact); max/min also carry the
+// raw 16-bit pattern of the current winner so the output is bit-preserving.
+template <int OP>
+struct Red<flagcxFloat16, OP> {
+  static constexpr int ES = 2;
+  static constexpr bool kSelect = (OP == flagcxMax || OP == flagcxMin);
+  struct Acc {
+    float a[8];
+    uint32_t b[kSelect ? 8 : 1];
+  };
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t lo = v[i] & 0xffffu, hi = v[i] >> 16;
+      c.a[2 * i] = halfToF32(lo);
+      c.a[2 * i + 1] = halfToF32(hi);
+      if (kSelect) {
+        c.b[2 * i] = lo;
+        c.b[2 * i + 1] = hi;
+      }
+    }
+  }
+  static __device__ __forceinline__ void fold1(Acc &c, int i, uint32_t bits) {
+    float x = halfToF32(bits);
+    if (kSelect) {
+      bool take = (OP == flagcxMax) ? (c.a[i] < x) : (x < c.a[i]);
+      c.a[i] = take ? x : c.a[i];
+      c.b[i] = take ? bits : c.b[i];
+    } else {
+      c.a[i] = opF32<OP>(c.a[i], x);
+    }
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      fold1(c, 2 * i, v[i] & 0xffffu);
+      fold1(c, 2 * i + 1, v[i] >> 16);
+    }
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t lo, hi;
+      if (kSelect) {
+        lo = c.b[2 * i];
+        hi = c.b[2 * i + 1];
+      } else {
+        lo = f32ToHalf(c.a[2 * i]);
+        hi = f32ToHalf(c.a[2 * i + 1]);
+      }
+      r[i] = (hi << 16) | lo;
+    }
+    return r;
+  }
+};
+
+// Plain byte mover with ES-byte granularity (ES = 1, 2 or 4), used with k = 1
+// for the all-gather copy phase and the alltoallv pack / unpack.
+template <int ESZ>
+struct CopyRed {
+  static constexpr int ES = ESZ;
+  struct Acc {
+    u32x4 v;
+  };
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) { c.v = v; }
+  static __device__ __forceinline__ void fold(Acc &, u32x4) {}
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) { return c.v; }
+};
+
+// ------------------------------------------------------------- one segment
+
+// A segment in the output-anchored index space.  Element v of the space lives
+// at base + v*ES; valid elements are [lead, end).  outBase is 16-byte aligned.
+template <int K>
+struct Seg {
+  const char *in[K];
+  char *out;
+  uint64_t lead, end;
+  bool coAligned;   // every input is 16-byte aligned like out
+  __device__ __forceinline__ const char *inp(int p) const { return in[p]; }
+  __device__ __forceinline__ int inputs() const { return K; }
+};
+
+// Runtime-k variant: the pointer table stays where it is (kernel argument
+// block) and is read through scalar loads instead of being copied.
+template <>
+struct Seg<0> {
+  const void *const *raw;
+  uint64_t mis;
+  char *out;
+  uint64_t lead, end;
+  int k;
+  bool coAligned;
+  __device__ __forceinline__ const char *inp(int p) const { return (const char *)raw[p] - mis; }
+  __device__ __forceinline__ int inputs() const { return k; }
+};
+
+template <int ES>
+__device__ __forceinline__ u32x4 gatherElems(const char *base, uint64_t e0, int lo, int hi) {
+  constexpr int VE = 16 / ES;
+  u32x4 r = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int s = 0; s < VE; s++) {
+    if (s >= lo && s < hi) {
+      if (ES == 4) {
+        r[s] = *reinterpret_cast<const uint32_t *>(base + (e0 + s) * 4);
+      } else if (ES == 2) {
+        uint32_t h = *reinterpret_cast<const uint16_t *>(base + (e0 + s) * 2);
+        r[s / 2] |= h << (16 * (s & 1));
+      } else {
+        uint32_t h = *reinterpret_cast<const uint8_t *>(base + e0 + s);
+        r[s / 4] |= h << (8 * (s & 3));
+      }
+    }
+  }
+  return r;
+}
+
+template <int ES>
+__device__ __forceinline__ void scatterElems(char *base, uint64_t e0, int lo, int hi, u32x4 v) {
+  constexpr int VE = 16 / ES;
+#pragma unroll
+  for (int s = 0; s < VE; s++) {
+    if (s >= lo && s < hi) {
+      if (ES == 4)
+        *reinterpret_cast<uint32_t *>(base + (e0 + s) * 4) = v[s];
+      else if (ES == 2)
+        *reinterpret_cast<uint16_t *>(base + (e0 + s) * 2) = (uint16_t)(v[s / 2] >> (16 * (s & 1)));
+      else
+        *reinterpret_cast<uint8_t *>(base + e0 + s) = (uint8_t)(v[s / 4] >> (8 * (s & 3)));
+    }
+  }
+}
+
+// Reduce vector j of the segment with full bounds / alignment handling.
+template <class R, int K>
+__device__ __forceinline__ void reduceVectorChecked(const Seg<K> &sg, uint64_t j) {
+  constexpr int VE = 16 / R::ES;
+  const uint64_t e0 = j * VE;
+  if (e0 >= sg.end || e0 + VE <= sg.lead) return;
+  const int lo = (sg.lead > e0) ? (int)(sg.lead - e0) : 0;
+  const int hi = (sg.end - e0 < (uint64_t)VE) ? (int)(sg.end - e0) : VE;
+  const bool full = (lo == 0 && hi == VE);
+  const bool vec = full && sg.coAligned;
+  typename R::Acc acc;
+  const int k = sg.inputs();
+  R::init(acc, vec ? ldg_stream(sg.inp(0) + j * 16) : gatherElems<R::ES>(sg.inp(0), e0, lo, hi));
+  for (int p = 1; p < k; p++)
+    R::fold(acc, vec ? ldg_stream(sg.inp(p) + j * 16) : gatherElems<R::ES>(sg.inp(p), e0, lo, hi));
+  u32x4 r = R::finish(acc);
+  if (full)
+    stg_stream(sg.out + j * 16, r);
+  else
+    scatterElems<R::ES>(sg.out, e0, lo, hi, r);
+}
+
+// One tile = U * kBlock vectors.  Interior tiles of co-aligned segments run the
+// branch-free path with all K*U loads in flight.
+template <class R, int K, int U>
+__device__ __forceinline__ void reduceTile(const Seg<K> &sg, uint64_t tile) {
+  constexpr int VE = 16 / R::ES;
+  const uint64_t j0 = tile * (uint64_t)(U * kBlock);
+  const uint64_t firstFull = (sg.lead + VE - 1) / VE;
+  const uint64_t endFull = sg.end / VE;
+  const bool interior = sg.coAligned && j0 >= firstFull && j0 + U * kBlock <= endFull;
+  if (interior) {
+    const uint64_t off = (j0 + threadIdx.x) * 16;
+    if (K > 0) {
+      u32x4 v[U][K > 0 ? K : 1];
+#pragma unroll
+      for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int p = 0; p < K; p++) v[u][p] = ldg_stream(sg.inp(p) + off + (uint64_t)u * (kBlock * 16));
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        typename R::Acc acc;
+        R::init(acc, v[u][0]);
+#pragma unroll
+        for (int p = 1; p < K; p++) R::fold(acc, v[u][p]);
+        stg_stream(sg.out + off + (uint64_t)u * (kBlock * 16), R::finish(acc));
+      }
+    } else {
+      typename R::Acc acc[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) R::init(acc[u], ldg_stream(sg.inp(0) + off + (uint64_t)u * (kBlock * 16)));
+      for (int p = 1; p < sg.inputs(); p++) {
+        const char *ip = sg.inp(p);
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = ldg_stream(ip + off + (uint64_t)u * (kBlock * 16));
+#pragma unroll
+        for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++) stg_stream(sg.out + off + (uint64_t)u * (kBlock * 16), R::finish(acc[u]));
+    }
+  } else {
+#pragma unroll 1
+    for (int u = 0; u < U; u++) reduceVectorChecked<R, K>(sg, j0 + (uint64_t)u * kBlock + threadIdx.x);
+  }
+}
+
+// Build the output-anchored segment from raw element pointers.
+template <int ES, int K>
+__device__ __forceinline__ void makeSeg(Seg<K> &sg, const void *const *in, void *out, uint64_t count, int) {
+  const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
+  sg.out = (char *)out - mis;
+  sg.lead = mis / ES;
+  sg.end = sg.lead + count;
+  bool co = true;
+#pragma unroll
+  for (int p = 0; p < K; p++) {
+    co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
+    sg.in[p] = (const char *)in[p] - mis;
+  }
+  sg.coAligned = co;
+}
+
+template <int ES>
+__device__ __forceinline__ void makeSeg(Seg<0> &sg, const void *const *in, void *out, uint64_t count, int k) {
+  const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
+  sg.raw = in;
+  sg.mis = mis;
+  sg.out = (char *)out - mis;
+  sg.lead = mis / ES;
+  sg.end = sg.lead + count;
+  sg.k = k;
+  bool co = true;
+  for (int p = 0; p < k; p++) co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
+  sg.coAligned = co;
+}
+
+// Vectors spanned by a segment of `count` elements whose output pointer has
+// byte misalignment `mis` (host and device use the same formula).
+__host__ __device__ inline uint64_t segVectors(uint64_t mis, uint64_t count, int es) {
+  return (mis + count * (uint64_t)es + 15u) / 16u;
+}
+
+// --------------------------------------------------------- kernel arguments
+
+template <int K>
+struct DirectArgs {
+  const void *in[K > 0 ? K : kMaxK];
+  void *out;
+  uint64_t count;
+  uint32_t ntiles;
+  int k;
+  int xcdSpread;   // 1: consecutive tiles of one XCD are contiguous in memory
+};
+
+// Workgroups are dealt round-robin to the 8 XCDs.  With xcdSpread the tile
+// index is rearranged so that each XCD walks one contiguous eighth of the
+// segment instead of every eighth tile.
+__device__ __forceinline__ uint32_t tileOfBlock(uint32_t b, uint32_t ntiles, int xcdSpread) {
+  if (!xcdSpread) return b;
+  const uint32_t per = (ntiles + 7u) / 8u;
+  return (b & 7u) * per + (b >> 3);
+}
+
+template <class R, int K, int U>
+__global__ void __launch_bounds__(kBlock) reduceCopyDirect(DirectArgs<K> a) {
+  Seg<K> sg;
+  makeSeg<R::ES>(sg, a.in, a.out, a.count, a.k);
+  const uint32_t t = tileOfBlock(blockIdx.x, a.ntiles, a.xcdSpread);
+  if (t < a.ntiles) reduceTile<R, K, U>(sg, t);
+}
+
+// Batched slices: a table of independent segments sharing dtype, op and k.
+// tileStart[i] is the first workgroup of slice i, tileStart[n] the grid size.
+struct SliceDescDev {
+  const void *in[kMaxFixedK];
+  void *out;
+  uint64_t count;
+};
+
+constexpr int kInlineSlices = 32;  // slices carried in the kernel argument block
+
+struct InlineSliceTable {
+  SliceDescDev d[kInlineSlices];
+  uint32_t tileStart[kInlineSlices + 1];
+  uint32_t n;
+};
+
+__device__ __forceinline__ uint32_t findSlice(const uint32_t *tileStart, uint32_t n, uint32_t b) {
+  uint32_t lo = 0, hi = n;  // invariant: tileStart[lo] <= b < tileStart[hi]
+  while (hi - lo > 1) {
+    uint32_t mid = (lo + hi) >> 1;
+    if (tileStart[mid] <= b) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+template <class R, int K, int U>
+__device__ __forceinline__ void reduceSlicesBody(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n) {
+  const uint32_t b = blockIdx.x;
+  const uint32_t i = findSlice(tileStart, n, b);
+  Seg<K> sg;
+  makeSeg<R::ES>(sg, d[i].in, d[i].out, d[i].count, K);
+  reduceTile<R, K, U>(sg, b - tileStart[i]);
+}
+
+template <class R, int K, int U>
+__global__ void __launch_bounds__(kBlock) reduceSlicesInline(InlineSliceTable t) {
+  reduceSlicesBody<R, K, U>(t.d, t.tileStart, t.n);
+}
+
+template <class R, int K, int U>
+__global__ void __launch_bounds__(kBlock)
+reduceSlicesTable(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n) {
+  reduceSlicesBody<R, K, U>(d, tileStart, n);
+}
+
+}  // namespace fx

@@ -1,0 +1,151 @@
+/*
+ * C ABI of the MI355X (gfx950) reduce / slice / pack kernel layer.
+ *
+ * Plain pointers and sizes only.  Every function returns a flagcxResult_t
+ * value (0 = flagcxSuccess, 1 = device error, 4 = invalid argument,
+ * 9 = not supported -- callers fall through on 9 exactly as FlagCX does,
+ * flagcx/flagcx.cc:2673-2680).  `stream` is a raw hipStream_t (NULL = the
+ * default stream); all launches are enqueue-only.  dtype / op are FlagCX enum
+ * values (flagcx/include/flagcx.h:36-66): int32 = 2, fp16 = 6, fp32 = 7,
+ * bf16 = 9; sum = 0, prod = 1, max = 2, min = 3.
+ */
+#ifndef FLAGCX_AMD_FX_KERNELS_H_
+#define FLAGCX_AMD_FX_KERNELS_H_
+
+#include "flagcx_amd/fx_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FX_MAX_INPUTS 64      /* k accepted by fx_reduce_copy            */
+#define FX_MAX_SLICE_INPUTS 8 /* k accepted by the slice descriptors     */
+
+/*
+ * k-way element-wise reduce-copy over peer buffers:
+ *   out[i] = in[first][i] (op) in[(first+1)%k][i] (op) ... left to right.
+ * Replaces lsa_reduce + flagcxLsaAllReduceKernel
+ * (flagcx/adaptor/kernel/nvidia/custom_allreduce.cu:337-394) including the
+ * tail the reference drops (:383-384) and unaligned buffers it rejects
+ * (:633-635).  bf16/fp16 sum/prod accumulate in fp32 and round once.
+ * `in` is a host array of k device pointers; out may equal any in[p]
+ * (in-place), partial overlap is undefined.  first = 0 is the reference order;
+ * another value gives the rotated order a ring produces for that chunk.
+ */
+int fx_reduce_copy(void *out, const void *const *in, int k, size_t count,
+                   int dtype, int op, int first, void *stream);
+
+/*
+ * Two-input slice reduce out = in1 (op) in2, for every dtype / op.  Replaces
+ * the device function flagcxReduceKernel
+ * (flagcx/adaptor/kernel/nvidia/flagcx_reduce_kernel_device.cu:75-86), which
+ * is fp32-sum only.  out may alias in1 (ring: output == input1).
+ */
+int fx_reduce2(void *out, const void *in1, const void *in2, size_t count,
+               int dtype, int op, void *stream);
+
+/*
+ * The reference's 32-byte slice descriptor, bit for bit
+ * (flagcx/include/flagcx_kernel_core.h:146-162,209-230): value[0..2] = in1,
+ * in2, out; value[3] = count[31:0] | nthreads[47:32] | datatype[51:48] |
+ * redop[55:52] | state[57:56].
+ */
+typedef struct fxReduceTrigger {
+  uint64_t value[4];
+} fxReduceTrigger;
+
+enum {
+  fxTriggerAvailable = 0,
+  fxTriggerEnqueued = 1,
+  fxTriggerInprogress = 2,
+  fxTriggerComplete = 3
+};
+
+/* flagcxReduceTrigger::setValue (flagcx/core/flagcx_reduce_kernel_host.cc:6-26) */
+void fx_trigger_set(fxReduceTrigger *t, uint64_t in1, uint64_t in2,
+                    uint64_t out, size_t count, size_t nthreads, int dtype,
+                    int op, int state);
+/* the device-side getters (flagcx_reduce_kernel_device.cu:15-43) */
+void fx_trigger_get(const fxReduceTrigger *t, uint64_t *in1, uint64_t *in2,
+                    uint64_t *out, uint64_t *count, uint64_t *nthreads,
+                    int *dtype, int *op, int *state);
+
+/*
+ * Execute n triggers (host array) as batched launches: the stream-ordered
+ * replacement of the polling consumer flagcxCollectiveKernel
+ * (flagcx_reduce_kernel_device.cu:88-186).  Consecutive triggers with equal
+ * dtype/op share a launch; triggers of one launch must not depend on each
+ * other.  nthreads and state fields are ignored.
+ */
+int fx_reduce_triggers(const fxReduceTrigger *triggers, size_t n, void *stream);
+
+/* k-way slice descriptor: up to 8 inputs, `count` elements. */
+typedef struct fxSliceDesc {
+  const void *in[FX_MAX_SLICE_INPUTS];
+  void *out;
+  uint64_t count;
+} fxSliceDesc;
+
+/*
+ * Reduce n independent slices (host array), each k-way in input order, with
+ * as few launches as possible.  This is what the chunk / slice / red-slice
+ * partition of flagcx/runner/uni_runner_impl.cc:661-1007 feeds: one descriptor
+ * per reduce node.
+ */
+int fx_reduce_slices(const fxSliceDesc *slices, size_t n, int k, int dtype,
+                     int op, void *stream);
+
+/*
+ * Copy n independent byte ranges (in[0] -> out, `count` = BYTES): the Cpy node
+ * and the all-gather landing copies (uni_runner_impl.cc:322-344,1649-1662;
+ * flagcx/core/p2p.cc:257-283) as one launch.
+ */
+int fx_copy_slices(const fxSliceDesc *slices, size_t n, void *stream);
+
+/*
+ * Device-resident descriptor tables for plans that are launched repeatedly.
+ * Creation uploads synchronously; launch is enqueue-only.  op = -1 makes a
+ * copy plan (count in bytes, dtype ignored, k = 1).
+ */
+typedef struct fxPlan *fxPlan_t;
+int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k,
+                   int dtype, int op);
+int fx_plan_launch(fxPlan_t plan, void *stream);
+int fx_plan_destroy(fxPlan_t plan);
+
+/*
+ * alltoallv pack: gather npeers segments of sendbuff (element displacements
+ * sdispls[i], element counts sendcounts[i]; host arrays) into contiguous
+ * slots of `packed`, slot_i = sum_{j<i} sendcounts[j].  unpack is the inverse
+ * scatter into recvbuff at rdispls[i].  Segment addressing is that of
+ * flagcx/service/bootstrap.cc:1253-1258 and flagcx/runner/uni_runner.cc:197-210;
+ * zero counts are skipped (flagcx/adaptor/include/adaptor.h:77).
+ */
+int fx_pack(void *packed, const void *sendbuff, const size_t *sendcounts,
+            const size_t *sdispls, int npeers, int dtype, void *stream);
+int fx_unpack(void *recvbuff, const void *packed, const size_t *recvcounts,
+              const size_t *rdispls, int npeers, int dtype, void *stream);
+
+/* getFlagcxDataTypeSize (flagcx/flagcx.cc:35-66) for every FlagCX dtype. */
+size_t fx_dtype_size(int dtype);
+
+/*
+ * Remainder-balanced split used (nested) for rank chunks, slices and
+ * red-slices (uni_runner_impl.cc:100-131,433-457,854-866); offsets in elements.
+ */
+void fx_split(size_t total, size_t parts, size_t idx, size_t *cnt, size_t *off);
+
+/* Automatic red-slice count, single-precision as in uni_runner_impl.cc:694-701. */
+size_t fx_nredslices(size_t count, int nranks, size_t nslices,
+                     size_t nredslices, size_t redslicesize);
+
+/* Tuning knob for measurements: 0 = tiles in launch order, 1 = each XCD walks
+ * a contiguous eighth of the buffer.  Returns the previous value. */
+int fx_set_xcd_spread(int mode);
+
+const char *fx_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLAGCX_AMD_FX_KERNELS_H_ */

@@ -1,0 +1,177 @@
+"""GPU parity of the k-way reduce-copy (through the C ABI) against the CPU
+oracle on identical seeded inputs."""
+import itertools
+
+import numpy as np
+import pytest
+
+from flagcx_amd import _native as N
+from flagcx_amd import kernels as K
+from oracle import fx_oracle as O
+from tests.util import DTYPES, OPS, DevBufs, assert_parity, seeded_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def run_reduce(dev, ins, dtype, op, first=0, inplace=False, offs=None):
+    """Upload ins (optionally at per-buffer byte offsets), reduce on the GPU,
+    return the host result."""
+    n = ins[0].size
+    es = N.DTYPE_SIZE[dtype]
+    offs = offs or [0] * (len(ins) + 1)
+    with DevBufs(dev) as b:
+        dins = [b.put(a, pad_before=o) for a, o in zip(ins, offs[1:])]
+        dout = dins[0] if inplace else b.alloc(n * es + 256) + offs[0]
+        if not inplace:
+            dev.memset(dout - offs[0], 0xA5, n * es + 256)
+        N.check(K.reduce_copy(dout, dins, n, dtype, op, first), "fx_reduce_copy")
+        dev.sync()
+        got = dev.to_host(dout, n, N.NP_DTYPE[dtype])
+        if not inplace:  # nothing written past the end
+            tail = dev.to_host(dout + n * es, 64, np.uint8)
+            assert (tail == 0xA5).all(), "wrote past the end of the output"
+    return got
+
+
+def test_reference_known_answers(dev):
+    # test/unittest/service/test_reduction_ops.cpp:11-75
+    f = np.float32
+    cases = [
+        (N.DT_FP32, N.OP_SUM, [1, 2, 3], [4, 5, 6], [5, 7, 9], f),
+        (N.DT_INT32, N.OP_SUM, [10, 20, 30], [1, 2, 3], [11, 22, 33], np.int32),
+        (N.DT_FP32, N.OP_MIN, [3, 1, 4], [1, 5, 2], [1, 1, 2], f),
+        (N.DT_FP32, N.OP_MAX, [3, 1, 4], [1, 5, 2], [3, 5, 4], f),
+        (N.DT_FP32, N.OP_SUM, [42], [8], [50], f),
+    ]
+    for dtype, op, a, b, want, t in cases:
+        got = run_reduce(dev, [np.array(a, t), np.array(b, t)], dtype, op)
+        assert got.tolist() == want
+
+
+@pytest.mark.parametrize("dname", list(DTYPES))
+@pytest.mark.parametrize("oname", list(OPS))
+def test_seeded_parity_k_and_sizes(dev, dname, oname):
+    dtype, op = DTYPES[dname], OPS[oname]
+    sizes = [1, 3, 8, 63, 1000, 4097, 65536 + 3, (1 << 20) + 5]
+    for k, n in itertools.product([1, 2, 3, 4, 5, 6, 7, 8, 9, 17], sizes):
+        if k > 8 and n > 70000:
+            continue
+        ins = seeded_inputs(dtype, k, n, seed=100 + k)
+        want = O.reduce_copy(ins, dtype, op)
+        got = run_reduce(dev, ins, dtype, op)
+        assert_parity(got, want, dtype, op, f"{dname} {oname} k={k} n={n}")
+
+
+@pytest.mark.parametrize("dname", list(DTYPES))
+def test_inplace_matches_out_of_place(dev, dname):
+    dtype = DTYPES[dname]
+    for op, k, n in itertools.product(OPS.values(), [2, 4, 8], [5, 70001, (1 << 20) + 9]):
+        ins = seeded_inputs(dtype, k, n, seed=7)
+        want = O.reduce_copy(ins, dtype, op)
+        got = run_reduce(dev, ins, dtype, op, inplace=True)
+        assert_parity(got, want, dtype, op, f"in-place {dname} op={op} k={k} n={n}")
+
+
+@pytest.mark.parametrize("dname", list(DTYPES))
+def test_rotated_order(dev, dname):
+    dtype = DTYPES[dname]
+    k, n = 8, 50001
+    ins = seeded_inputs(dtype, k, n, seed=11)
+    for op in OPS.values():
+        for first in (0, 1, 5, 7):
+            want = O.reduce_copy(ins, dtype, op, first=first)
+            got = run_reduce(dev, ins, dtype, op, first=first)
+            assert_parity(got, want, dtype, op, f"{dname} op={op} first={first}")
+
+
+@pytest.mark.parametrize("dname", list(DTYPES))
+def test_unaligned_buffers(dev, dname):
+    """Output / inputs at element offsets that are not 16-byte aligned, both
+    all-equal (vector path with a peeled head) and mixed (gather path)."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    k = 3
+    for n in (1, 2, 9, 255, 5000, 300007):
+        ins = seeded_inputs(dtype, k, n, seed=n)
+        for offs_el in ([1, 1, 1, 1], [3, 3, 3, 3], [0, 1, 2, 3], [2, 0, 0, 0], [0, 0, 1, 0]):
+            offs = [o * es for o in offs_el]
+            for op in (N.OP_SUM, N.OP_MAX):
+                want = O.reduce_copy(ins, dtype, op)
+                got = run_reduce(dev, ins, dtype, op, offs=offs)
+                assert_parity(got, want, dtype, op, f"{dname} n={n} offs={offs_el} op={op}")
+
+
+def _special_f32():
+    v = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.17549435e-38, 3.4028235e38,
+                  -3.4028235e38, 1e8, 1.0, -1e8, 16777216.0, 1.0, 0.5, 1.5, 2.5], np.float32)
+    return v
+
+
+def test_special_values_fp32(dev):
+    v = _special_f32()
+    grid = np.array(list(itertools.product(v, v, v)), np.float32)  # all triples
+    ins = [np.ascontiguousarray(grid[:, j]) for j in range(3)]
+    for op in OPS.values():
+        want = O.reduce_copy(ins, N.DT_FP32, op)
+        got = run_reduce(dev, ins, N.DT_FP32, op)
+        if op in (N.OP_SUM, N.OP_PROD):  # NaN payloads of arithmetic are not part of the contract
+            gn, wn = np.isnan(got), np.isnan(want)
+            assert np.array_equal(gn, wn)
+            assert np.array_equal(got[~gn].view(np.uint32), want[~wn].view(np.uint32))
+        else:
+            assert_parity(got, want, N.DT_FP32, op, f"special fp32 op={op}")
+
+
+@pytest.mark.parametrize("dname", ["bf16", "fp16"])
+def test_all_16bit_patterns(dev, dname):
+    """Every 16-bit pattern (incl. NaNs, infinities, subnormals, +-0) against
+    shuffled copies of itself."""
+    dtype = DTYPES[dname]
+    allbits = np.arange(65536, dtype=np.uint16)
+    rng = np.random.default_rng(5)
+    ins = [allbits] + [rng.permutation(allbits) for _ in range(3)]
+    for op in OPS.values():
+        want = O.reduce_copy(ins, dtype, op)
+        got = run_reduce(dev, ins, dtype, op)
+        assert_parity(got, want, dtype, op, f"all {dname} patterns op={op}")
+    # pairs around rounding ties: x + tiny
+    for op in (N.OP_SUM, N.OP_PROD):
+        a = np.repeat(allbits[::7], 8)
+        b = np.tile(np.array([0x0001, 0x8001, 0x3c00, 0x3f80, 0x0400, 0x0080, 0x7bff, 0x7f7f], np.uint16),
+                    a.size // 8)
+        want = O.reduce_copy([a, b], dtype, op)
+        got = run_reduce(dev, [a, b], dtype, op)
+        assert_parity(got, want, dtype, op, f"{dname} ties op={op}")
+
+
+def test_int32_wraparound(dev):
+    a = np.array([2**31 - 1, -2**31, 123456789, -1, 65536, 46341], np.int32)
+    b = np.array([1, -1, 987654321, -2**31, 65536, 46341], np.int32)
+    c = np.array([2**31 - 1, -2**31, 2, 2, 3, 2], np.int32)
+    for op in OPS.values():
+        want = O.reduce_copy([a, b, c], N.DT_INT32, op)
+        got = run_reduce(dev, [a, b, c], N.DT_INT32, op)
+        assert_parity(got, want, N.DT_INT32, op, f"int32 wrap op={op}")
+    s = run_reduce(dev, [a, b, c], N.DT_INT32, N.OP_SUM).astype(np.int64)
+    assert np.array_equal(s, ((a.astype(np.int64) + b + c + 2**31) % 2**32) - 2**31)
+
+
+def test_error_paths(dev):
+    p = dev.malloc(64)
+    try:
+        ok = lambda dtype, op, k=2, first=0, out=p, ins=None, n=4: K.reduce_copy(out, ins or [p] * k, n, dtype, op, first)
+        assert ok(N.DT_FP32, N.OP_SUM) == N.SUCCESS
+        assert ok(N.DT_FP64, N.OP_SUM) == N.NOT_SUPPORTED      # known to FlagCX, not on this path
+        assert ok(N.DT_INT8, N.OP_SUM) == N.NOT_SUPPORTED
+        assert ok(N.DT_FP32, N.OP_AVG) == N.NOT_SUPPORTED
+        assert ok(10, N.OP_SUM) == N.INVALID_ARGUMENT           # outside the enums
+        assert ok(N.DT_FP32, 5) == N.INVALID_ARGUMENT
+        assert ok(N.DT_FP32, N.OP_SUM, first=2) == N.INVALID_ARGUMENT
+        assert ok(N.DT_FP32, N.OP_SUM, out=None) == N.INVALID_ARGUMENT
+        assert ok(N.DT_FP32, N.OP_SUM, out=p + 2) == N.INVALID_ARGUMENT   # not element aligned
+        assert ok(N.DT_FP32, N.OP_SUM, ins=[p, None]) == N.INVALID_ARGUMENT
+        assert K.reduce_copy(p, [p] * 65, 4, N.DT_FP32, N.OP_SUM) == N.INVALID_ARGUMENT
+        assert K.reduce_copy(None, [None], 0, N.DT_FP32, N.OP_SUM) == N.SUCCESS  # empty input
+        dev.sync()
+    finally:
+        dev.free(p)

@@ -74,6 +74,31 @@ _SIGS = {
     "fx_version": (C.c_char_p, []),
     "fx_synth_fill": (_i, [_vp, _sz, _i, _i, C.c_double, C.c_double, C.c_uint64, C.c_uint64, _i]),
 }
+class RedNode(C.Structure):
+    _fields_ = [("step", C.c_int32), ("rank", C.c_int32), ("in1_buf", C.c_int32), ("in2_buf", C.c_int32),
+                ("out_buf", C.c_int32), ("slice", C.c_int32), ("in1_off", C.c_uint64), ("in2_off", C.c_uint64),
+                ("out_off", C.c_uint64), ("count", C.c_uint64)]
+
+
+_szp = C.POINTER(_sz)
+_SIGS.update({
+    # include/flagcx_amd/fx_sim.h
+    "fxSimCommInitAll": (_i, [C.POINTER(_vp), _i]),
+    "fxSimCommDestroyAll": (_i, [C.POINTER(_vp), _i]),
+    "fxSimCommConfig": (_i, [_vp, _i, C.c_longlong]),
+    "fxSimRegisterWindows": (_i, [_vp, C.POINTER(_vp), _sz]),
+    "flagcxCommCount": (_i, [_vp, C.POINTER(_i)]),
+    "flagcxCommUserRank": (_i, [_vp, C.POINTER(_i)]),
+    "flagcxReduce": (_i, [_vp, _vp, _sz, _i, _i, _i, _vp, _vp]),
+    "flagcxAllReduce": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
+    "flagcxReduceScatter": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
+    "flagcxAllGather": (_i, [_vp, _vp, _sz, _i, _vp, _vp]),
+    "flagcxAlltoAllv": (_i, [_vp, _szp, _szp, _vp, _szp, _szp, _i, _vp, _vp]),
+    "flagcxCustomAllReduceImpl": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
+    "fx_part_ring_ar": (_sz, [_sz, _i, _i, _sz, _sz, C.POINTER(RedNode)]),
+    "fx_part_ring_rs": (_sz, [_sz, _i, _i, _sz, _sz, C.POINTER(RedNode)]),
+    "fx_part_locred": (_sz, [_sz, _i, _i, _sz, C.POINTER(RedNode)]),
+})
 for _name, (_res, _args) in _SIGS.items():
     _f = getattr(lib, _name)
     _f.restype, _f.argtypes = _res, _args

@@ -261,7 +261,10 @@ flagcxResult_t fxGetDeviceProperties(struct flagcxDevProps *props, int d) {
     (void)hipGetLastError();
     return flagcxUnhandledDeviceError;
   }
-  strncpy(props->name, p.name, sizeof(props->name) - 1);
+  // Some driver stacks report no marketing name; callers expect a non-empty
+  // one, so fall back to the ISA name (e.g. "gfx950:sramecc+:xnack-").
+  const char *nm = p.name[0] ? p.name : p.gcnArchName;
+  strncpy(props->name, nm[0] ? nm : "AMD GPU", sizeof(props->name) - 1);
   props->name[sizeof(props->name) - 1] = '\0';
   props->pciBusId = p.pciBusID;
   props->pciDeviceId = p.pciDeviceID;

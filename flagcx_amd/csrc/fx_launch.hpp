@@ -8,7 +8,7 @@ namespace fx {
 
 // Vectors per lane per input: keep roughly 8..16 independent 16-byte loads in
 // flight per lane whatever the input count.
-constexpr int unrollFor(int K) { return K == 0 ? 2 : (K == 1 ? 8 : (K <= 4 ? 4 : 2)); }
+constexpr int unrollFor(int K) { return K == 0 ? 2 : (K == 1 ? 8 : 4); }
 
 struct KernelSet {
   // index = compile-time input count, 0 = runtime-k kernel

@@ -1,0 +1,681 @@
+// FlagCX collective entry points over simulated ranks on one GPU, plus the
+// chunk / slice / red-slice partition they are built from.
+//
+// Reference behaviour followed:
+//   partition ............ flagcx/runner/uni_runner_impl.cc:82-157 (LocRed),
+//                          :661-1007 (sliced ring allreduce), :1009-1264 (ring
+//                          reduce-scatter)
+//   nranks == 1 .......... copy if out of place, else nothing (:669-691)
+//   alltoallv addressing . flagcx/service/bootstrap.cc:1253-1279
+//   custom allreduce ..... flagcx/adaptor/kernel/nvidia/custom_allreduce.cu:604-677
+// The transport between ranks is elided: a rank reads its peer's buffer where
+// the reference would receive a copy of it.
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "flagcx_amd/fx_kernels.h"
+#include "flagcx_amd/fx_sim.h"
+
+struct flagcxStream {
+  hipStream_t base;
+};
+
+namespace {
+
+enum Kind { kNone = 0, kReduce, kAllReduce, kReduceScatter, kAllGather, kAlltoAllv, kCustomAllReduce };
+
+struct Post {
+  bool posted = false;
+  const void *send = nullptr;
+  void *recv = nullptr;
+  hipStream_t stream = nullptr;
+  std::vector<size_t> sendcounts, sdispls, recvcounts, rdispls;
+};
+
+struct Group {
+  int n = 0;
+  int device = 0;
+  std::mutex mu;
+  // pending collective
+  Kind kind = kNone;
+  size_t count = 0;
+  int dtype = 0, op = 0, root = 0, nposted = 0;
+  std::vector<Post> posts;
+  std::vector<hipEvent_t> ready;
+  hipEvent_t done = nullptr;
+  // configuration
+  long long algo = FX_ALGO_DIRECT, order = FX_ORDER_RANK;
+  long long nslices = 1, nredslices = 0, redslicesize = 65536;
+  // scratch: ring reduce-scatter partials / alltoallv staging
+  void *scratch = nullptr;
+  size_t scratchBytes = 0;
+  std::vector<void *> windows;
+  size_t windowBytes = 0;
+};
+
+long long envParam(const char *name, long long dflt) {
+  const char *e = getenv(name);
+  if (!e || !*e) return dflt;
+  char *end = nullptr;
+  long long v = strtoll(e, &end, 0);
+  return (end && *end == '\0') ? v : dflt;
+}
+
+inline flagcxResult_t R(int rc) { return (flagcxResult_t)rc; }
+inline int mod(int a, int n) { return ((a % n) + n) % n; }
+inline const char *cadd(const void *p, size_t bytes) { return (const char *)p + bytes; }
+inline char *madd(void *p, size_t bytes) { return (char *)p + bytes; }
+
+flagcxResult_t ensureScratch(Group *g, size_t bytes) {
+  if (bytes <= g->scratchBytes) return flagcxSuccess;
+  if (g->scratch) (void)hipFree(g->scratch);  // waits for the device: earlier launches are done
+  g->scratch = nullptr;
+  g->scratchBytes = 0;
+  if (hipMalloc(&g->scratch, bytes) != hipSuccess) return flagcxUnhandledDeviceError;
+  g->scratchBytes = bytes;
+  return flagcxSuccess;
+}
+
+fxSliceDesc copyDesc(const void *src, void *dst, size_t bytes) {
+  fxSliceDesc d;
+  memset(&d, 0, sizeof(d));
+  d.in[0] = src;
+  d.out = dst;
+  d.count = bytes;
+  return d;
+}
+
+struct Ctx {
+  Group *g;
+  hipStream_t s;
+  int n;
+  size_t ts;
+  const void *send(int r) const { return g->posts[r].send; }
+  void *recv(int r) const { return g->posts[r].recv; }
+};
+
+// k-way reduce of element range [off, off+cnt) of every rank's sendbuff (+sendBase
+// elements) into out, in order first, first+1, ...
+flagcxResult_t kway(const Ctx &c, std::vector<fxSliceDesc> &descs, size_t sendOff, size_t cnt, void *out, int first) {
+  if (cnt == 0) return flagcxSuccess;
+  if (c.n <= FX_MAX_SLICE_INPUTS) {
+    fxSliceDesc d;
+    memset(&d, 0, sizeof(d));
+    for (int j = 0; j < c.n; j++) d.in[j] = cadd(c.send(mod(first + j, c.n)), sendOff * c.ts);
+    d.out = out;
+    d.count = cnt;
+    descs.push_back(d);
+    return flagcxSuccess;
+  }
+  std::vector<const void *> in(c.n);
+  for (int j = 0; j < c.n; j++) in[j] = cadd(c.send(j), sendOff * c.ts);
+  return R(fx_reduce_copy(out, in.data(), c.n, cnt, c.g->dtype, c.g->op, first, c.s));
+}
+
+flagcxResult_t flushKway(const Ctx &c, std::vector<fxSliceDesc> &descs) {
+  if (descs.empty()) return flagcxSuccess;
+  flagcxResult_t rc = R(fx_reduce_slices(descs.data(), descs.size(), c.n, c.g->dtype, c.g->op, c.s));
+  descs.clear();
+  return rc;
+}
+
+// Visit the (slice, red-slice) pieces of a chunk of ccnt elements at element
+// offset coff, exactly as the reference nests its three splits.
+template <class F>
+flagcxResult_t forPieces(const Group *g, size_t ccnt, size_t coff, size_t nred, F f) {
+  for (size_t s = 0; s < (size_t)g->nslices; s++) {
+    size_t scnt, soff;
+    fx_split(ccnt, (size_t)g->nslices, s, &scnt, &soff);
+    for (size_t q = 0; q < nred; q++) {
+      size_t rcnt, roff;
+      fx_split(scnt, nred, q, &rcnt, &roff);
+      flagcxResult_t rc = f(coff + soff + roff, soff + roff, rcnt);
+      if (rc != flagcxSuccess) return rc;
+    }
+  }
+  return flagcxSuccess;
+}
+
+flagcxResult_t runAllReduce(const Ctx &c) {
+  Group *g = c.g;
+  const int n = c.n;
+  const size_t count = g->count, ts = c.ts;
+  if (n == 1) {
+    if (count && c.send(0) != c.recv(0)) {
+      fxSliceDesc d = copyDesc(c.send(0), c.recv(0), count * ts);
+      return R(fx_copy_slices(&d, 1, c.s));
+    }
+    return flagcxSuccess;
+  }
+  const size_t nred = fx_nredslices(count, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
+  std::vector<fxSliceDesc> descs;
+  if (g->algo == FX_ALGO_RING) {
+    // reduce-scatter: step i, rank r reduces chunk (r-i-1)%n: partial from the
+    // previous rank (its sendbuff at step 0, its recvbuff afterwards) + own data.
+    for (int i = 0; i < n - 1; i++) {
+      for (int r = 0; r < n; r++) {
+        const int prev = mod(r - 1, n), rx = mod(r - i - 1, n);
+        size_t ccnt, coff;
+        fx_split(count, n, rx, &ccnt, &coff);
+        const void *partial = (i == 0) ? c.send(prev) : (const void *)c.recv(prev);
+        flagcxResult_t rc = forPieces(g, ccnt, coff, nred, [&](size_t off, size_t, size_t cnt) {
+          if (cnt == 0) return flagcxSuccess;
+          fxSliceDesc d;
+          memset(&d, 0, sizeof(d));
+          d.in[0] = cadd(partial, off * ts);
+          d.in[1] = cadd(c.send(r), off * ts);
+          d.out = madd(c.recv(r), off * ts);
+          d.count = cnt;
+          descs.push_back(d);
+          return flagcxSuccess;
+        });
+        if (rc != flagcxSuccess) return rc;
+      }
+      flagcxResult_t rc = R(fx_reduce_slices(descs.data(), descs.size(), 2, g->dtype, g->op, c.s));
+      descs.clear();
+      if (rc != flagcxSuccess) return rc;
+    }
+    // all-gather: step i, rank r receives chunk (r-i)%n from the previous rank.
+    for (int i = 0; i < n - 1; i++) {
+      for (int r = 0; r < n; r++) {
+        const int prev = mod(r - 1, n), rx = mod(r - i, n);
+        size_t ccnt, coff;
+        fx_split(count, n, rx, &ccnt, &coff);
+        if (ccnt) descs.push_back(copyDesc(cadd(c.recv(prev), coff * ts), madd(c.recv(r), coff * ts), ccnt * ts));
+      }
+      flagcxResult_t rc = R(fx_copy_slices(descs.data(), descs.size(), c.s));
+      descs.clear();
+      if (rc != flagcxSuccess) return rc;
+    }
+    return flagcxSuccess;
+  }
+  // direct: chunk ch is reduced k-way into the rank the ring would leave it
+  // on, (ch-1)%n, then copied to everyone else.
+  for (int ch = 0; ch < n; ch++) {
+    size_t ccnt, coff;
+    fx_split(count, n, ch, &ccnt, &coff);
+    const int owner = mod(ch - 1, n);
+    const int first = (g->order == FX_ORDER_RING) ? ch : 0;
+    flagcxResult_t rc = forPieces(g, ccnt, coff, nred, [&](size_t off, size_t, size_t cnt) {
+      return kway(c, descs, off, cnt, madd(c.recv(owner), off * ts), first);
+    });
+    if (rc != flagcxSuccess) return rc;
+  }
+  flagcxResult_t rc = flushKway(c, descs);
+  if (rc != flagcxSuccess) return rc;
+  for (int ch = 0; ch < n; ch++) {
+    size_t ccnt, coff;
+    fx_split(count, n, ch, &ccnt, &coff);
+    const int owner = mod(ch - 1, n);
+    for (int r = 0; r < n; r++)
+      if (r != owner && ccnt)
+        descs.push_back(copyDesc(cadd(c.recv(owner), coff * ts), madd(c.recv(r), coff * ts), ccnt * ts));
+  }
+  return R(fx_copy_slices(descs.data(), descs.size(), c.s));
+}
+
+flagcxResult_t runReduce(const Ctx &c) {
+  Group *g = c.g;
+  if (g->count == 0) return flagcxSuccess;
+  std::vector<const void *> in(c.n);
+  for (int j = 0; j < c.n; j++) in[j] = c.send(j);
+  return R(fx_reduce_copy(c.recv(g->root), in.data(), c.n, g->count, g->dtype, g->op, 0, c.s));
+}
+
+flagcxResult_t runReduceScatter(const Ctx &c) {
+  Group *g = c.g;
+  const int n = c.n;
+  const size_t rcount = g->count, ts = c.ts;
+  if (n == 1) {
+    if (rcount && c.send(0) != c.recv(0)) {
+      fxSliceDesc d = copyDesc(c.send(0), c.recv(0), rcount * ts);
+      return R(fx_copy_slices(&d, 1, c.s));
+    }
+    return flagcxSuccess;
+  }
+  const size_t nred = fx_nredslices(rcount, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
+  std::vector<fxSliceDesc> descs;
+  if (g->algo == FX_ALGO_RING) {
+    // Per-rank scratch of n*recvcount elements holds the travelling partials.
+    flagcxResult_t rc = ensureScratch(g, (size_t)n * n * rcount * ts);
+    if (rc != flagcxSuccess) return rc;
+    auto scratch = [&](int r) { return madd(g->scratch, (size_t)r * n * rcount * ts); };
+    for (int i = 0; i < n - 1; i++) {
+      for (int r = 0; r < n; r++) {
+        const int prev = mod(r - 1, n), rx = mod(r - i - 2, n);
+        const void *partial = (i == 0) ? c.send(prev) : (const void *)scratch(prev);
+        rc = forPieces(g, rcount, (size_t)rx * rcount, nred, [&](size_t off, size_t inSlice, size_t cnt) {
+          if (cnt == 0) return flagcxSuccess;
+          fxSliceDesc d;
+          memset(&d, 0, sizeof(d));
+          d.in[0] = cadd(partial, off * ts);
+          d.in[1] = cadd(c.send(r), off * ts);
+          d.out = (i == n - 2) ? madd(c.recv(r), inSlice * ts) : madd(scratch(r), off * ts);
+          d.count = cnt;
+          descs.push_back(d);
+          return flagcxSuccess;
+        });
+        if (rc != flagcxSuccess) return rc;
+      }
+      rc = R(fx_reduce_slices(descs.data(), descs.size(), 2, g->dtype, g->op, c.s));
+      descs.clear();
+      if (rc != flagcxSuccess) return rc;
+    }
+    return flagcxSuccess;
+  }
+  for (int r = 0; r < n; r++) {
+    const int first = (g->order == FX_ORDER_RING) ? mod(r + 1, n) : 0;
+    flagcxResult_t rc = forPieces(g, rcount, (size_t)r * rcount, nred, [&](size_t off, size_t inSlice, size_t cnt) {
+      return kway(c, descs, off, cnt, madd(c.recv(r), inSlice * ts), first);
+    });
+    if (rc != flagcxSuccess) return rc;
+  }
+  return flushKway(c, descs);
+}
+
+flagcxResult_t runAllGather(const Ctx &c) {
+  const size_t bytes = c.g->count * c.ts;
+  if (bytes == 0) return flagcxSuccess;
+  std::vector<fxSliceDesc> descs;
+  for (int r = 0; r < c.n; r++)
+    for (int j = 0; j < c.n; j++) {
+      void *dst = madd(c.recv(j), (size_t)r * bytes);
+      if (dst != c.send(r)) descs.push_back(copyDesc(c.send(r), dst, bytes));
+    }
+  return R(fx_copy_slices(descs.data(), descs.size(), c.s));
+}
+
+// pack every rank's segments into its contiguous staging slots, then unpack
+// from the peers' slots: two batched launches, safe for send == recv.
+flagcxResult_t runAlltoAllv(const Ctx &c) {
+  Group *g = c.g;
+  const int n = c.n;
+  const size_t ts = c.ts;
+  std::vector<size_t> base(n + 1, 0);
+  for (int r = 0; r < n; r++) {
+    size_t tot = 0;
+    for (int i = 0; i < n; i++) {
+      if (g->posts[r].sendcounts[i] != g->posts[i].recvcounts[r]) return flagcxInvalidArgument;
+      tot += g->posts[r].sendcounts[i];
+    }
+    base[r + 1] = base[r] + ((tot * ts + 255) & ~(size_t)255);
+  }
+  if (base[n] == 0) return flagcxSuccess;
+  flagcxResult_t rc = ensureScratch(g, base[n]);
+  if (rc != flagcxSuccess) return rc;
+  std::vector<fxSliceDesc> pack, unpack;
+  for (int r = 0; r < n; r++) {
+    size_t slot = 0;
+    for (int i = 0; i < n; i++) {
+      const size_t cnt = g->posts[r].sendcounts[i];
+      if (cnt) {
+        void *stage = madd(g->scratch, base[r] + slot * ts);
+        pack.push_back(copyDesc(cadd(c.send(r), g->posts[r].sdispls[i] * ts), stage, cnt * ts));
+        unpack.push_back(copyDesc(stage, madd(c.recv(i), g->posts[i].rdispls[r] * ts), cnt * ts));
+      }
+      slot += cnt;
+    }
+  }
+  rc = R(fx_copy_slices(pack.data(), pack.size(), c.s));
+  if (rc != flagcxSuccess) return rc;
+  return R(fx_copy_slices(unpack.data(), unpack.size(), c.s));
+}
+
+flagcxResult_t runCustomAllReduce(const Ctx &c) {
+  Group *g = c.g;
+  if (g->count == 0) return flagcxSuccess;
+  std::vector<fxSliceDesc> descs;
+  for (int r = 0; r < c.n; r++) {
+    if (c.n <= FX_MAX_SLICE_INPUTS) {
+      fxSliceDesc d;
+      memset(&d, 0, sizeof(d));
+      for (int j = 0; j < c.n; j++) d.in[j] = g->windows[j];
+      d.out = c.recv(r);
+      d.count = g->count;
+      descs.push_back(d);
+    } else {
+      flagcxResult_t rc = R(fx_reduce_copy(c.recv(r), (const void *const *)g->windows.data(), c.n, g->count,
+                                           g->dtype, g->op, 0, c.s));
+      if (rc != flagcxSuccess) return rc;
+    }
+  }
+  return flushKway(c, descs);
+}
+
+void resetPending(Group *g) {
+  g->kind = kNone;
+  g->nposted = 0;
+  for (auto &p : g->posts) p = Post();
+}
+
+// Record one rank's call; the last rank to arrive launches the collective.
+flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, void *recv, size_t count, int dtype,
+                               int op, int root, flagcxStream_t stream, const size_t *sc = nullptr,
+                               const size_t *sd = nullptr, const size_t *rc_ = nullptr, const size_t *rd = nullptr);
+
+}  // namespace
+
+struct flagcxComm {
+  Group *g;
+  int rank;
+};
+
+namespace {
+
+flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, void *recv, size_t count, int dtype,
+                               int op, int root, flagcxStream_t stream, const size_t *sc, const size_t *sd,
+                               const size_t *rc_, const size_t *rd) {
+  if (!comm || !comm->g || !stream) return flagcxInvalidArgument;
+  Group *g = comm->g;
+  const int rank = comm->rank;
+  std::lock_guard<std::mutex> lock(g->mu);
+  if (g->nposted == 0) {
+    g->kind = kind;
+    g->count = count;
+    g->dtype = dtype;
+    g->op = op;
+    g->root = root;
+  } else if (g->kind != kind || g->count != count || g->dtype != dtype || g->op != op || g->root != root) {
+    resetPending(g);
+    return flagcxInvalidArgument;  // ranks disagree on the collective
+  }
+  Post &p = g->posts[rank];
+  if (p.posted) {
+    resetPending(g);
+    return flagcxInvalidUsage;  // same rank called twice before the others arrived
+  }
+  p.posted = true;
+  p.send = send;
+  p.recv = recv;
+  p.stream = stream->base;
+  if (kind == kAlltoAllv) {
+    p.sendcounts.assign(sc, sc + g->n);
+    p.sdispls.assign(sd, sd + g->n);
+    p.recvcounts.assign(rc_, rc_ + g->n);
+    p.rdispls.assign(rd, rd + g->n);
+  }
+  if (hipEventRecord(g->ready[rank], p.stream) != hipSuccess) {
+    resetPending(g);
+    return flagcxUnhandledDeviceError;
+  }
+  if (++g->nposted < g->n) return flagcxSuccess;
+
+  Ctx c{g, p.stream, g->n, fx_dtype_size(dtype)};
+  flagcxResult_t res = flagcxSuccess;
+  for (int r = 0; r < g->n && res == flagcxSuccess; r++)
+    if (g->posts[r].stream != c.s && hipStreamWaitEvent(c.s, g->ready[r], 0) != hipSuccess)
+      res = flagcxUnhandledDeviceError;
+  if (res == flagcxSuccess) {
+    switch (kind) {
+      case kAllReduce: res = runAllReduce(c); break;
+      case kReduce: res = runReduce(c); break;
+      case kReduceScatter: res = runReduceScatter(c); break;
+      case kAllGather: res = runAllGather(c); break;
+      case kAlltoAllv: res = runAlltoAllv(c); break;
+      case kCustomAllReduce: res = runCustomAllReduce(c); break;
+      default: res = flagcxInternalError;
+    }
+  }
+  if (res == flagcxSuccess) {
+    bool others = false;
+    for (int r = 0; r < g->n; r++) others = others || (g->posts[r].stream != c.s);
+    if (others) {
+      if (hipEventRecord(g->done, c.s) != hipSuccess) res = flagcxUnhandledDeviceError;
+      for (int r = 0; r < g->n && res == flagcxSuccess; r++)
+        if (g->posts[r].stream != c.s && hipStreamWaitEvent(g->posts[r].stream, g->done, 0) != hipSuccess)
+          res = flagcxUnhandledDeviceError;
+    }
+  }
+  resetPending(g);
+  return res;
+}
+
+// Argument screening shared by the reducing collectives: same verdicts as the
+// kernel layer (unsupported-but-known -> flagcxNotSupported).
+flagcxResult_t screenReduce(int dtype, int op) {
+  if (dtype < 0 || dtype >= flagcxNumTypes || op < 0 || op >= flagcxNumRedOps) return flagcxInvalidArgument;
+  if (dtype != flagcxInt32 && dtype != flagcxFloat32 && dtype != flagcxFloat16 && dtype != flagcxBfloat16)
+    return flagcxNotSupported;
+  if (op > flagcxMin) return flagcxNotSupported;
+  return flagcxSuccess;
+}
+
+void partNode(fxRedNode *n, int step, int rank, size_t slice, int in1, int in2, int out, size_t inOff, size_t outOff,
+              size_t cnt) {
+  n->step = step;
+  n->rank = rank;
+  n->slice = (int32_t)slice;
+  n->in1_buf = in1;
+  n->in2_buf = in2;
+  n->out_buf = out;
+  n->in1_off = n->in2_off = inOff;
+  n->out_off = outOff;
+  n->count = cnt;
+}
+
+}  // namespace
+
+extern "C" {
+#pragma GCC visibility push(default)
+
+flagcxResult_t fxSimCommInitAll(flagcxComm_t *comms, int nranks) {
+  if (!comms || nranks < 1 || nranks > FX_MAX_INPUTS) return flagcxInvalidArgument;
+  Group *g = new (std::nothrow) Group();
+  if (!g) return flagcxSystemError;
+  g->n = nranks;
+  g->posts.resize(nranks);
+  g->ready.assign(nranks, nullptr);
+  if (hipGetDevice(&g->device) != hipSuccess) {
+    delete g;
+    return flagcxUnhandledDeviceError;
+  }
+  bool ok = hipEventCreateWithFlags(&g->done, hipEventDisableTiming) == hipSuccess;
+  for (int r = 0; r < nranks && ok; r++)
+    ok = hipEventCreateWithFlags(&g->ready[r], hipEventDisableTiming) == hipSuccess;
+  if (!ok) {
+    for (auto e : g->ready)
+      if (e) (void)hipEventDestroy(e);
+    if (g->done) (void)hipEventDestroy(g->done);
+    delete g;
+    return flagcxUnhandledDeviceError;
+  }
+  g->nslices = envParam("FLAGCX_UNIRUNNER_NSLICES", 1);
+  g->nredslices = envParam("FLAGCX_UNIRUNNER_NREDSLICES", 0);
+  g->redslicesize = envParam("FLAGCX_UNIRUNNER_REDSLICESIZE", 65536);
+  if (g->nslices < 1) g->nslices = 1;
+  if (g->nredslices < 0) g->nredslices = 0;
+  if (g->redslicesize < 0) g->redslicesize = 0;
+  for (int r = 0; r < nranks; r++) {
+    comms[r] = new (std::nothrow) flagcxComm{g, r};
+    if (!comms[r]) return flagcxSystemError;
+  }
+  return flagcxSuccess;
+}
+
+flagcxResult_t fxSimCommDestroyAll(flagcxComm_t *comms, int nranks) {
+  if (!comms || nranks < 1 || !comms[0]) return flagcxInvalidArgument;
+  Group *g = comms[0]->g;
+  if (g->n != nranks) return flagcxInvalidArgument;
+  (void)hipDeviceSynchronize();
+  for (auto e : g->ready) (void)hipEventDestroy(e);
+  (void)hipEventDestroy(g->done);
+  if (g->scratch) (void)hipFree(g->scratch);
+  delete g;
+  for (int r = 0; r < nranks; r++) {
+    delete comms[r];
+    comms[r] = nullptr;
+  }
+  return flagcxSuccess;
+}
+
+flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
+  if (!comm || !comm->g) return flagcxInvalidArgument;
+  Group *g = comm->g;
+  std::lock_guard<std::mutex> lock(g->mu);
+  switch (key) {
+    case FX_SIM_ALGO:
+      if (value != FX_ALGO_DIRECT && value != FX_ALGO_RING) return flagcxInvalidArgument;
+      g->algo = value;
+      break;
+    case FX_SIM_ORDER:
+      if (value != FX_ORDER_RANK && value != FX_ORDER_RING) return flagcxInvalidArgument;
+      g->order = value;
+      break;
+    case FX_SIM_NSLICES:
+      if (value < 1) return flagcxInvalidArgument;
+      g->nslices = value;
+      break;
+    case FX_SIM_NREDSLICES:
+      if (value < 0) return flagcxInvalidArgument;
+      g->nredslices = value;
+      break;
+    case FX_SIM_REDSLICESIZE:
+      if (value < 0) return flagcxInvalidArgument;
+      g->redslicesize = value;
+      break;
+    default: return flagcxInvalidArgument;
+  }
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxCommCount(const flagcxComm_t comm, int *count) {
+  if (!comm || !count) return flagcxInvalidArgument;
+  *count = comm->g->n;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxCommUserRank(const flagcxComm_t comm, int *rank) {
+  if (!comm || !rank) return flagcxInvalidArgument;
+  *rank = comm->rank;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxAllReduce(const void *sendbuff, void *recvbuff, size_t count, flagcxDataType_t datatype,
+                               flagcxRedOp_t op, flagcxComm_t comm, flagcxStream_t stream) {
+  flagcxResult_t rc = screenReduce(datatype, op);
+  if (rc != flagcxSuccess) return rc;
+  if (count && (!sendbuff || !recvbuff)) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kAllReduce, sendbuff, recvbuff, count, datatype, op, 0, stream);
+}
+
+flagcxResult_t flagcxReduce(const void *sendbuff, void *recvbuff, size_t count, flagcxDataType_t datatype,
+                            flagcxRedOp_t op, int root, flagcxComm_t comm, flagcxStream_t stream) {
+  flagcxResult_t rc = screenReduce(datatype, op);
+  if (rc != flagcxSuccess) return rc;
+  if (!comm || root < 0 || root >= comm->g->n) return flagcxInvalidArgument;
+  // recvbuff may be NULL except on the root (flagcx.h:365-366)
+  if (count && (!sendbuff || (comm->rank == root && !recvbuff))) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kReduce, sendbuff, recvbuff, count, datatype, op, root, stream);
+}
+
+flagcxResult_t flagcxReduceScatter(const void *sendbuff, void *recvbuff, size_t recvcount, flagcxDataType_t datatype,
+                                   flagcxRedOp_t op, flagcxComm_t comm, flagcxStream_t stream) {
+  flagcxResult_t rc = screenReduce(datatype, op);
+  if (rc != flagcxSuccess) return rc;
+  if (recvcount && (!sendbuff || !recvbuff)) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kReduceScatter, sendbuff, recvbuff, recvcount, datatype, op, 0, stream);
+}
+
+flagcxResult_t flagcxAllGather(const void *sendbuff, void *recvbuff, size_t sendcount, flagcxDataType_t datatype,
+                               flagcxComm_t comm, flagcxStream_t stream) {
+  if (fx_dtype_size(datatype) == 0) return flagcxInvalidArgument;
+  if (sendcount && (!sendbuff || !recvbuff)) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kAllGather, sendbuff, recvbuff, sendcount, datatype, 0, 0, stream);
+}
+
+flagcxResult_t flagcxAlltoAllv(const void *sendbuff, size_t *sendcounts, size_t *sdispls, void *recvbuff,
+                               size_t *recvcounts, size_t *rdispls, flagcxDataType_t datatype, flagcxComm_t comm,
+                               flagcxStream_t stream) {
+  if (fx_dtype_size(datatype) == 0) return flagcxInvalidArgument;
+  if (!sendcounts || !sdispls || !recvcounts || !rdispls) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kAlltoAllv, sendbuff, recvbuff, 0, datatype, 0, 0, stream, sendcounts, sdispls,
+                         recvcounts, rdispls);
+}
+
+flagcxResult_t fxSimRegisterWindows(flagcxComm_t comm, void *const *windows, size_t bytes) {
+  if (!comm || !comm->g) return flagcxInvalidArgument;
+  Group *g = comm->g;
+  std::lock_guard<std::mutex> lock(g->mu);
+  g->windows.clear();
+  g->windowBytes = 0;
+  if (!windows) return flagcxSuccess;
+  for (int r = 0; r < g->n; r++)
+    if (!windows[r]) return flagcxInvalidArgument;
+  g->windows.assign(windows, windows + g->n);
+  g->windowBytes = bytes;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxCustomAllReduceImpl(const void *sendbuff, void *recvbuff, size_t count,
+                                         flagcxDataType_t datatype, flagcxRedOp_t op, flagcxComm_t comm,
+                                         flagcxStream_t stream) {
+  if (!comm || !comm->g || !stream) return flagcxInvalidArgument;
+  flagcxResult_t rc = screenReduce(datatype, op);
+  if (rc != flagcxSuccess) return flagcxNotSupported;  // the hook only ever declines
+  Group *g = comm->g;
+  const size_t bytes = count * fx_dtype_size(datatype);
+  if (g->windows.empty() || bytes > g->windowBytes) return flagcxNotSupported;
+  if (count && (!sendbuff || !recvbuff)) return flagcxInvalidArgument;
+  void *win = g->windows[comm->rank];
+  if (bytes && sendbuff != win &&
+      hipMemcpyAsync(win, sendbuff, bytes, hipMemcpyDeviceToDevice, stream->base) != hipSuccess)
+    return flagcxUnhandledDeviceError;
+  return postAndMaybeRun(comm, kCustomAllReduce, win, recvbuff, count, datatype, op, 0, stream);
+}
+
+size_t fx_part_ring_ar(size_t count, int nranks, int rank, size_t nslices, size_t nred, fxRedNode *nodes) {
+  if (nranks < 2 || nslices == 0 || nred == 0) return 0;
+  size_t w = 0;
+  for (size_t s = 0; s < nslices; s++)
+    for (int i = 0; i < nranks - 1; i++) {
+      size_t ccnt, coff, scnt, soff;
+      fx_split(count, nranks, mod(rank - i - 1, nranks), &ccnt, &coff);
+      fx_split(ccnt, nslices, s, &scnt, &soff);
+      for (size_t q = 0; q < nred; q++, w++) {
+        size_t rcnt, roff;
+        fx_split(scnt, nred, q, &rcnt, &roff);
+        if (nodes) partNode(&nodes[w], i, rank, s, 1, 0, 1, coff + soff + roff, coff + soff + roff, rcnt);
+      }
+    }
+  return w;
+}
+
+size_t fx_part_ring_rs(size_t recvcount, int nranks, int rank, size_t nslices, size_t nred, fxRedNode *nodes) {
+  if (nranks < 2 || nslices == 0 || nred == 0) return 0;
+  size_t w = 0;
+  for (size_t s = 0; s < nslices; s++)
+    for (int i = 0; i < nranks - 1; i++) {
+      const size_t coff = (size_t)mod(rank - i - 2, nranks) * recvcount;
+      size_t scnt, soff;
+      fx_split(recvcount, nslices, s, &scnt, &soff);
+      for (size_t q = 0; q < nred; q++, w++) {
+        size_t rcnt, roff;
+        fx_split(scnt, nred, q, &rcnt, &roff);
+        if (!nodes) continue;
+        const bool last = (i == nranks - 2);
+        partNode(&nodes[w], i, rank, s, 2, 0, last ? 1 : 2, coff + soff + roff, last ? soff + roff : coff + soff + roff,
+                 rcnt);
+      }
+    }
+  return w;
+}
+
+size_t fx_part_locred(size_t count, int nranks, int rank, size_t nslices, fxRedNode *nodes) {
+  if (nranks < 2 || nslices == 0) return 0;
+  size_t ccnt, coff;
+  fx_split(count, nranks, rank, &ccnt, &coff);
+  for (size_t s = 0; s < nslices && nodes; s++) {
+    size_t scnt, soff;
+    fx_split(ccnt, nslices, s, &scnt, &soff);
+    partNode(&nodes[s], 0, rank, s, 1, 0, 1, coff + soff, coff + soff, scnt);
+  }
+  return nslices;
+}
+
+#pragma GCC visibility pop
+}  // extern "C"

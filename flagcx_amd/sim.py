@@ -1,0 +1,79 @@
+"""Simulated-rank communicator group (include/flagcx_amd/fx_sim.h) for tests
+and the benchmark.  Every rank posts the same collective; the last post runs it."""
+import ctypes as C
+
+from . import _native as N
+
+lib = N.lib
+
+ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE = 0, 1, 2, 3, 4
+ALGO_DIRECT, ALGO_RING = 0, 1
+ORDER_RANK, ORDER_RING = 0, 1
+
+
+def _szs(v):
+    return (C.c_size_t * max(len(v), 1))(*[int(x) for x in v])
+
+
+class SimGroup:
+    def __init__(self, nranks, **config):
+        self.n = nranks
+        self.comms = (C.c_void_p * nranks)()
+        N.check(lib.fxSimCommInitAll(self.comms, nranks), "fxSimCommInitAll")
+        self.configure(**config)
+
+    def configure(self, algo=None, order=None, nslices=None, nredslices=None, redslicesize=None):
+        for key, val in ((ALGO, algo), (ORDER, order), (NSLICES, nslices), (NREDSLICES, nredslices),
+                         (REDSLICESIZE, redslicesize)):
+            if val is not None:
+                N.check(lib.fxSimCommConfig(self.comms[0], key, val), f"fxSimCommConfig({key})")
+
+    def destroy(self):
+        if self.comms is not None:
+            lib.fxSimCommDestroyAll(self.comms, self.n)
+            self.comms = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.destroy()
+
+    # each method posts for every rank in turn and returns the LAST call's code
+    def _each(self, fn, streams):
+        rc = N.SUCCESS
+        for r in range(self.n):
+            s = streams[r] if isinstance(streams, (list, tuple)) else streams
+            rc = fn(r, s)
+            if rc != N.SUCCESS:
+                return rc
+        return rc
+
+    def all_reduce(self, sends, recvs, count, dtype, op, streams):
+        return self._each(lambda r, s: lib.flagcxAllReduce(sends[r], recvs[r], count, dtype, op, self.comms[r], s),
+                          streams)
+
+    def custom_all_reduce(self, sends, recvs, count, dtype, op, streams):
+        return self._each(
+            lambda r, s: lib.flagcxCustomAllReduceImpl(sends[r], recvs[r], count, dtype, op, self.comms[r], s), streams)
+
+    def reduce(self, sends, recvs, count, dtype, op, root, streams):
+        return self._each(
+            lambda r, s: lib.flagcxReduce(sends[r], recvs[r], count, dtype, op, root, self.comms[r], s), streams)
+
+    def reduce_scatter(self, sends, recvs, recvcount, dtype, op, streams):
+        return self._each(
+            lambda r, s: lib.flagcxReduceScatter(sends[r], recvs[r], recvcount, dtype, op, self.comms[r], s), streams)
+
+    def all_gather(self, sends, recvs, sendcount, dtype, streams):
+        return self._each(lambda r, s: lib.flagcxAllGather(sends[r], recvs[r], sendcount, dtype, self.comms[r], s),
+                          streams)
+
+    def all_to_allv(self, sends, sendcounts, sdispls, recvs, recvcounts, rdispls, dtype, streams):
+        return self._each(
+            lambda r, s: lib.flagcxAlltoAllv(sends[r], _szs(sendcounts[r]), _szs(sdispls[r]), recvs[r],
+                                             _szs(recvcounts[r]), _szs(rdispls[r]), dtype, self.comms[r], s), streams)
+
+    def register_windows(self, windows, nbytes):
+        arr = (C.c_void_p * self.n)(*windows) if windows else None
+        return lib.fxSimRegisterWindows(self.comms[0], arr, nbytes)

@@ -1,0 +1,118 @@
+/*
+ * FlagCX collective entry points over SIMULATED ranks on one GPU.
+ *
+ * The five collectives keep the exact C signatures of flagcx/include/flagcx.h
+ * (flagcxReduce :371-373, flagcxAllReduce :425-428, flagcxReduceScatter
+ * :441-444, flagcxAllGather :456-458, flagcxAlltoAllv :480-484) and the
+ * custom-op hook flagcxCustomAllReduceImpl that of
+ * flagcx/adaptor/kernel/nvidia/custom_allreduce.cu:604-607 (typedef
+ * flagcx/core/include/dev_comm_state.h:20-23).  What differs is the
+ * communicator: a group of n `flagcxComm_t` living in one process, whose
+ * "peer IPC buffers" are ordinary allocations in the same GPU's HBM.  No
+ * inter-GPU transport exists here.
+ *
+ * Calling convention (single-process multi-rank, like a grouped launch): every
+ * rank of the group calls the same collective once; calls are enqueue-only
+ * (flagcx.h:345-346).  The work is launched when the last rank has posted, on
+ * that caller's stream, after waiting for the other ranks' streams; those
+ * streams in turn wait for the result.  In-place rules are FlagCX's
+ * (flagcx.h:369,423,439,454).
+ */
+#ifndef FLAGCX_AMD_FX_SIM_H_
+#define FLAGCX_AMD_FX_SIM_H_
+
+#include "flagcx_amd/fx_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Create / destroy a group of nranks communicators on the current device
+ * (stand-in for flagcxCommInitRank, flagcx/flagcx.cc:1943-2358, whose
+ * bootstrap is multi-process). */
+flagcxResult_t fxSimCommInitAll(flagcxComm_t *comms, int nranks);
+flagcxResult_t fxSimCommDestroyAll(flagcxComm_t *comms, int nranks);
+
+/* Configuration keys (defaults come from the same environment variables the
+ * reference reads, flagcx/runner/uni_runner_impl.cc:21-26, uni_runner.cc:10-12). */
+enum {
+  FX_SIM_ALGO = 0,         /* FX_ALGO_*                                   */
+  FX_SIM_ORDER = 1,        /* FX_ORDER_*                                  */
+  FX_SIM_NSLICES = 2,      /* FLAGCX_UNIRUNNER_NSLICES (default 1)        */
+  FX_SIM_NREDSLICES = 3,   /* FLAGCX_UNIRUNNER_NREDSLICES (0 = automatic) */
+  FX_SIM_REDSLICESIZE = 4  /* FLAGCX_UNIRUNNER_REDSLICESIZE (65536 elems) */
+};
+enum {
+  FX_ALGO_DIRECT = 0, /* one k-way reduce per slice, then all-gather copies */
+  FX_ALGO_RING = 1    /* n-1 two-input ring steps, then n-1 copy steps      */
+};
+enum {
+  FX_ORDER_RANK = 0, /* rank 0,1,..,n-1: the custom allreduce's peer loop    */
+  FX_ORDER_RING = 1  /* the rotated order a ring yields for each chunk       */
+};
+flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value);
+
+flagcxResult_t flagcxCommCount(const flagcxComm_t comm, int *count);
+flagcxResult_t flagcxCommUserRank(const flagcxComm_t comm, int *rank);
+
+flagcxResult_t flagcxReduce(const void *sendbuff, void *recvbuff, size_t count,
+                            flagcxDataType_t datatype, flagcxRedOp_t op,
+                            int root, flagcxComm_t comm, flagcxStream_t stream);
+flagcxResult_t flagcxAllReduce(const void *sendbuff, void *recvbuff,
+                               size_t count, flagcxDataType_t datatype,
+                               flagcxRedOp_t op, flagcxComm_t comm,
+                               flagcxStream_t stream);
+flagcxResult_t flagcxReduceScatter(const void *sendbuff, void *recvbuff,
+                                   size_t recvcount, flagcxDataType_t datatype,
+                                   flagcxRedOp_t op, flagcxComm_t comm,
+                                   flagcxStream_t stream);
+flagcxResult_t flagcxAllGather(const void *sendbuff, void *recvbuff,
+                               size_t sendcount, flagcxDataType_t datatype,
+                               flagcxComm_t comm, flagcxStream_t stream);
+flagcxResult_t flagcxAlltoAllv(const void *sendbuff, size_t *sendcounts,
+                               size_t *sdispls, void *recvbuff,
+                               size_t *recvcounts, size_t *rdispls,
+                               flagcxDataType_t datatype, flagcxComm_t comm,
+                               flagcxStream_t stream);
+
+/*
+ * Custom allreduce hook: this rank's result = k-way reduce over all ranks'
+ * registered send windows, in rank order, written to recvbuff.  sendbuff is
+ * first staged into this rank's window unless it already is the window.
+ * Returns flagcxNotSupported (caller falls through, flagcx.cc:2673-2680) for
+ * avg, for types outside {fp16, bf16, fp32, int32}, when no window is
+ * registered or when the message exceeds it.  Unlike the reference it accepts
+ * every op on every type, odd counts and unaligned recvbuff.
+ */
+flagcxResult_t flagcxCustomAllReduceImpl(const void *sendbuff, void *recvbuff,
+                                         size_t count,
+                                         flagcxDataType_t datatype,
+                                         flagcxRedOp_t op, flagcxComm_t comm,
+                                         flagcxStream_t stream);
+/* Register the per-rank staged send windows (the reference's IPC-mapped
+ * sendStagedBuff, flagcx.cc:1617-1779; default size 8 MiB, :1606).  `windows`
+ * has nranks device pointers of `bytes` each; NULL unregisters. */
+flagcxResult_t fxSimRegisterWindows(flagcxComm_t comm, void *const *windows,
+                                    size_t bytes);
+
+/* Partition nodes of the reference's DAG builders, for inspection and tests. */
+typedef struct fxRedNode {
+  int32_t step, rank;
+  int32_t in1_buf, in2_buf, out_buf; /* 0 sendbuff, 1 recvbuff, 2 scratch */
+  int32_t slice;
+  uint64_t in1_off, in2_off, out_off, count; /* elements */
+} fxRedNode;
+/* initUniRunnerStateSlicedAR (uni_runner_impl.cc:661-1007), reduce nodes only */
+size_t fx_part_ring_ar(size_t count, int nranks, int rank, size_t nslices,
+                       size_t nred, fxRedNode *nodes);
+/* initUniRunnerStateRingRS (uni_runner_impl.cc:1009-1264) */
+size_t fx_part_ring_rs(size_t recvcount, int nranks, int rank, size_t nslices,
+                       size_t nred, fxRedNode *nodes);
+/* initUniRunnerStateLocRed (uni_runner_impl.cc:82-157) */
+size_t fx_part_locred(size_t count, int nranks, int rank, size_t nslices,
+                      fxRedNode *nodes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

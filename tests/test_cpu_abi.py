@@ -1,0 +1,195 @@
+"""Host-side checks that need no GPU: the shared libraries load, export every
+symbol the headers declare, the plugin passes the reference loader's validation,
+and the host arithmetic (partition, trigger layout, synthetic data) agrees with
+the oracle."""
+import ctypes as C
+import glob
+import itertools
+import os
+import re
+
+import numpy as np
+import pytest
+
+from flagcx_amd import _native as N
+from flagcx_amd import adaptor
+from flagcx_amd import kernels as K
+from oracle import fx_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    names = set()
+    for h in glob.glob(os.path.join(ROOT, "include", "flagcx_amd", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(h).read(), flags=re.S)
+        text = text.split("struct flagcxDeviceAdaptor_v1")[0]          # function POINTERS are not exports
+        for m in re.finditer(r"^(?!typedef)[A-Za-z_][\w \*]*?\b(\w+)\s*\([^;{]*\)\s*;", text, flags=re.M):
+            names.add(m.group(1))
+    return names
+
+
+def test_kernel_library_exports_every_declared_symbol():
+    declared = _declared_functions()
+    assert {"fx_reduce_copy", "fx_reduce_slices", "fx_pack", "flagcxAllReduce", "flagcxCustomAllReduceImpl",
+            "fx_synth_fill", "fx_part_ring_ar"} <= declared
+    missing = [n for n in sorted(declared) if not hasattr(N.lib, n)]
+    assert not missing, f"declared in include/ but not exported: {missing}"
+    assert set(N.exported_symbols()) <= declared          # the binding uses nothing undeclared
+
+
+def test_plugin_passes_the_reference_loader_checks():
+    t = adaptor.load_plugin()
+    assert t.name == b"MI355X"
+    # name[32] + 48 pointers (flagcx_device_adaptor.h:30-116)
+    assert C.sizeof(adaptor.DeviceAdaptorV1) == 32 + 48 * C.sizeof(C.c_void_p)
+    assert len(adaptor.REQUIRED) == 32
+    for f in adaptor.REQUIRED:
+        assert getattr(t, f), f
+    # the hot path additionally needs these two (uni_runner_impl.cc:1815; core/group.cc:451-453)
+    assert t.hostGetDevicePointer and t.launchDeviceFunc
+    assert t.getDeviceProperties and t.getDevicePciBusId and t.getDeviceByPciBusId and t.dmaSupport
+    # only the plugin symbol is exported
+    out = os.popen(f"nm -D --defined-only {N.PLUGIN_LIB}").read()
+    syms = [l.split()[-1] for l in out.splitlines() if " D " in l or " T " in l]
+    assert syms == ["flagcxDeviceAdaptorPlugin_v1"]
+
+
+def test_loader_rejects_bad_plugins(tmp_path):
+    with pytest.raises(ImportError):
+        adaptor.load_plugin(str(tmp_path / "nope.so"))
+    with pytest.raises(ImportError):                       # a library without the versioned symbol
+        adaptor.load_plugin(N.KERNEL_LIB)
+
+
+def test_host_argument_guards_of_the_plugin():
+    t = adaptor.load_plugin()
+    assert t.getDevice(None) == N.INVALID_ARGUMENT
+    assert t.getDeviceCount(None) == N.INVALID_ARGUMENT
+    assert t.getVendor(None) == N.INVALID_ARGUMENT
+    v = C.create_string_buffer(128)
+    assert t.getVendor(v) == N.SUCCESS and v.value == b"AMD"
+    assert t.hostGetDevicePointer(None, None) == N.INVALID_ARGUMENT
+    assert t.eventElapsedTime(None, None, None) == N.INVALID_ARGUMENT
+    assert t.ipcMemHandleGet(None, None) == N.INVALID_ARGUMENT
+    assert t.ipcMemHandleClose(None) == N.INVALID_ARGUMENT
+    assert t.getDevicePciBusId(None, 16, 0) == N.INVALID_ARGUMENT
+    assert t.getDeviceProperties(None, 0) == N.INVALID_ARGUMENT
+    assert t.getDeviceByPciBusId(None, None) == N.INVALID_ARGUMENT
+    assert t.streamFree(None) == N.SUCCESS and t.streamDestroy(None) == N.SUCCESS
+    assert t.eventDestroy(None) == N.SUCCESS
+    h, sz = C.c_void_p(), C.c_size_t()
+    assert t.ipcMemHandleCreate(C.byref(h), C.byref(sz)) == N.SUCCESS and h.value and sz.value == 64
+    assert t.ipcMemHandleFree(h) == N.SUCCESS
+    dma = C.c_bool(True)
+    assert t.dmaSupport(C.byref(dma)) == N.SUCCESS and dma.value is False
+
+
+def test_dtype_sizes():
+    # flagcx/flagcx.cc:35-66
+    want = {0: 1, 1: 1, 2: 4, 3: 4, 4: 8, 5: 8, 6: 2, 7: 4, 8: 8, 9: 2, 10: 0, -1: 0}
+    for dt, sz in want.items():
+        assert N.lib.fx_dtype_size(dt) == sz
+        if sz and dt in (2, 6, 7, 9):
+            assert O.lib.oracle_dtype_size(dt) == sz
+
+
+def test_split_and_nredslices_match_oracle():
+    for total, parts in itertools.product([0, 1, 5, 63, 64, 65, 1000003, 33554432, 2**33 + 7], [1, 2, 3, 7, 8, 64]):
+        for idx in {0, 1, parts // 2, parts - 1}:
+            if idx < parts:
+                assert K.split(total, parts, idx) == O.split(total, parts, idx)
+    for count, n, S, R, sz in itertools.product([0, 1, 5, 524288, 524289, 33554432, 10**9], [1, 2, 8], [1, 3, 8],
+                                                [0, 4], [0, 1, 65536, 262144]):
+        assert N.lib.fx_nredslices(count, n, S, R, sz) == O.lib.oracle_nredslices(count, n, S, R, sz)
+
+
+def _nodes(fn, *args):
+    n = fn(*args, None)
+    arr = (N.RedNode * max(n, 1))()
+    assert fn(*args, arr) == n
+    return [arr[i] for i in range(n)]
+
+
+def _same(a, b):
+    f = ["step", "rank", "in1_buf", "in2_buf", "out_buf", "slice", "in1_off", "in2_off", "out_off", "count"]
+    return all(getattr(a, x) == getattr(b, x) for x in f)
+
+
+@pytest.mark.parametrize("count,n,S,R", [(33554432, 8, 8, 2), (1000003, 8, 3, 2), (17, 4, 2, 3), (5, 8, 1, 1),
+                                          (64, 2, 1, 1), (12345, 3, 4, 5), (0, 4, 2, 2)])
+def test_partition_plans_match_oracle(count, n, S, R):
+    for rank in range(n):
+        a, b = _nodes(N.lib.fx_part_ring_ar, count, n, rank, S, R), O.plan_ring_ar(count, n, rank, S, R)
+        assert len(a) == len(b) and all(_same(x, y) for x, y in zip(a, b))
+        a, b = _nodes(N.lib.fx_part_ring_rs, count, n, rank, S, R), O.plan_ring_rs(count, n, rank, S, R)
+        assert len(a) == len(b) and all(_same(x, y) for x, y in zip(a, b))
+        a, b = _nodes(N.lib.fx_part_locred, count, n, rank, S), O.plan_locred(count, n, rank, S)
+        assert len(a) == len(b) and all(_same(x, y) for x, y in zip(a, b))
+    assert N.lib.fx_part_ring_ar(count, 1, 0, S, R, None) == 0
+
+
+def test_trigger_set_get_round_trip_and_oracle_layout():
+    rng = np.random.default_rng(2)
+    for _ in range(200):
+        in1, in2, out = (int(x) for x in rng.integers(0, 2**63, 3))
+        count, nth = int(rng.integers(0, 2**32)), int(rng.integers(0, 2**16))
+        dt, op, st = int(rng.integers(0, 16)), int(rng.integers(0, 16)), int(rng.integers(0, 4))
+        t = K.make_trigger(in1, in2, out, count, nth, dt, op, st)
+        assert list(t.value) == O.trigger_encode(in1, in2, out, count, nth, dt, op, st)
+        assert K.trigger_fields(t) == dict(in1=in1, in2=in2, out=out, count=count, nthreads=nth, dtype=dt, op=op,
+                                           state=st)
+    assert C.sizeof(N.ReduceTrigger) == 32 and C.sizeof(N.SliceDesc) == 80
+
+
+def test_synth_is_deterministic_and_thread_independent():
+    for dtype, dist, a, b in ((N.DT_FP32, K.SYNTH_UNIFORM, -1, 1), (N.DT_BF16, K.SYNTH_NORMAL, 0, 1),
+                              (N.DT_FP16, K.SYNTH_NORMAL, 0, 1), (N.DT_INT32, K.SYNTH_UNIFORM_INT, -2**20, 2**20)):
+        x1 = K.synth(100001, dtype, dist, a, b, seed=5, stream=2, threads=1)
+        x8 = K.synth(100001, dtype, dist, a, b, seed=5, stream=2, threads=8)
+        assert np.array_equal(x1, x8)
+        assert np.array_equal(x1[:777], K.synth(777, dtype, dist, a, b, seed=5, stream=2))   # prefix property
+        assert not np.array_equal(x1, K.synth(100001, dtype, dist, a, b, seed=5, stream=3))
+        assert not np.array_equal(x1, K.synth(100001, dtype, dist, a, b, seed=6, stream=2))
+    u = K.synth(400000, N.DT_FP32, K.SYNTH_UNIFORM, -1, 1, seed=0)
+    assert -1 <= u.min() and u.max() < 1 and abs(u.mean()) < 0.01 and abs(u.std() - 3 ** -0.5) < 0.01
+    g = K.synth(400000, N.DT_FP64, K.SYNTH_NORMAL, 0, 0.02, seed=4)
+    assert abs(g.mean()) < 2e-4 and abs(g.std() - 0.02) < 2e-4
+    i = K.synth(400000, N.DT_INT32, K.SYNTH_UNIFORM_INT, -2**20, 2**20, seed=2)
+    assert i.min() >= -2**20 and i.max() <= 2**20 and i.min() < -2**20 + 100 and i.max() > 2**20 - 100
+    # 16-bit outputs are correctly rounded versions of the same fp32 stream
+    f = K.synth(50000, N.DT_FP32, K.SYNTH_NORMAL, 0, 1, seed=1)
+    h = K.synth(50000, N.DT_FP16, K.SYNTH_NORMAL, 0, 1, seed=1)
+    bf = K.synth(50000, N.DT_BF16, K.SYNTH_NORMAL, 0, 1, seed=1)
+    assert np.array_equal(h, f.astype(np.float16).view(np.uint16))
+    assert np.array_equal(bf, np.array([O.lib.oracle_f32_to_bf16(float(x)) for x in f], np.uint16))
+
+
+def test_argument_screening_needs_no_gpu():
+    """Rejections happen before any device call, so they are testable here."""
+    p = 0x1000
+    rc = lambda **kw: K.reduce_copy(kw.get("out", p), kw.get("ins", [p, p]), kw.get("n", 4), kw.get("dtype", N.DT_FP32),
+                                    kw.get("op", N.OP_SUM), kw.get("first", 0))
+    assert rc(dtype=N.DT_FP64) == N.NOT_SUPPORTED
+    assert rc(dtype=N.DT_UINT8) == N.NOT_SUPPORTED
+    assert rc(op=N.OP_AVG) == N.NOT_SUPPORTED
+    assert rc(dtype=10) == N.INVALID_ARGUMENT and rc(dtype=-1) == N.INVALID_ARGUMENT
+    assert rc(op=5) == N.INVALID_ARGUMENT
+    assert rc(first=2) == N.INVALID_ARGUMENT and rc(first=-1) == N.INVALID_ARGUMENT
+    assert rc(out=None) == N.INVALID_ARGUMENT
+    assert rc(out=p + 1) == N.INVALID_ARGUMENT
+    assert rc(dtype=N.DT_BF16, ins=[p, p + 1]) == N.INVALID_ARGUMENT
+    assert rc(ins=[p] * 65) == N.INVALID_ARGUMENT
+    assert rc(n=0, out=None, ins=[None]) == N.SUCCESS
+    assert K.reduce_slices([], 2, N.DT_FP32, N.OP_SUM) == N.SUCCESS
+    assert K.reduce_slices([([p, p], p, 4)], 9, N.DT_FP32, N.OP_SUM) == N.INVALID_ARGUMENT
+    assert K.reduce_slices([([p, None], p, 4)], 2, N.DT_FP32, N.OP_SUM) == N.INVALID_ARGUMENT
+    assert K.copy_slices([(None, p, 4)]) == N.INVALID_ARGUMENT
+    assert K.copy_slices([(None, None, 0)]) == N.SUCCESS
+    assert K.pack(p, p, [1], [0], 10) == N.INVALID_ARGUMENT
+    assert K.pack(None, None, [0, 0], [0, 0], N.DT_FP32) == N.SUCCESS
+    assert N.lib.fxSimCommInitAll(None, 2) == N.INVALID_ARGUMENT
+    comms = (C.c_void_p * 2)()
+    assert N.lib.fxSimCommInitAll(comms, 0) == N.INVALID_ARGUMENT
+    assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP64, N.OP_SUM, None, None) == N.NOT_SUPPORTED
+    assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, None, None) == N.INVALID_ARGUMENT

@@ -1,0 +1,250 @@
+"""Collective-shaped entry points over simulated ranks: closed forms of the
+reference's own collective tests, parity with the hop-by-hop ring oracle, and
+the custom allreduce hook."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from flagcx_amd import _native as N
+from flagcx_amd import sim as S
+from oracle import fx_oracle as O
+from tests.util import DTYPES, DevBufs, assert_parity, seeded_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def stream(dev):
+    s = dev.stream_create()
+    yield s
+    dev.stream_destroy(s)
+
+
+def _allreduce(dev, stream, sends, dtype, op, inplace=False, **cfg):
+    n, count = len(sends), sends[0].size
+    es = N.DTYPE_SIZE[dtype]
+    with DevBufs(dev) as b, S.SimGroup(n, **cfg) as g:
+        ds = [b.put(a) for a in sends]
+        dr = ds if inplace else [b.alloc(count * es) for _ in range(n)]
+        N.check(g.all_reduce(ds, dr, count, dtype, op, stream), "flagcxAllReduce")
+        dev.stream_sync(stream)
+        return [dev.to_host(p, count, N.NP_DTYPE[dtype]) for p in dr]
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 8])
+@pytest.mark.parametrize("algo", [S.ALGO_DIRECT, S.ALGO_RING])
+def test_allreduce_closed_forms(dev, stream, n, algo):
+    count = 4 * 1024 * 1024 // 4 if n == 8 else 10007       # runner/main_mpi.cpp:33-80 uses 4 MiB float buffers
+    i = np.arange(count)
+    # coll_allreduce.cpp:9-37
+    sends = [(r * 1000 + i % 10).astype(np.float32) for r in range(n)]
+    want = (n * (n - 1) // 2 * 1000 + n * (i % 10)).astype(np.float32)
+    for got in _allreduce(dev, stream, sends, N.DT_FP32, N.OP_SUM, algo=algo):
+        assert np.array_equal(got, want)
+    # coll_deviceptr_allreduce.cpp:72-73
+    sends = [np.full(count, r + 1, np.float32) for r in range(n)]
+    for got in _allreduce(dev, stream, sends, N.DT_FP32, N.OP_SUM, algo=algo, inplace=True):
+        assert (got == n * (n + 1) / 2).all()
+    # test/perf/host_api/test_allreduce.cpp:20-32 (exact in fp32)
+    sends = [((i % 10) * 2.0 ** (r % 30)).astype(np.float32) for r in range(n)]
+    want = sum(s.astype(np.float64) for s in sends).astype(np.float32)
+    for got in _allreduce(dev, stream, sends, N.DT_FP32, N.OP_SUM, algo=algo, nslices=3):
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dname", ["fp32", "int32"])
+@pytest.mark.parametrize("n,count,nslices,nred", [(8, 100003, 8, 2), (5, 77, 2, 0), (4, 3, 1, 0), (2, 65536, 4, 3)])
+def test_allreduce_matches_ring_oracle_bit_for_bit(dev, stream, dname, n, count, nslices, nred):
+    """fp32 sums depend on order: the ring algorithm and the direct k-way
+    algorithm in ring order must both reproduce the hop-by-hop oracle."""
+    dtype = DTYPES[dname]
+    sends = seeded_inputs(dtype, n, count, seed=13)
+    for op in (N.OP_SUM, N.OP_PROD, N.OP_MAX, N.OP_MIN):
+        want = O.ring_allreduce(sends, dtype, op)
+        for cfg in (dict(algo=S.ALGO_RING), dict(algo=S.ALGO_DIRECT, order=S.ORDER_RING)):
+            for inplace in (False, True):
+                got = _allreduce(dev, stream, sends, dtype, op, inplace=inplace, nslices=nslices, nredslices=nred,
+                                 redslicesize=1024, **cfg)
+                for r in range(n):
+                    assert_parity(got[r], want[r], dtype, op, f"{cfg} inplace={inplace} rank {r} op={op}")
+
+
+@pytest.mark.parametrize("dname", ["bf16", "fp16"])
+def test_allreduce_16bit_rank_order(dev, stream, dname):
+    """Default order = rank order = the custom allreduce's peer loop; 16-bit sums
+    accumulate in fp32 across all 8 ranks and round once."""
+    dtype = DTYPES[dname]
+    n, count = 8, 262144 + 5
+    sends = seeded_inputs(dtype, n, count, seed=1)
+    for op in (N.OP_SUM, N.OP_MAX):
+        want = O.reduce_copy(sends, dtype, op)
+        for got in _allreduce(dev, stream, sends, dtype, op, nslices=8, nredslices=2):
+            assert_parity(got, want, dtype, op, f"allreduce {dname} op={op}")
+
+
+def test_reduce_reducescatter_allgather(dev, stream):
+    n, rc = 8, 5001
+    dtype, es = N.DT_FP32, 4
+    sends = seeded_inputs(dtype, n, n * rc, seed=3)
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        ds = [b.put(a) for a in sends]
+        # Reduce to root 3; recvbuff NULL elsewhere (flagcx.h:365-366)
+        droot = b.alloc(n * rc * es)
+        recvs = [droot if r == 3 else None for r in range(n)]
+        N.check(g.reduce(ds, recvs, n * rc, dtype, N.OP_SUM, 3, stream))
+        dev.stream_sync(stream)
+        assert_parity(dev.to_host(droot, n * rc, np.float32), O.reduce_copy(sends, dtype, N.OP_SUM), dtype, N.OP_SUM)
+        # ReduceScatter: rank r gets block r; ring order and ring algorithm agree bit for bit
+        for cfg in (dict(algo=S.ALGO_RING, nslices=2, nredslices=3), dict(algo=S.ALGO_DIRECT, order=S.ORDER_RING),
+                    dict(algo=S.ALGO_DIRECT, order=S.ORDER_RANK)):
+            g.configure(**cfg)
+            dr = [b.alloc(rc * es) for _ in range(n)]
+            N.check(g.reduce_scatter(ds, dr, rc, dtype, N.OP_SUM, stream))
+            dev.stream_sync(stream)
+            for r in range(n):
+                first = (r + 1) % n if cfg.get("order", S.ORDER_RING) == S.ORDER_RING else 0
+                want = O.reduce_copy([s[r * rc:(r + 1) * rc] for s in sends], dtype, N.OP_SUM, first=first)
+                assert_parity(dev.to_host(dr[r], rc, np.float32), want, dtype, N.OP_SUM, f"RS {cfg} rank {r}")
+        # closed form of coll_reducescatter.cpp:27-39 style data
+        # AllGather: block r of every recvbuff is rank r's sendbuff; in place when send == recv + r*count
+        g.configure(algo=S.ALGO_DIRECT, order=S.ORDER_RANK, nslices=1, nredslices=0)
+        dg = [b.alloc(n * rc * es) for _ in range(n)]
+        small = [s[:rc] for s in sends]
+        for r in range(n):
+            dev.upload(dg[r] + r * rc * es, small[r])
+        N.check(g.all_gather([dg[r] + r * rc * es for r in range(n)], dg, rc, dtype, stream))
+        dev.stream_sync(stream)
+        want = np.concatenate(small)
+        for r in range(n):
+            assert np.array_equal(dev.to_host(dg[r], n * rc, np.float32), want)
+
+
+def test_reduce_scatter_in_place(dev, stream):
+    n, rc = 4, 3003
+    sends = seeded_inputs(N.DT_INT32, n, n * rc, seed=8)
+    for cfg in (dict(algo=S.ALGO_RING), dict(algo=S.ALGO_DIRECT)):
+        with DevBufs(dev) as b, S.SimGroup(n, order=S.ORDER_RING, **cfg) as g:
+            ds = [b.put(a) for a in sends]
+            dr = [ds[r] + r * rc * 4 for r in range(n)]           # flagcx.h:439
+            N.check(g.reduce_scatter(ds, dr, rc, N.DT_INT32, N.OP_SUM, stream))
+            dev.stream_sync(stream)
+            for r in range(n):
+                want = O.reduce_copy([s[r * rc:(r + 1) * rc] for s in sends], N.DT_INT32, N.OP_SUM)
+                assert np.array_equal(dev.to_host(dr[r], rc, np.int32), want)
+
+
+def test_alltoallv_matches_oracle(dev, stream):
+    n = 8
+    rng = np.random.default_rng(3)
+    counts = np.exp(rng.uniform(0, np.log(50000), (n, n))).astype(np.int64)     # counts[r][i]: r -> i
+    counts[2, 5] = 0
+    counts[4, 4] = 0
+    sd = np.zeros((n, n), np.int64)
+    rd = np.zeros((n, n), np.int64)
+    slen, rlen = [], []
+    for r in range(n):
+        order, pos = rng.permutation(n), 0
+        for i in order:
+            pos += int(rng.integers(0, 5))
+            sd[r, i] = pos
+            pos += int(counts[r, i])
+        slen.append(pos + 3)
+        order, pos = rng.permutation(n), 0
+        for i in order:
+            pos += int(rng.integers(0, 5))
+            rd[r, i] = pos
+            pos += int(counts[i, r])
+        rlen.append(pos + 3)
+    sends = [rng.integers(0, 2**32, slen[r], dtype=np.uint64).astype(np.uint32) for r in range(n)]
+    want = [np.zeros(rlen[r], np.uint32) for r in range(n)]
+    szs = lambda a: (C.c_size_t * a.size)(*[int(x) for x in a.ravel()])
+    vp = lambda arrs: (C.c_void_p * n)(*[a.ctypes.data for a in arrs])
+    O.lib.oracle_alltoallv(vp(want), vp(sends), szs(counts), szs(sd), szs(rd), n, 4)
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        ds = [b.put(a) for a in sends]
+        dr = [b.alloc(rlen[r] * 4) for r in range(n)]
+        for r in range(n):
+            dev.memset(dr[r], 0, rlen[r] * 4)
+        N.check(g.all_to_allv(ds, counts, sd, dr, counts.T, rd, N.DT_FP32, stream))
+        dev.stream_sync(stream)
+        for r in range(n):
+            assert np.array_equal(dev.to_host(dr[r], rlen[r], np.uint32), want[r]), r
+        bad = counts.T.copy()
+        bad[0, 1] += 1                                             # receiver expects more than is sent
+        assert g.all_to_allv(ds, counts, sd, dr, bad, rd, N.DT_FP32, stream) == N.INVALID_ARGUMENT
+
+
+def test_custom_allreduce_hook(dev, stream):
+    n, count = 8, (8 << 20) // 2            # the reference's 8 MiB staged window, bf16
+    dtype = N.DT_BF16
+    sends = seeded_inputs(dtype, n, count, seed=1)
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        ds = [b.put(a) for a in sends]
+        dr = [b.alloc(count * 2) for _ in range(n)]
+        # no windows registered -> caller falls through (flagcx.cc:2673-2680)
+        assert g.custom_all_reduce(ds, dr, count, dtype, N.OP_SUM, stream) == N.NOT_SUPPORTED
+        wins = [b.alloc(8 << 20) for _ in range(n)]
+        N.check(g.register_windows(wins, 8 << 20))
+        assert g.custom_all_reduce(ds, dr, count + 1, dtype, N.OP_SUM, stream) == N.NOT_SUPPORTED   # > window
+        assert g.custom_all_reduce(ds, dr, count, N.DT_FP64, N.OP_SUM, stream) == N.NOT_SUPPORTED
+        assert g.custom_all_reduce(ds, dr, count, dtype, N.OP_AVG, stream) == N.NOT_SUPPORTED
+        for op in (N.OP_SUM, N.OP_MIN):
+            N.check(g.custom_all_reduce(ds, dr, count, dtype, op, stream))
+            dev.stream_sync(stream)
+            want = O.reduce_copy(sends, dtype, op)
+            for r in range(n):
+                assert_parity(dev.to_host(dr[r], count, np.uint16), want, dtype, op, f"custom AR rank {r}")
+        # odd count (the reference drops the tail, custom_allreduce.cu:383-384) and in-place on the window
+        for r in range(n):
+            dev.upload(wins[r], sends[r][:1001])
+        N.check(g.custom_all_reduce(wins, dr, 1001, dtype, N.OP_SUM, stream))
+        dev.stream_sync(stream)
+        want = O.reduce_copy([s[:1001] for s in sends], dtype, N.OP_SUM)
+        assert_parity(dev.to_host(dr[5], 1001, np.uint16), want, dtype, N.OP_SUM, "odd count")
+
+
+def test_group_misuse_is_reported(dev, stream):
+    with DevBufs(dev) as b, S.SimGroup(2) as g:
+        p = b.alloc(64)
+        lib = N.lib
+        assert lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, g.comms[0], stream) == N.SUCCESS
+        assert lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, g.comms[0], stream) == N.INVALID_USAGE   # rank 0 twice
+        assert lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, g.comms[0], stream) == N.SUCCESS
+        assert lib.flagcxAllReduce(p, p, 8, N.DT_FP32, N.OP_SUM, g.comms[1], stream) == N.INVALID_ARGUMENT  # count differs
+        assert lib.flagcxReduce(p, p, 4, N.DT_FP32, N.OP_SUM, 2, g.comms[0], stream) == N.INVALID_ARGUMENT   # bad root
+        assert lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, g.comms[0], None) == N.INVALID_ARGUMENT     # no stream
+        cnt, rank = C.c_int(), C.c_int()
+        assert lib.flagcxCommCount(g.comms[1], C.byref(cnt)) == N.SUCCESS and cnt.value == 2
+        assert lib.flagcxCommUserRank(g.comms[1], C.byref(rank)) == N.SUCCESS and rank.value == 1
+        dev.stream_sync(stream)
+
+
+def test_ranks_on_different_streams(dev):
+    """Each simulated rank posts on its own stream; the last post waits for the
+    others' pending uploads and the others wait for the result."""
+    n, count = 4, 1 << 20
+    sends = seeded_inputs(N.DT_FP32, n, count, seed=17)
+    streams = [dev.stream_create() for _ in range(n)]
+    try:
+        with DevBufs(dev) as b, S.SimGroup(n) as g:
+            ds = [b.alloc(count * 4) for _ in range(n)]
+            dr = [b.alloc(count * 4) for _ in range(n)]
+            hosts = [dev.malloc(count * 4, N.MEM_HOST) for _ in range(n)]
+            for r in range(n):
+                C.memmove(hosts[r], sends[r].ctypes.data, count * 4)
+                N.check(dev.t.deviceMemcpy(ds[r], hosts[r], count * 4, N.MEMCPY_H2D, streams[r], None))  # async, own stream
+            N.check(g.all_reduce(ds, dr, count, N.DT_FP32, N.OP_SUM, streams))
+            out = [np.empty(count, np.float32) for _ in range(n)]
+            for r in range(n):          # read back on each rank's OWN stream, no device-wide sync
+                N.check(dev.t.deviceMemcpy(hosts[r], dr[r], count * 4, N.MEMCPY_D2H, streams[r], None))
+                dev.stream_sync(streams[r])
+                C.memmove(out[r].ctypes.data, hosts[r], count * 4)
+            want = O.reduce_copy(sends, N.DT_FP32, N.OP_SUM)
+            for r in range(n):
+                assert np.array_equal(out[r], want)
+            for h in hosts:
+                dev.free(h, N.MEM_HOST)
+    finally:
+        for s in streams:
+            dev.stream_destroy(s)

@@ -1,0 +1,174 @@
+"""GPU parity of the batched slice kernels (k-way descriptors, the reference's
+2-input triggers, device-resident plans), the copy phase and alltoallv
+pack / unpack, against the CPU oracle."""
+import numpy as np
+import pytest
+
+from flagcx_amd import _native as N
+from flagcx_amd import kernels as K
+from oracle import fx_oracle as O
+from tests.util import DTYPES, OPS, DevBufs, assert_parity, seeded_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _ragged_slices(rng, total, nslices):
+    """Non-overlapping (offset, count) pieces of [0,total) with gaps, odd sizes and an empty one."""
+    cuts = np.sort(rng.choice(np.arange(1, total), size=2 * nslices - 1, replace=False))
+    bounds = np.concatenate([[0], cuts, [total]])
+    sl = [(int(bounds[2 * i]), int(bounds[2 * i + 1] - bounds[2 * i])) for i in range(nslices)]
+    sl.insert(len(sl) // 2, (sl[0][0], 0))
+    return sl
+
+
+@pytest.mark.parametrize("dname", list(DTYPES))
+@pytest.mark.parametrize("k", [1, 2, 5, 8])
+def test_reduce_slices_ragged(dev, dname, k):
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    rng = np.random.default_rng(k)
+    total = 400000
+    ins = seeded_inputs(dtype, k, total, seed=21)
+    for nsl, op in ((3, N.OP_SUM), (40, N.OP_MAX), (70, N.OP_PROD), (5, N.OP_MIN)):   # 40, 70 > one argument block
+        sl = _ragged_slices(rng, total, nsl)
+        with DevBufs(dev) as b:
+            dins = [b.put(a) for a in ins]
+            dout = b.alloc(total * es)
+            dev.memset(dout, 0x5A, total * es)
+            descs = [([p + o * es for p in dins], dout + o * es, c) for o, c in sl]
+            N.check(K.reduce_slices(descs, k, dtype, op), "fx_reduce_slices")
+            dev.sync()
+            got = dev.to_host(dout, total, N.NP_DTYPE[dtype])
+        want = np.frombuffer(bytes([0x5A]) * (total * es), dtype=N.NP_DTYPE[dtype]).copy()
+        for o, c in sl:
+            if c:
+                want[o:o + c] = O.reduce_copy([a[o:o + c] for a in ins], dtype, op)
+        assert_parity(got, want, dtype, op, f"slices {dname} k={k} n={nsl}")
+
+
+def test_plan_equals_inline_slices_and_is_relaunchable(dev):
+    dtype, op, k, total = N.DT_BF16, N.OP_SUM, 8, 600000
+    rng = np.random.default_rng(3)
+    ins = seeded_inputs(dtype, k, total, seed=1)
+    sl = _ragged_slices(rng, total, 50)
+    with DevBufs(dev) as b:
+        dins = [b.put(a) for a in ins]
+        dout = b.alloc(total * 2)
+        descs = [([p + o * 2 for p in dins], dout + o * 2, c) for o, c in sl]
+        plan = K.Plan(descs, k, dtype, op)
+        for _ in range(3):
+            dev.memset(dout, 0, total * 2)
+            N.check(plan.launch(), "fx_plan_launch")
+            dev.sync()
+            got = dev.to_host(dout, total, np.uint16)
+            want = np.zeros(total, np.uint16)
+            for o, c in sl:
+                if c:
+                    want[o:o + c] = O.reduce_copy([a[o:o + c] for a in ins], dtype, op)
+            assert_parity(got, want, dtype, op, "plan")
+        plan.destroy()
+        empty = K.Plan([], 2, dtype, op)
+        assert empty.launch() == N.SUCCESS
+        empty.destroy()
+
+
+def test_triggers_ring_step_semantics(dev):
+    """2-input triggers in the reference's 32-byte format, output aliasing input1
+    (ring: output == input1, uni_runner_impl.cc:864-878), mixed dtype/op runs."""
+    n = 70001
+    f = seeded_inputs(N.DT_FP32, 2, n, seed=2)
+    i = seeded_inputs(N.DT_INT32, 2, n, seed=3)
+    h = seeded_inputs(N.DT_FP16, 2, n, seed=4)
+    with DevBufs(dev) as b:
+        df, di, dh = [b.put(a) for a in f], [b.put(a) for a in i], [b.put(a) for a in h]
+        half = n // 2
+        trig = [
+            K.make_trigger(df[0], df[1], df[0], half, 32, N.DT_FP32, N.OP_SUM),                      # in place on in1
+            K.make_trigger(df[0] + half * 4, df[1] + half * 4, df[0] + half * 4, n - half, 32, N.DT_FP32, N.OP_SUM),
+            K.make_trigger(di[0], di[1], di[0], n, 32, N.DT_INT32, N.OP_PROD),
+            K.make_trigger(dh[0], dh[1], dh[0], n, 32, N.DT_FP16, N.OP_MAX),
+            K.make_trigger(dh[0], dh[1], dh[1], 0, 32, N.DT_FP16, N.OP_MAX),                         # empty
+        ]
+        N.check(K.reduce_triggers(trig), "fx_reduce_triggers")
+        dev.sync()
+        assert_parity(dev.to_host(df[0], n, np.float32), O.reduce2(f[0], f[1], N.DT_FP32, N.OP_SUM), N.DT_FP32, N.OP_SUM)
+        assert_parity(dev.to_host(di[0], n, np.int32), O.reduce2(i[0], i[1], N.DT_INT32, N.OP_PROD), N.DT_INT32,
+                      N.OP_PROD)
+        assert_parity(dev.to_host(dh[0], n, np.uint16), O.reduce2(h[0], h[1], N.DT_FP16, N.OP_MAX), N.DT_FP16, N.OP_MAX)
+        bad = [K.make_trigger(df[0], df[1], df[0], 4, 32, N.DT_FP64, N.OP_SUM)]
+        assert K.reduce_triggers(bad) == N.NOT_SUPPORTED
+
+
+def test_reduce2_all_types(dev):
+    for dname, dtype in DTYPES.items():
+        a, c = seeded_inputs(dtype, 2, 12345, seed=9)
+        for op in OPS.values():
+            with DevBufs(dev) as b:
+                da, dc, do = b.put(a), b.put(c), b.alloc(12345 * 4)
+                N.check(K.reduce2(do, da, dc, 12345, dtype, op), "fx_reduce2")
+                dev.sync()
+                got = dev.to_host(do, 12345, N.NP_DTYPE[dtype])
+            assert_parity(got, O.reduce2(a, c, dtype, op), dtype, op, f"reduce2 {dname} {op}")
+
+
+def test_copy_slices_byte_granular(dev):
+    rng = np.random.default_rng(12)
+    src = rng.integers(0, 256, 3_000_000, dtype=np.uint8)
+    # (src offset, dst offset, bytes): aligned, co-misaligned, differently misaligned, odd lengths, tiny, empty
+    cases = [(0, 0, 1 << 20), (1 << 20, (1 << 20) + 16, 65536), (1200003, 1300003, 70001), (1400001, 1500006, 33333),
+             (1600000, 1700002, 2), (1800001, 1800001 + 100000, 1), (5, 2000000, 0), (2100002, 2200004, 40000)]
+    with DevBufs(dev) as b:
+        dsrc = b.put(src)
+        ddst = b.alloc(src.size)
+        dev.memset(ddst, 0xEE, src.size)
+        N.check(K.copy_slices([(dsrc + s, ddst + d, n) for s, d, n in cases]), "fx_copy_slices")
+        dev.sync()
+        got = dev.to_host(ddst, src.size, np.uint8)
+    want = np.full(src.size, 0xEE, np.uint8)
+    for s, d, n in cases:
+        want[d:d + n] = src[s:s + n]
+    assert np.array_equal(got, want)
+
+
+def _random_layout(rng, counts, slack):
+    """Random non-overlapping displacements for the given segment counts."""
+    order = rng.permutation(len(counts))
+    displs, pos = [0] * len(counts), 0
+    for i in order:
+        pos += int(rng.integers(0, slack))
+        displs[i] = pos
+        pos += int(counts[i])
+    return displs, pos + int(rng.integers(0, slack))
+
+
+@pytest.mark.parametrize("dname,np_t", [("fp32", np.uint32), ("bf16", np.uint16)])
+def test_pack_unpack_random_displacements(dev, dname, np_t):
+    dtype = DTYPES[dname]
+    rng = np.random.default_rng(31)
+    for trial in range(4):
+        npeers = [8, 8, 3, 40][trial]
+        counts = [int(np.exp(rng.uniform(0, np.log(200000)))) for _ in range(npeers)]
+        counts[rng.integers(0, npeers)] = 0                       # a silent peer
+        if trial == 1:
+            counts = [c // 4 * 4 for c in counts]                 # 16-byte friendly segments
+        sdispls, slen = _random_layout(rng, counts, 9)
+        rdispls, rlen = _random_layout(rng, counts, 9)
+        send = rng.integers(0, np.iinfo(np_t).max, slen, dtype=np.uint64).astype(np_t)
+        total = sum(counts)
+        with DevBufs(dev) as b:
+            dsend = b.put(send)
+            dpacked = b.alloc(total * send.itemsize + 64)
+            drecv = b.alloc(rlen * send.itemsize)
+            dev.memset(dpacked, 0x77, total * send.itemsize + 64)
+            dev.memset(drecv, 0, rlen * send.itemsize)
+            N.check(K.pack(dpacked, dsend, counts, sdispls, dtype), "fx_pack")
+            N.check(K.unpack(drecv, dpacked, counts, rdispls, dtype), "fx_unpack")
+            dev.sync()
+            packed = dev.to_host(dpacked, total, np_t)
+            guard = dev.to_host(dpacked + total * send.itemsize, 64, np.uint8)
+            recv = dev.to_host(drecv, rlen, np_t)
+        assert np.array_equal(packed, O.pack(send, counts, sdispls))
+        assert (guard == 0x77).all()
+        assert np.array_equal(recv, O.unpack(np.zeros(rlen, np_t), O.pack(send, counts, sdispls), counts, rdispls))
+        for c, sd, rd in zip(counts, sdispls, rdispls):           # the identity, segment by segment
+            assert np.array_equal(recv[rd:rd + c], send[sd:sd + c])

@@ -1,0 +1,146 @@
+#!/usr/bin/env python3
+"""Headline benchmark: achieved HBM GB/s of the k-way reduce-copy, bf16 sum,
+8 inputs x 512 MiB, fp32 accumulate, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one pass of the hot path over one batch: one fx_reduce_copy of
+8 x 268,435,456 bf16 elements into a ninth buffer.  Inputs are resident in HBM
+before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
+K_INPUTS = 8
+ELEMS = 268_435_456            # per input: 512 MiB of bf16
+SEED = 4                       # values N(0, 0.02)
+
+
+def cpu_baseline(k, sample_elems, threads_all):
+    """The reference's host reduce path shape -- k-1 successive two-input passes
+    over a running partial -- on a bounded sample of the same workload, timed on
+    this box's host cores.  bf16 has no CPU path in the reference, so this is the
+    oracle port."""
+    import numpy as np
+
+    from flagcx_amd import _native as N
+    from flagcx_amd import kernels as K
+    from oracle import fx_oracle as O
+
+    ins = [K.synth(sample_elems, N.DT_BF16, K.SYNTH_NORMAL, 0.0, 0.02, SEED, p, threads_all) for p in range(k)]
+    algo_bytes = (k + 1) * sample_elems * 2
+
+    def best(threads, reps):
+        O.lib.oracle_set_threads(threads)
+        t = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            O.host_ring_passes(ins, N.DT_BF16, N.OP_SUM)
+            t.append(time.perf_counter() - t0)
+        O.lib.oracle_set_threads(1)
+        return min(t)
+
+    t1 = best(1, 2)
+    tn = best(threads_all, 3)
+    return {
+        "value": round(algo_bytes / t1 / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"{k} inputs x {sample_elems} bf16 elements (N(0,0.02), seed {SEED}), {k - 1} two-input passes, "
+                  f"fp32 accumulate per pass, best of 2; same (k+1)*size byte count as the GPU figure",
+        "all_cores": {"value": round(algo_bytes / tn / 1e9, 3), "cores": threads_all},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--synthetic-fill", choices=["seeded", "memset"], default="seeded",
+                    help="memset skips host generation (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
+              "(no collectives or second GPU are used anywhere in this run)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+
+    from flagcx_amd import _native as N
+    from flagcx_amd import kernels as K
+    from flagcx_amd.adaptor import Device
+
+    dev = Device(0)
+    nbytes = ELEMS * 2
+    threads = min(16, len(os.sched_getaffinity(0)))
+    ins = []
+    for p in range(K_INPUTS):
+        d = dev.malloc(nbytes)
+        if args.synthetic_fill == "seeded":
+            host = K.synth(ELEMS, N.DT_BF16, K.SYNTH_NORMAL, 0.0, 0.02, SEED, p, threads)
+            dev.upload(d, host)
+            del host
+        else:
+            dev.memset(d, 0x3c + p, nbytes)
+        ins.append(d)
+    out = dev.malloc(nbytes)
+    stream = dev.stream_create()
+    raw = dev.raw_stream(stream)
+    algo_bytes = (K_INPUTS + 1) * nbytes
+
+    def step(dst):
+        N.check(K.reduce_copy(dst, ins, ELEMS, N.DT_BF16, N.OP_SUM, 0, raw), "fx_reduce_copy")
+
+    def timed(dst, steps, warmup):
+        for _ in range(warmup):
+            step(dst)
+        dev.sync()
+        e0, e1 = dev.event_create(), dev.event_create()
+        t0 = time.perf_counter()
+        dev.event_record(e0, stream)
+        for _ in range(steps):
+            step(dst)
+        dev.event_record(e1, stream)
+        dev.sync()
+        wall = time.perf_counter() - t0
+        ev_ms = dev.event_ms(e0, e1)
+        dev.event_destroy(e0)
+        dev.event_destroy(e1)
+        return wall * 1e3 / steps, ev_ms / steps
+
+    wall_ms, kern_ms = timed(out, args.steps, args.warmup)
+    _, inplace_ms = timed(ins[0], max(args.steps // 2, 1), 2)      # out = in[0]; destroys input 0, run last
+    gbs = algo_bytes / (wall_ms * 1e-3) / 1e9
+    kern_gbs = algo_bytes / (kern_ms * 1e-3) / 1e9
+    result = {
+        "metric": "achieved HBM GB/s (% of peak) for k-way reduce-copy, bf16 8-input 512 MiB",
+        "value": round(gbs, 1), "unit": "GB/s", "pct_of_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in/out, f32 accumulate",
+        "data": "synthetic" if args.synthetic_fill == "seeded" else "synthetic (memset pattern)",
+        "config": {"workload": "BASELINE configs[4]: bf16 sum reduce-copy, 8 inputs x 268,435,456 elements "
+                               "(512 MiB each), N(0,0.02) seed 4, out-of-place, one launch per step",
+                   "inputs": K_INPUTS, "elements_per_input": ELEMS, "op": "sum",
+                   "in_place_GBs": round(algo_bytes / (inplace_ms * 1e-3) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "achieved": round(kern_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(kern_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "reduceCopyDirect<bf16,sum,K=8>", "bytes_per_launch": algo_bytes,
+                     "avg_launch_ms": round(kern_ms, 4)},
+    }
+    for p in ins + [out]:
+        dev.free(p)
+    dev.stream_destroy(stream)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(K_INPUTS, 64 * 1024 * 1024, threads)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -65,6 +65,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--synthetic-fill", choices=["seeded", "memset"], default="seeded",
                     help="memset skips host generation (profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a plain 512 MiB -> 512 MiB copy instead (known traffic, used to scale "
+                         "the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
@@ -79,6 +82,16 @@ def main():
 
     dev = Device(0)
     nbytes = ELEMS * 2
+    if args.calibrate_copy:
+        src, dst = dev.malloc(nbytes), dev.malloc(nbytes)
+        dev.memset(src, 0x5a, nbytes)
+        dev.sync()
+        for _ in range(args.warmup + args.steps):
+            N.check(K.copy_slices([(src, dst, nbytes)]), "fx_copy_slices")
+        dev.sync()
+        print(json.dumps({"calibration": "copy", "bytes_read_per_launch": nbytes, "bytes_written_per_launch": nbytes,
+                          "launches": args.warmup + args.steps}))
+        return
     threads = min(16, len(os.sched_getaffinity(0)))
     ins = []
     for p in range(K_INPUTS):

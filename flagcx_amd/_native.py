@@ -70,7 +70,6 @@ _SIGS = {
     "fx_dtype_size": (_sz, [_i]),
     "fx_split": (None, [_sz, _sz, _sz, C.POINTER(_sz), C.POINTER(_sz)]),
     "fx_nredslices": (_sz, [_sz, _i, _sz, _sz, _sz]),
-    "fx_set_xcd_spread": (_i, [_i]),
     "fx_version": (C.c_char_p, []),
     "fx_synth_fill": (_i, [_vp, _sz, _i, _i, C.c_double, C.c_double, C.c_uint64, C.c_uint64, _i]),
 }

@@ -1,6 +1,5 @@
 // C ABI over the gfx950 kernels: argument checking, batching of slice
 // descriptors into launches, and device-resident plans.
-#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -13,18 +12,6 @@
 using namespace fx;
 
 namespace {
-
-std::atomic<int> gXcdSpread{-1};
-
-int xcdSpread() {
-  int v = gXcdSpread.load(std::memory_order_relaxed);
-  if (v < 0) {
-    const char *e = getenv("FX_XCD_SPREAD");
-    v = (e && *e) ? (atoi(e) != 0) : 0;
-    gXcdSpread.store(v, std::memory_order_relaxed);
-  }
-  return v;
-}
 
 // dtype / op screening.  Types FlagCX knows but this path does not carry
 // return flagcxNotSupported so a caller can fall through to another path;
@@ -58,7 +45,7 @@ flagcxResult_t sliceTiles(const fxSliceDesc &s, int k, int es, int U, uint64_t *
   if (!s.out || !aligned(s.out, es)) return flagcxInvalidArgument;
   for (int p = 0; p < k; p++)
     if (!s.in[p] || !aligned(s.in[p], es)) return flagcxInvalidArgument;
-  *tiles = tilesFor(s.out, s.count, es, U);
+  *tiles = tilesFor(s.out, s.in, k, s.count, es, U);
   return flagcxSuccess;
 }
 
@@ -119,12 +106,6 @@ extern "C" {
 
 const char *fx_version(void) { return "flagcx_amd 0.1 (gfx950)"; }
 
-int fx_set_xcd_spread(int mode) {
-  int prev = xcdSpread();
-  gXcdSpread.store(mode ? 1 : 0, std::memory_order_relaxed);
-  return prev;
-}
-
 size_t fx_dtype_size(int dtype) {
   switch (dtype) {
     case flagcxInt8:
@@ -156,7 +137,7 @@ int fx_reduce_copy(void *out, const void *const *in, int k, size_t count, int dt
     rot[j] = p;
   }
   const KernelSet *ks = setFor(dtype, op);
-  return ks->direct[k <= kMaxFixedK ? k : 0](out, rot, k, count, xcdSpread(), (hipStream_t)stream);
+  return ks->direct[k <= kMaxFixedK ? k : 0](out, rot, k, count, (hipStream_t)stream);
 }
 
 int fx_reduce2(void *out, const void *in1, const void *in2, size_t count, int dtype, int op, void *stream) {

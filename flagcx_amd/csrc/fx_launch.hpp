@@ -12,8 +12,7 @@ constexpr int unrollFor(int K) { return K == 0 ? 2 : (K == 1 ? 8 : 4); }
 
 struct KernelSet {
   // index = compile-time input count, 0 = runtime-k kernel
-  flagcxResult_t (*direct[kMaxFixedK + 1])(void *out, const void *const *in, int k, uint64_t count,
-                                           int xcdSpread, hipStream_t s);
+  flagcxResult_t (*direct[kMaxFixedK + 1])(void *out, const void *const *in, int k, uint64_t count, hipStream_t s);
   flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const InlineSliceTable &t, hipStream_t s);
   flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
                                                 uint32_t grid, hipStream_t s);
@@ -21,13 +20,13 @@ struct KernelSet {
 };
 
 // Tiles (workgroups) a segment of `count` elements needs with unroll U.
-inline uint64_t tilesFor(const void *out, uint64_t count, int es, int U) {
-  uint64_t nv = segVectors((uint64_t)(uintptr_t)out & 15u, count, es);
-  return (nv + (uint64_t)U * kBlock - 1) / ((uint64_t)U * kBlock);
+inline uint64_t tilesFor(const void *out, const void *const *in, int k, uint64_t count, int es, int U) {
+  if (count == 0) return 0;
+  return planTiles((uint64_t)(uintptr_t)out, count, es, U, coAlignedHost(out, in, k)).tiles();
 }
 
 template <class R, int K>
-flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t count, int xcdSpread, hipStream_t s) {
+flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t count, hipStream_t s) {
   constexpr int U = unrollFor(K);
   DirectArgs<K> a;
   const int kk = (K > 0) ? K : k;
@@ -35,13 +34,10 @@ flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t co
   a.out = out;
   a.count = count;
   a.k = kk;
-  uint64_t ntiles = tilesFor(out, count, R::ES, U);
+  uint64_t ntiles = tilesFor(out, in, kk, count, R::ES, U);
   if (ntiles == 0) return flagcxSuccess;
   if (ntiles > 0x7ffffff0ull) return flagcxInvalidArgument;
-  a.ntiles = (uint32_t)ntiles;
-  a.xcdSpread = (xcdSpread && ntiles >= 64) ? 1 : 0;
-  uint32_t grid = a.xcdSpread ? (uint32_t)((ntiles + 7) / 8 * 8) : (uint32_t)ntiles;
-  hipLaunchKernelGGL((reduceCopyDirect<R, K, U>), dim3(grid), dim3(kBlock), 0, s, a);
+  hipLaunchKernelGGL((reduceCopyDirect<R, K, U>), dim3((uint32_t)ntiles), dim3(kBlock), 0, s, a);
   FX_HIP(hipGetLastError());
   return flagcxSuccess;
 }

@@ -16,7 +16,9 @@
 // are always whole aligned vectors except in the first and last vector of a
 // segment, which fall back to element accesses.  Inputs that share the
 // output's misalignment take the vector-load path; others are gathered
-// element by element (coalesced across lanes, still one pass).
+// element by element (coalesced across lanes, still one pass).  Large
+// segments are handed to workgroups as 512-byte pieces 32 KiB apart (see
+// TilePlan) instead of contiguous 16 KiB runs.
 #pragma once
 #include "fx_common.hpp"
 
@@ -214,8 +216,52 @@ struct CopyRed {
 
 // ------------------------------------------------------------- one segment
 
-// A segment in the output-anchored index space.  Element v of the space lives
-// at base + v*ES; valid elements are [lead, end).  outBase is 16-byte aligned.
+// Tiling of a segment.  The index space is anchored at the output pointer
+// rounded down to 16 bytes: vector j covers bytes [16j, 16j+16) from there and
+// the valid elements are [lead, end).  A tile is V = U*kBlock vectors.
+//
+// Striped zone.  On MI355X a workgroup that touches one contiguous 16 KiB per
+// stream spreads its few stores thinly over many DRAM channels, and a sparse
+// write stream mixed into reads is expensive (measured: 5.9 TB/s for 8 inputs).
+// The same bytes moved as 512-byte pieces 32 KiB apart reach 6.4-6.5 TB/s.  So
+// the part of a segment that consists of whole regions of kStripeTiles tiles,
+// aligned in ABSOLUTE address, is handed out striped: tile i of a region owns
+// piece i of every 32 KiB row of that region.  The rest (head before the first
+// region boundary, tail after the last) is handed out contiguously.
+constexpr uint32_t kPieceVecs = 32;                           // 512 bytes
+constexpr uint32_t kStripeTiles = 64;                         // tiles per region
+constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;      // 32 KiB
+
+struct TilePlan {
+  uint64_t nv;                 // vectors spanned by the segment
+  uint64_t firstFull, endFull; // vectors [firstFull, endFull) lie wholly inside the segment
+  uint64_t zs, ze;             // striped zone [zs, ze) in vectors; empty when zs == ze
+  uint32_t zoneTiles, headTiles, tailTiles;
+  __host__ __device__ uint64_t tiles() const { return (uint64_t)zoneTiles + headTiles + tailTiles; }
+};
+
+// Same function on host (grid size, tile prefix tables) and device (mapping).
+__host__ __device__ inline TilePlan planTiles(uint64_t outAddr, uint64_t count, int es, int U, bool coAligned) {
+  TilePlan tp;
+  const uint64_t V = (uint64_t)U * kBlock, RV = V * kStripeTiles, ve = 16u / (uint32_t)es;
+  const uint64_t mis = outAddr & 15u, lead = mis / (uint32_t)es, end = lead + count;
+  tp.nv = (end + ve - 1) / ve;
+  tp.firstFull = (lead + ve - 1) / ve;
+  tp.endFull = end / ve;
+  const uint64_t a0 = (outAddr - mis) >> 4;  // absolute vector number of vector 0
+  uint64_t zs = (a0 + tp.firstFull + RV - 1) / RV * RV, ze = (a0 + tp.endFull) / RV * RV;
+  if (!coAligned || ze <= zs || count == 0) {
+    tp.zs = tp.ze = 0;
+  } else {
+    tp.zs = zs - a0;
+    tp.ze = ze - a0;
+  }
+  tp.zoneTiles = (uint32_t)((tp.ze - tp.zs) / V);
+  tp.headTiles = (uint32_t)((tp.zs + V - 1) / V);
+  tp.tailTiles = (uint32_t)((tp.nv - tp.ze + V - 1) / V);
+  return tp;
+}
+
 template <int K>
 struct Seg {
   const char *in[K];
@@ -299,55 +345,78 @@ __device__ __forceinline__ void reduceVectorChecked(const Seg<K> &sg, uint64_t j
     scatterElems<R::ES>(sg.out, e0, lo, hi, r);
 }
 
-// One tile = U * kBlock vectors.  Interior tiles of co-aligned segments run the
-// branch-free path with all K*U loads in flight.
+// Branch-free body: lane handles U whole vectors at byte offsets off + u*ustride
+// of every stream, all K*U loads in flight before the first use.
 template <class R, int K, int U>
-__device__ __forceinline__ void reduceTile(const Seg<K> &sg, uint64_t tile) {
-  constexpr int VE = 16 / R::ES;
-  const uint64_t j0 = tile * (uint64_t)(U * kBlock);
-  const uint64_t firstFull = (sg.lead + VE - 1) / VE;
-  const uint64_t endFull = sg.end / VE;
-  const bool interior = sg.coAligned && j0 >= firstFull && j0 + U * kBlock <= endFull;
-  if (interior) {
-    const uint64_t off = (j0 + threadIdx.x) * 16;
-    if (K > 0) {
-      u32x4 v[U][K > 0 ? K : 1];
+__device__ __forceinline__ void reduceVectorsFast(const Seg<K> &sg, uint64_t off, uint64_t ustride) {
+  if (K > 0) {
+    u32x4 v[U][K > 0 ? K : 1];
 #pragma unroll
-      for (int u = 0; u < U; u++)
+    for (int u = 0; u < U; u++)
 #pragma unroll
-        for (int p = 0; p < K; p++) v[u][p] = ldg_stream(sg.inp(p) + off + (uint64_t)u * (kBlock * 16));
+      for (int p = 0; p < K; p++) v[u][p] = ldg_stream(sg.inp(p) + off + u * ustride);
 #pragma unroll
-      for (int u = 0; u < U; u++) {
-        typename R::Acc acc;
-        R::init(acc, v[u][0]);
+    for (int u = 0; u < U; u++) {
+      typename R::Acc acc;
+      R::init(acc, v[u][0]);
 #pragma unroll
-        for (int p = 1; p < K; p++) R::fold(acc, v[u][p]);
-        stg_stream(sg.out + off + (uint64_t)u * (kBlock * 16), R::finish(acc));
-      }
-    } else {
-      typename R::Acc acc[U];
-#pragma unroll
-      for (int u = 0; u < U; u++) R::init(acc[u], ldg_stream(sg.inp(0) + off + (uint64_t)u * (kBlock * 16)));
-      for (int p = 1; p < sg.inputs(); p++) {
-        const char *ip = sg.inp(p);
-        u32x4 v[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) v[u] = ldg_stream(ip + off + (uint64_t)u * (kBlock * 16));
-#pragma unroll
-        for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < U; u++) stg_stream(sg.out + off + (uint64_t)u * (kBlock * 16), R::finish(acc[u]));
+      for (int p = 1; p < K; p++) R::fold(acc, v[u][p]);
+      stg_stream(sg.out + off + u * ustride, R::finish(acc));
     }
   } else {
+    typename R::Acc acc[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) R::init(acc[u], ldg_stream(sg.inp(0) + off + u * ustride));
+    for (int p = 1; p < sg.inputs(); p++) {
+      const char *ip = sg.inp(p);
+      u32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u] = ldg_stream(ip + off + u * ustride);
+#pragma unroll
+      for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) stg_stream(sg.out + off + u * ustride, R::finish(acc[u]));
+  }
+}
+
+// Tile `tile` of the segment: striped zone first, then head, then tail.
+template <class R, int K, int U>
+__device__ __forceinline__ void reduceTile(const Seg<K> &sg, const TilePlan &tp, uint32_t tile) {
+  constexpr uint64_t V = (uint64_t)U * kBlock;
+  if (tile < tp.zoneTiles) {
+    // tile i of region r owns vectors zs + r*RV + row*kRowVecs + i*kPieceVecs + [0, kPieceVecs)
+    // for row = 0 .. V/kPieceVecs-1; lane (u, tid) takes row u*(kBlock/kPieceVecs) + tid/kPieceVecs.
+    const uint32_t r = tile / kStripeTiles, i = tile % kStripeTiles;
+    const uint64_t j = tp.zs + (uint64_t)r * (V * kStripeTiles) + (uint64_t)(threadIdx.x / kPieceVecs) * kRowVecs +
+                       i * kPieceVecs + (threadIdx.x % kPieceVecs);
+    reduceVectorsFast<R, K, U>(sg, j * 16, (uint64_t)(kBlock / kPieceVecs) * kRowVecs * 16);
+    return;
+  }
+  uint32_t t = tile - tp.zoneTiles;
+  uint64_t j0, limit;
+  if (t < tp.headTiles) {
+    j0 = (uint64_t)t * V;
+    limit = (tp.ze > tp.zs) ? tp.zs : tp.nv;   // the head stops where the zone begins
+  } else {
+    j0 = tp.ze + (uint64_t)(t - tp.headTiles) * V;
+    limit = tp.nv;
+  }
+  const uint64_t fastEnd = (limit < tp.endFull) ? limit : tp.endFull;
+  if (sg.coAligned && j0 >= tp.firstFull && j0 + V <= fastEnd) {
+    reduceVectorsFast<R, K, U>(sg, (j0 + threadIdx.x) * 16, (uint64_t)kBlock * 16);
+  } else {
 #pragma unroll 1
-    for (int u = 0; u < U; u++) reduceVectorChecked<R, K>(sg, j0 + (uint64_t)u * kBlock + threadIdx.x);
+    for (int u = 0; u < U; u++) {
+      const uint64_t j = j0 + (uint64_t)u * kBlock + threadIdx.x;
+      if (j < limit) reduceVectorChecked<R, K>(sg, j);
+    }
   }
 }
 
 // Build the output-anchored segment from raw element pointers.
-template <int ES, int K>
-__device__ __forceinline__ void makeSeg(Seg<K> &sg, const void *const *in, void *out, uint64_t count, int) {
+template <int ES, int U, int K>
+__device__ __forceinline__ TilePlan makeSeg(Seg<K> &sg, const void *const *in, void *out, uint64_t count, int) {
   const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
   sg.out = (char *)out - mis;
   sg.lead = mis / ES;
@@ -359,10 +428,11 @@ __device__ __forceinline__ void makeSeg(Seg<K> &sg, const void *const *in, void 
     sg.in[p] = (const char *)in[p] - mis;
   }
   sg.coAligned = co;
+  return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
 }
 
-template <int ES>
-__device__ __forceinline__ void makeSeg(Seg<0> &sg, const void *const *in, void *out, uint64_t count, int k) {
+template <int ES, int U>
+__device__ __forceinline__ TilePlan makeSeg(Seg<0> &sg, const void *const *in, void *out, uint64_t count, int k) {
   const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
   sg.raw = in;
   sg.mis = mis;
@@ -373,12 +443,15 @@ __device__ __forceinline__ void makeSeg(Seg<0> &sg, const void *const *in, void 
   bool co = true;
   for (int p = 0; p < k; p++) co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
   sg.coAligned = co;
+  return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
 }
 
-// Vectors spanned by a segment of `count` elements whose output pointer has
-// byte misalignment `mis` (host and device use the same formula).
-__host__ __device__ inline uint64_t segVectors(uint64_t mis, uint64_t count, int es) {
-  return (mis + count * (uint64_t)es + 15u) / 16u;
+// Host twin of the co-alignment test above.
+inline bool coAlignedHost(const void *out, const void *const *in, int k) {
+  const uintptr_t mis = (uintptr_t)out & 15u;
+  for (int p = 0; p < k; p++)
+    if (((uintptr_t)in[p] & 15u) != mis) return false;
+  return true;
 }
 
 // --------------------------------------------------------- kernel arguments
@@ -388,26 +461,14 @@ struct DirectArgs {
   const void *in[K > 0 ? K : kMaxK];
   void *out;
   uint64_t count;
-  uint32_t ntiles;
   int k;
-  int xcdSpread;   // 1: consecutive tiles of one XCD are contiguous in memory
 };
-
-// Workgroups are dealt round-robin to the 8 XCDs.  With xcdSpread the tile
-// index is rearranged so that each XCD walks one contiguous eighth of the
-// segment instead of every eighth tile.
-__device__ __forceinline__ uint32_t tileOfBlock(uint32_t b, uint32_t ntiles, int xcdSpread) {
-  if (!xcdSpread) return b;
-  const uint32_t per = (ntiles + 7u) / 8u;
-  return (b & 7u) * per + (b >> 3);
-}
 
 template <class R, int K, int U>
 __global__ void __launch_bounds__(kBlock) reduceCopyDirect(DirectArgs<K> a) {
   Seg<K> sg;
-  makeSeg<R::ES>(sg, a.in, a.out, a.count, a.k);
-  const uint32_t t = tileOfBlock(blockIdx.x, a.ntiles, a.xcdSpread);
-  if (t < a.ntiles) reduceTile<R, K, U>(sg, t);
+  const TilePlan tp = makeSeg<R::ES, U>(sg, a.in, a.out, a.count, a.k);
+  reduceTile<R, K, U>(sg, tp, blockIdx.x);
 }
 
 // Batched slices: a table of independent segments sharing dtype, op and k.
@@ -440,8 +501,8 @@ __device__ __forceinline__ void reduceSlicesBody(const SliceDescDev *d, const ui
   const uint32_t b = blockIdx.x;
   const uint32_t i = findSlice(tileStart, n, b);
   Seg<K> sg;
-  makeSeg<R::ES>(sg, d[i].in, d[i].out, d[i].count, K);
-  reduceTile<R, K, U>(sg, b - tileStart[i]);
+  const TilePlan tp = makeSeg<R::ES, U>(sg, d[i].in, d[i].out, d[i].count, K);
+  reduceTile<R, K, U>(sg, tp, b - tileStart[i]);
 }
 
 template <class R, int K, int U>

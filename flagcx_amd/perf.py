@@ -1,0 +1,182 @@
+"""Size / op sweeps in the style of FlagCX's perf harness
+(test/perf_common.cc:140-239: warmup 5, iters 20, sizes min..max x factor,
+algBw = bytes / 1e9 / t).  Usage:
+
+    python -m flagcx_amd.perf reduce  -k 4 -d fp16 -o sum -b 1K -e 1G -f 2 [--inplace]
+    python -m flagcx_amd.perf slices            # BASELINE config 2: rank shares in 512 KiB pieces + all-gather copy
+    python -m flagcx_amd.perf pack              # BASELINE config 4: alltoallv pack / unpack
+    python -m flagcx_amd.perf allreduce -n 8 -d bf16 -b 1M -e 64M
+"""
+import argparse
+import sys
+
+import numpy as np
+
+from . import _native as N
+from . import kernels as K
+from . import sim as S
+from .adaptor import Device
+
+DT = {"fp32": N.DT_FP32, "fp16": N.DT_FP16, "bf16": N.DT_BF16, "int32": N.DT_INT32}
+OP = {"sum": N.OP_SUM, "prod": N.OP_PROD, "max": N.OP_MAX, "min": N.OP_MIN}
+
+
+def size(s):
+    mult = {"K": 1 << 10, "M": 1 << 20, "G": 1 << 30}
+    return int(s[:-1]) * mult[s[-1].upper()] if s[-1].upper() in mult else int(s)
+
+
+class Timer:
+    def __init__(self, dev, warmup=5, iters=20):
+        self.dev, self.warmup, self.iters = dev, warmup, iters
+        self.stream = dev.stream_create()
+        self.raw = dev.raw_stream(self.stream)
+
+    def ms(self, fn):
+        d = self.dev
+        for _ in range(self.warmup):
+            fn()
+        d.stream_sync(self.stream)
+        e0, e1 = d.event_create(), d.event_create()
+        d.event_record(e0, self.stream)
+        for _ in range(self.iters):
+            fn()
+        d.event_record(e1, self.stream)
+        d.event_sync(e1)
+        t = d.event_ms(e0, e1) / self.iters
+        d.event_destroy(e0)
+        d.event_destroy(e1)
+        return t
+
+
+def row(label, nbytes, ms, algo_bytes):
+    print(f"{label:<44s} size {nbytes:>12d} B   {ms * 1e3:10.2f} us   {algo_bytes / ms / 1e6:9.1f} GB/s", flush=True)
+
+
+def run_reduce(dev, a):
+    t = Timer(dev)
+    dtype, op, k = DT[a.dtype], OP[a.op], a.k
+    es = N.DTYPE_SIZE[dtype]
+    emax = size(a.max)
+    ins = [dev.malloc(emax + a.misalign * es) for _ in range(k)]
+    for i, p in enumerate(ins):
+        dev.memset(p, 0x3c + i, emax)
+    out = ins[0] if a.inplace else dev.malloc(emax + a.misalign * es)
+    nbytes = size(a.min)
+    while nbytes <= emax:
+        n = nbytes // es
+        shift = [(a.misalign * es if a.mixed and i % 2 else 0) for i in range(k)]
+        fn = lambda: N.check(K.reduce_copy(out + (0 if a.inplace else a.misalign * es),
+                                           [p + (a.misalign * es if not a.mixed else s) for p, s in zip(ins, shift)]
+                                           if not a.inplace else ins, n, dtype, op, 0, t.raw))
+        row(f"reduce k={k} {a.dtype} {a.op}{' inplace' if a.inplace else ''}", nbytes, t.ms(fn), (k + 1) * nbytes)
+        nbytes *= a.factor
+
+
+def run_slices(dev, a):
+    """Config 2: 8 peers x 33,554,432 bf16; each rank share (4,194,304 el) in 8 slices x 2 pieces of 512 KiB."""
+    t = Timer(dev)
+    k, n, es = 8, 33_554_432, 2
+    ds = [dev.malloc(n * es) for _ in range(k)]
+    dr = [dev.malloc(n * es) for _ in range(k)]
+    for i, p in enumerate(ds):
+        dev.memset(p, 0x3c + i, n * es)
+    per_rank, copies = [], []
+    for ch in range(k):
+        ccnt, coff = K.split(n, k, ch)
+        owner = (ch - 1) % k
+        descs = []
+        for s in range(8):
+            scnt, soff = K.split(ccnt, 8, s)
+            for q in range(2):
+                rcnt, roff = K.split(scnt, 2, q)
+                off = (coff + soff + roff) * es
+                descs.append(([p + off for p in ds], dr[owner] + off, rcnt))
+        per_rank.append(descs)
+        copies += [(dr[owner] + coff * es, dr[r] + coff * es, ccnt * es) for r in range(k) if r != owner]
+    share_bytes = n // k * es
+    one = per_rank[0]
+    row("one rank share: 16 x 512 KiB, 8-way", share_bytes, t.ms(lambda: N.check(K.reduce_slices(one, k, N.DT_BF16, N.OP_SUM, t.raw))),
+        9 * share_bytes)
+    allr = [d for r in per_rank for d in r]
+    row("all 8 shares: 128 x 512 KiB, 8-way", n * es, t.ms(lambda: N.check(K.reduce_slices(allr, k, N.DT_BF16, N.OP_SUM, t.raw))),
+        9 * n * es)
+    plan = K.Plan(allr, k, N.DT_BF16, N.OP_SUM)
+    row("all 8 shares as a device-resident plan", n * es, t.ms(lambda: N.check(plan.launch(t.raw))), 9 * n * es)
+    onechunk = [([p for p in ds], dr[0], n // k)]
+    row("one share as ONE contiguous slice", share_bytes, t.ms(lambda: N.check(K.reduce_slices(onechunk, k, N.DT_BF16, N.OP_SUM, t.raw))),
+        9 * share_bytes)
+    # ring-faithful: 7 successive 2-input steps over the share (reported, not the target)
+    steps = [[([ds[0] + o, ds[1] + o], dr[0] + o, c) for (ins_, _, c), o in
+              zip(one, [d[1] - dr[-1 % k] for d in one])]]
+    two = [([d[0][0], d[0][1]], d[1], d[2]) for d in one]
+    row("ring-faithful: 7 x (16 x 512 KiB, 2-input)", share_bytes,
+        t.ms(lambda: [N.check(K.reduce_slices(two, 2, N.DT_BF16, N.OP_SUM, t.raw)) for _ in range(7)]), 7 * 3 * share_bytes)
+    one_rank_ag = [c for c in copies if c[1] - dr[0] >= 0 and c[1] - dr[0] < n * es]
+    row("all-gather copy, one rank: 7 x 8 MiB", 7 * share_bytes, t.ms(lambda: N.check(K.copy_slices(one_rank_ag, t.raw))),
+        2 * 7 * share_bytes)
+    row("all-gather copy, all ranks: 56 x 8 MiB", 56 * share_bytes, t.ms(lambda: N.check(K.copy_slices(copies, t.raw))),
+        2 * 56 * share_bytes)
+    with S.SimGroup(k, nslices=8, redslicesize=262144) as g:
+        row("flagcxAllReduce, 8 simulated ranks, 64 MiB", n * es,
+            t.ms(lambda: N.check(g.all_reduce(ds, dr, n, N.DT_BF16, N.OP_SUM, t.stream))), 9 * n * es + 2 * 56 * share_bytes)
+
+
+def run_pack(dev, a):
+    from tests.golden import workloads as W
+    t = Timer(dev)
+    counts, sd, slen, rd, rlen = W.cfg4_layout()
+    total = sum(counts)
+    dsend, dpacked, drecv = dev.malloc(slen * 4), dev.malloc(total * 4), dev.malloc(rlen * 4)
+    dev.memset(dsend, 1, slen * 4)
+    print("counts", counts, "sdispls % 4 el:", [d % 4 for d in sd], "slots % 4:", [int(x) % 4 for x in np.cumsum([0] + counts[:-1])])
+    row("pack   (config 4 layout)", total * 4, t.ms(lambda: N.check(K.pack(dpacked, dsend, counts, sd, N.DT_FP32, t.raw))), 2 * total * 4)
+    row("unpack (config 4 layout)", total * 4, t.ms(lambda: N.check(K.unpack(drecv, dpacked, counts, rd, N.DT_FP32, t.raw))), 2 * total * 4)
+    c4 = [c // 4 * 4 for c in counts]
+    s4 = [d // 4 * 4 for d in sd]
+    row("pack, counts/displs multiples of 16 B", sum(c4) * 4, t.ms(lambda: N.check(K.pack(dpacked, dsend, c4, s4, N.DT_FP32, t.raw))), 2 * sum(c4) * 4)
+    big = [4_194_304] * 8
+    bd = [i * 4_194_304 + 0 for i in range(8)]
+    dbig, dpk = dev.malloc(8 * 4_194_304 * 4 + 64), dev.malloc(8 * 4_194_304 * 4)
+    row("pack, 8 x 4,194,304 el aligned", sum(big) * 4, t.ms(lambda: N.check(K.pack(dpk, dbig, big, bd, N.DT_FP32, t.raw))), 2 * sum(big) * 4)
+    row("pack, 8 x 4,194,304 el, source off by 1 el", sum(big) * 4,
+        t.ms(lambda: N.check(K.pack(dpk, dbig + 4, big, bd, N.DT_FP32, t.raw))), 2 * sum(big) * 4)
+
+
+def run_allreduce(dev, a):
+    t = Timer(dev)
+    dtype, n = DT[a.dtype], a.nranks
+    es = N.DTYPE_SIZE[dtype]
+    emax = size(a.max)
+    ds = [dev.malloc(emax) for _ in range(n)]
+    dr = [dev.malloc(emax) for _ in range(n)]
+    for algo in (S.ALGO_DIRECT, S.ALGO_RING):
+        with S.SimGroup(n, algo=algo) as g:
+            nbytes = size(a.min)
+            while nbytes <= emax:
+                cnt = nbytes // es
+                row(f"allreduce n={n} {a.dtype} {'ring' if algo else 'direct'}", nbytes,
+                    t.ms(lambda: N.check(g.all_reduce(ds, dr, cnt, dtype, OP[a.op], t.stream))), nbytes)
+                nbytes *= a.factor
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce"])
+    ap.add_argument("-k", type=int, default=4)
+    ap.add_argument("-n", "--nranks", type=int, default=8)
+    ap.add_argument("-d", "--dtype", default="fp32", choices=list(DT))
+    ap.add_argument("-o", "--op", default="sum", choices=list(OP))
+    ap.add_argument("-b", "--min", default="1M")
+    ap.add_argument("-e", "--max", default="1G")
+    ap.add_argument("-f", "--factor", type=int, default=2)
+    ap.add_argument("--inplace", action="store_true")
+    ap.add_argument("--misalign", type=int, default=0, help="shift buffers by this many elements")
+    ap.add_argument("--mixed", action="store_true", help="shift only every other input (gather path)")
+    a = ap.parse_args(argv)
+    dev = Device(0)
+    {"reduce": run_reduce, "slices": run_slices, "pack": run_pack, "allreduce": run_allreduce}[a.what](dev, a)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

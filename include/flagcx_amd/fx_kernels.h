@@ -139,10 +139,6 @@ void fx_split(size_t total, size_t parts, size_t idx, size_t *cnt, size_t *off);
 size_t fx_nredslices(size_t count, int nranks, size_t nslices,
                      size_t nredslices, size_t redslicesize);
 
-/* Tuning knob for measurements: 0 = tiles in launch order, 1 = each XCD walks
- * a contiguous eighth of the buffer.  Returns the previous value. */
-int fx_set_xcd_spread(int mode);
-
 const char *fx_version(void);
 
 #ifdef __cplusplus

@@ -21,9 +21,9 @@ def run_reduce(dev, ins, dtype, op, first=0, inplace=False, offs=None):
     offs = offs or [0] * (len(ins) + 1)
     with DevBufs(dev) as b:
         dins = [b.put(a, pad_before=o) for a, o in zip(ins, offs[1:])]
-        dout = dins[0] if inplace else b.alloc(n * es + 256) + offs[0]
+        dout = dins[0] if inplace else b.alloc(offs[0] + n * es + 256) + offs[0]
         if not inplace:
-            dev.memset(dout - offs[0], 0xA5, n * es + 256)
+            dev.memset(dout - offs[0], 0xA5, offs[0] + n * es + 256)
         N.check(K.reduce_copy(dout, dins, n, dtype, op, first), "fx_reduce_copy")
         dev.sync()
         got = dev.to_host(dout, n, N.NP_DTYPE[dtype])
@@ -99,6 +99,31 @@ def test_unaligned_buffers(dev, dname):
                 want = O.reduce_copy(ins, dtype, op)
                 got = run_reduce(dev, ins, dtype, op, offs=offs)
                 assert_parity(got, want, dtype, op, f"{dname} n={n} offs={offs_el} op={op}")
+
+
+@pytest.mark.parametrize("dname", ["fp32", "bf16"])
+def test_striped_zone_boundaries(dev, dname):
+    """Segments a few MiB long handed out as striped regions plus a head and a
+    tail: output at odd byte offsets inside its allocation, lengths just around
+    whole numbers of 1 MiB regions, in place and out of place, k = 1, 2, 8."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    mib = (1 << 20) // es
+    for n, off_el in ((3 * mib, 0), (3 * mib + 1, 0), (2 * mib - 1, 5), (4 * mib + 4097, 131), (mib + 7, mib // 2 + 3),
+                      (5 * mib, 4)):
+        for k in (1, 2, 8):
+            ins = seeded_inputs(dtype, k, n, seed=n % 1000 + k)
+            want = O.reduce_copy(ins, dtype, N.OP_SUM)
+            offs = [off_el * es] * (k + 1)
+            got = run_reduce(dev, ins, dtype, N.OP_SUM, offs=offs)
+            assert_parity(got, want, dtype, N.OP_SUM, f"zone {dname} n={n} off={off_el} k={k}")
+            got = run_reduce(dev, ins, dtype, N.OP_SUM, offs=offs, inplace=True)
+            assert_parity(got, want, dtype, N.OP_SUM, f"zone in-place {dname} n={n} off={off_el} k={k}")
+    # inputs NOT co-aligned with the output: no zone, gather path over a long segment
+    n = 3 * mib + 9
+    ins = seeded_inputs(dtype, 3, n, seed=4)
+    got = run_reduce(dev, ins, dtype, N.OP_MAX, offs=[0, es, 0, 3 * es])
+    assert_parity(got, O.reduce_copy(ins, dtype, N.OP_MAX), dtype, N.OP_MAX, "long gather")
 
 
 def _special_f32():

@@ -49,8 +49,42 @@ flagcxResult_t sliceTiles(const fxSliceDesc &s, int k, int es, int U, uint64_t *
   return flagcxSuccess;
 }
 
+// Slices that continue each other in every input and in the output are one
+// longer slice (the operation is element-wise).  Partitions such as the
+// reference's slice / red-slice split produce long runs of them, and a long
+// segment gets the striped hand-out where 512 KiB pieces would not.
+std::vector<fxSliceDesc> mergeAdjacent(const fxSliceDesc *slices, size_t n, int k, size_t es) {
+  std::vector<fxSliceDesc> out;
+  out.reserve(n);
+  for (size_t i = 0; i < n; i++) {
+    const fxSliceDesc &d = slices[i];
+    if (d.count == 0) continue;
+    if (!out.empty()) {
+      fxSliceDesc &l = out.back();
+      const size_t bytes = l.count * es;
+      bool cont = (const char *)d.out == (const char *)l.out + bytes;
+      for (int p = 0; p < k && cont; p++) cont = (const char *)d.in[p] == (const char *)l.in[p] + bytes;
+      if (cont) {
+        l.count += d.count;
+        continue;
+      }
+    }
+    out.push_back(d);
+  }
+  return out;
+}
+
 // Launch n slices through kernel-argument tables of up to kInlineSlices each.
-flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slices, size_t n, int k, hipStream_t s) {
+flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slicesIn, size_t nIn, int k, hipStream_t s) {
+  for (size_t i = 0; i < nIn; i++)   // validate before merging so a bad slice is still reported
+    if (slicesIn[i].count) {
+      if (!slicesIn[i].out) return flagcxInvalidArgument;
+      for (int p = 0; p < k; p++)
+        if (!slicesIn[i].in[p]) return flagcxInvalidArgument;
+    }
+  const std::vector<fxSliceDesc> merged = mergeAdjacent(slicesIn, nIn, k, (size_t)ks->elemSize);
+  const fxSliceDesc *slices = merged.data();
+  const size_t n = merged.size();
   const int U = unrollFor(k);
   InlineSliceTable t;
   t.n = 0;
@@ -241,9 +275,16 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
   const int U = unrollFor(k);
   std::vector<SliceDescDev> desc;
   std::vector<uint32_t> start(1, 0u);
-  for (size_t i = 0; i < n; i++) {
-    fxSliceDesc s = slices[i];
-    s.count /= div;
+  std::vector<fxSliceDesc> scaled(slices, slices + n);
+  for (auto &d : scaled) {
+    if (d.count && !d.out) return flagcxInvalidArgument;
+    for (int p = 0; p < k; p++)
+      if (d.count && !d.in[p]) return flagcxInvalidArgument;
+    d.count /= div;
+  }
+  const std::vector<fxSliceDesc> merged = mergeAdjacent(scaled.data(), scaled.size(), k, (size_t)ks->elemSize);
+  for (size_t i = 0; i < merged.size(); i++) {
+    fxSliceDesc s = merged[i];
     uint64_t tiles;
     flagcxResult_t rc = sliceTiles(s, k, ks->elemSize, U, &tiles);
     if (rc != flagcxSuccess) return rc;

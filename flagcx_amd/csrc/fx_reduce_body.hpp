@@ -231,6 +231,12 @@ struct CopyRed {
 constexpr uint32_t kPieceVecs = 32;                           // 512 bytes
 constexpr uint32_t kStripeTiles = 64;                         // tiles per region
 constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;      // 32 KiB
+#ifndef FX_STRIPE_MIN_BYTES
+#define FX_STRIPE_MIN_BYTES (4ull << 20)
+#endif
+// Segments shorter than this (output bytes) stay contiguous: with few
+// workgroups in flight the striped hand-out only adds latency.
+constexpr uint64_t kStripeMinBytes = FX_STRIPE_MIN_BYTES;
 
 struct TilePlan {
   uint64_t nv;                 // vectors spanned by the segment
@@ -250,7 +256,7 @@ __host__ __device__ inline TilePlan planTiles(uint64_t outAddr, uint64_t count, 
   tp.endFull = end / ve;
   const uint64_t a0 = (outAddr - mis) >> 4;  // absolute vector number of vector 0
   uint64_t zs = (a0 + tp.firstFull + RV - 1) / RV * RV, ze = (a0 + tp.endFull) / RV * RV;
-  if (!coAligned || ze <= zs || count == 0) {
+  if (!coAligned || ze <= zs || count * (uint64_t)es < kStripeMinBytes) {
     tp.zs = tp.ze = 0;
   } else {
     tp.zs = zs - a0;
@@ -323,6 +329,28 @@ __device__ __forceinline__ void scatterElems(char *base, uint64_t e0, int lo, in
   }
 }
 
+// A whole 16-byte vector from an address that is only element-aligned: aligned
+// dword loads plus a funnel shift.  The dword holding the first (last) byte may
+// start before (end after) the vector, but never leaves the 4-byte word that
+// holds valid data, so it cannot touch an unmapped page.
+template <int ES>
+__device__ __forceinline__ u32x4 loadVectorUnaligned(const char *p) {
+  const uint32_t sh = (uint32_t)(uintptr_t)p & 3u;  // 0 when ES == 4
+  const uint32_t *q = reinterpret_cast<const uint32_t *>(p - sh);
+  u32x4 r;
+  if (ES == 4 || sh == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = __builtin_nontemporal_load(q + i);
+  } else {
+    uint32_t d[5];
+#pragma unroll
+    for (int i = 0; i < 5; i++) d[i] = __builtin_nontemporal_load(q + i);
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], sh);
+  }
+  return r;
+}
+
 // Reduce vector j of the segment with full bounds / alignment handling.
 template <class R, int K>
 __device__ __forceinline__ void reduceVectorChecked(const Seg<K> &sg, uint64_t j) {
@@ -332,12 +360,14 @@ __device__ __forceinline__ void reduceVectorChecked(const Seg<K> &sg, uint64_t j
   const int lo = (sg.lead > e0) ? (int)(sg.lead - e0) : 0;
   const int hi = (sg.end - e0 < (uint64_t)VE) ? (int)(sg.end - e0) : VE;
   const bool full = (lo == 0 && hi == VE);
-  const bool vec = full && sg.coAligned;
   typename R::Acc acc;
   const int k = sg.inputs();
-  R::init(acc, vec ? ldg_stream(sg.inp(0) + j * 16) : gatherElems<R::ES>(sg.inp(0), e0, lo, hi));
-  for (int p = 1; p < k; p++)
-    R::fold(acc, vec ? ldg_stream(sg.inp(p) + j * 16) : gatherElems<R::ES>(sg.inp(p), e0, lo, hi));
+  auto fetch = [&](int p) -> u32x4 {
+    if (!full) return gatherElems<R::ES>(sg.inp(p), e0, lo, hi);
+    return sg.coAligned ? ldg_stream(sg.inp(p) + j * 16) : loadVectorUnaligned<R::ES>(sg.inp(p) + j * 16);
+  };
+  R::init(acc, fetch(0));
+  for (int p = 1; p < k; p++) R::fold(acc, fetch(p));
   u32x4 r = R::finish(acc);
   if (full)
     stg_stream(sg.out + j * 16, r);

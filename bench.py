@@ -22,7 +22,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the same counter's reading for a
 # plain copy of known size; numbers and commands in
 # profiles/reduceCopyDirect_bf16_sum_k8_512MiB.txt.
-MEASURED_TRAFFIC_BYTES = 4_831_574_000
+MEASURED_TRAFFIC_BYTES = 4_831_515_000
 K_INPUTS = 8
 ELEMS = 268_435_456            # per input: 512 MiB of bf16
 SEED = 4                       # values N(0, 0.02)
@@ -149,7 +149,7 @@ def main():
                    "in_place_GBs": round(algo_bytes / (inplace_ms * 1e-3) / 1e9, 1)},
         "roofline": {"bound": "hbm", "achieved": round(kern_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kern_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "reduceCopyDirect<bf16,sum,K=8>", "bytes_per_launch": algo_bytes,
+                     "kernel": "reduceCopyDirect<Red<bf16,sum>,8,8>", "bytes_per_launch": algo_bytes,
                      "avg_launch_ms": round(kern_ms, 4)},
     }
     for p in ins + [out]:

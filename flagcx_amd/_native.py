@@ -86,6 +86,17 @@ _SIGS.update({
     "fxSimCommDestroyAll": (_i, [C.POINTER(_vp), _i]),
     "fxSimCommConfig": (_i, [_vp, _i, C.c_longlong]),
     "fxSimRegisterWindows": (_i, [_vp, C.POINTER(_vp), _sz]),
+    "fxSimCommInitRank": (_i, [C.POINTER(_vp), _i, _vp, _sz, _i]),
+    "fxSimCommDestroy": (_i, [_vp]),
+    "fxSimCommDevice": (_i, [_vp, C.POINTER(_i)]),
+    "flagcxGather": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
+    "flagcxScatter": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
+    "flagcxBroadcast": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
+    "flagcxAlltoAll": (_i, [_vp, _vp, _sz, _i, _vp, _vp]),
+    "flagcxSend": (_i, [_vp, _sz, _i, _i, _vp, _vp]),
+    "flagcxRecv": (_i, [_vp, _sz, _i, _i, _vp, _vp]),
+    "flagcxGroupStart": (_i, [_vp]),
+    "flagcxGroupEnd": (_i, [_vp]),
     "flagcxCommCount": (_i, [_vp, C.POINTER(_i)]),
     "flagcxCommUserRank": (_i, [_vp, C.POINTER(_i)]),
     "flagcxReduce": (_i, [_vp, _vp, _sz, _i, _i, _i, _vp, _vp]),

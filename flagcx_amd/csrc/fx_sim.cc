@@ -14,7 +14,9 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
+#include <string>
 #include <new>
 #include <vector>
 
@@ -27,7 +29,10 @@ struct flagcxStream {
 
 namespace {
 
-enum Kind { kNone = 0, kReduce, kAllReduce, kReduceScatter, kAllGather, kAlltoAllv, kCustomAllReduce };
+enum Kind {
+  kNone = 0, kReduce, kAllReduce, kReduceScatter, kAllGather, kAlltoAllv, kCustomAllReduce,
+  kGather, kScatter, kBroadcast, kAlltoAll
+};
 
 struct Post {
   bool posted = false;
@@ -37,10 +42,24 @@ struct Post {
   std::vector<size_t> sendcounts, sdispls, recvcounts, rdispls;
 };
 
+// One half of a point-to-point transfer waiting for its partner.
+struct PendingP2p {
+  bool isSend;
+  int src, dst;            // ranks
+  const void *sbuf;
+  void *rbuf;
+  size_t bytes;
+  hipStream_t stream;
+  hipEvent_t posted;       // recorded on `stream` when the call was made
+};
+
 struct Group {
   int n = 0;
   int device = 0;
   std::mutex mu;
+  std::string id;          // non-empty when created rank by rank (fxSimCommInitRank)
+  int joined = 0, alive = 0;
+  std::vector<PendingP2p> p2p;
   // pending collective
   Kind kind = kNone;
   size_t count = 0;
@@ -326,6 +345,66 @@ flagcxResult_t runAlltoAllv(const Ctx &c) {
   return R(fx_copy_slices(unpack.data(), unpack.size(), c.s));
 }
 
+// gather / scatter / broadcast / alltoall move bytes only: one batched copy
+// launch each (the reference builds them from grouped send/recv pairs,
+// flagcx/adaptor/ccl/rccl_adaptor.cc:126-184,222-246).
+flagcxResult_t runGather(const Ctx &c) {
+  const size_t bytes = c.g->count * c.ts;
+  std::vector<fxSliceDesc> d;
+  for (int r = 0; r < c.n && bytes; r++) {
+    void *dst = madd(c.recv(c.g->root), (size_t)r * bytes);
+    if (dst != c.send(r)) d.push_back(copyDesc(c.send(r), dst, bytes));
+  }
+  return R(fx_copy_slices(d.data(), d.size(), c.s));
+}
+
+flagcxResult_t runScatter(const Ctx &c) {
+  const size_t bytes = c.g->count * c.ts;
+  std::vector<fxSliceDesc> d;
+  for (int r = 0; r < c.n && bytes; r++) {
+    const void *src = cadd(c.send(c.g->root), (size_t)r * bytes);
+    if (src != c.recv(r)) d.push_back(copyDesc(src, c.recv(r), bytes));
+  }
+  return R(fx_copy_slices(d.data(), d.size(), c.s));
+}
+
+flagcxResult_t runBroadcast(const Ctx &c) {
+  const size_t bytes = c.g->count * c.ts;
+  std::vector<fxSliceDesc> d;
+  for (int r = 0; r < c.n && bytes; r++)
+    if (c.recv(r) != c.send(c.g->root)) d.push_back(copyDesc(c.send(c.g->root), c.recv(r), bytes));
+  return R(fx_copy_slices(d.data(), d.size(), c.s));
+}
+
+// Block i of rank r's sendbuff becomes block r of rank i's recvbuff.  If any
+// rank runs in place the blocks go through staging first.
+flagcxResult_t runAlltoAll(const Ctx &c) {
+  Group *g = c.g;
+  const int n = c.n;
+  const size_t bytes = g->count * c.ts;
+  if (bytes == 0) return flagcxSuccess;
+  bool inplace = false;
+  for (int r = 0; r < n; r++) inplace = inplace || (c.send(r) == c.recv(r));
+  std::vector<fxSliceDesc> d;
+  if (!inplace) {
+    for (int r = 0; r < n; r++)
+      for (int i = 0; i < n; i++)
+        d.push_back(copyDesc(cadd(c.send(r), (size_t)i * bytes), madd(c.recv(i), (size_t)r * bytes), bytes));
+    return R(fx_copy_slices(d.data(), d.size(), c.s));
+  }
+  flagcxResult_t rc = ensureScratch(g, (size_t)n * n * bytes);
+  if (rc != flagcxSuccess) return rc;
+  for (int r = 0; r < n; r++)
+    d.push_back(copyDesc(c.send(r), madd(g->scratch, (size_t)r * n * bytes), (size_t)n * bytes));
+  rc = R(fx_copy_slices(d.data(), d.size(), c.s));
+  if (rc != flagcxSuccess) return rc;
+  d.clear();
+  for (int r = 0; r < n; r++)
+    for (int i = 0; i < n; i++)
+      d.push_back(copyDesc(cadd(g->scratch, ((size_t)r * n + i) * bytes), madd(c.recv(i), (size_t)r * bytes), bytes));
+  return R(fx_copy_slices(d.data(), d.size(), c.s));
+}
+
 flagcxResult_t runCustomAllReduce(const Ctx &c) {
   Group *g = c.g;
   if (g->count == 0) return flagcxSuccess;
@@ -418,6 +497,10 @@ flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, v
       case kAllGather: res = runAllGather(c); break;
       case kAlltoAllv: res = runAlltoAllv(c); break;
       case kCustomAllReduce: res = runCustomAllReduce(c); break;
+      case kGather: res = runGather(c); break;
+      case kScatter: res = runScatter(c); break;
+      case kBroadcast: res = runBroadcast(c); break;
+      case kAlltoAll: res = runAlltoAll(c); break;
       default: res = flagcxInternalError;
     }
   }
@@ -445,6 +528,87 @@ flagcxResult_t screenReduce(int dtype, int op) {
   return flagcxSuccess;
 }
 
+std::mutex gRegistryMu;
+std::map<std::string, Group *> gRegistry;  // groups still waiting for ranks to join, by id
+
+flagcxResult_t newGroup(int nranks, Group **out) {
+  Group *g = new (std::nothrow) Group();
+  if (!g) return flagcxSystemError;
+  g->n = nranks;
+  g->posts.resize(nranks);
+  g->ready.assign(nranks, nullptr);
+  bool ok = hipGetDevice(&g->device) == hipSuccess;
+  ok = ok && hipEventCreateWithFlags(&g->done, hipEventDisableTiming) == hipSuccess;
+  for (int r = 0; r < nranks && ok; r++)
+    ok = hipEventCreateWithFlags(&g->ready[r], hipEventDisableTiming) == hipSuccess;
+  if (!ok) {
+    for (auto e : g->ready)
+      if (e) (void)hipEventDestroy(e);
+    if (g->done) (void)hipEventDestroy(g->done);
+    delete g;
+    return flagcxUnhandledDeviceError;
+  }
+  // same knobs, same names, same defaults as the reference's uniRunner
+  g->nslices = envParam("FLAGCX_UNIRUNNER_NSLICES", 1);
+  g->nredslices = envParam("FLAGCX_UNIRUNNER_NREDSLICES", 0);
+  g->redslicesize = envParam("FLAGCX_UNIRUNNER_REDSLICESIZE", 65536);
+  if (g->nslices < 1) g->nslices = 1;
+  if (g->nredslices < 0) g->nredslices = 0;
+  if (g->redslicesize < 0) g->redslicesize = 0;
+  *out = g;
+  return flagcxSuccess;
+}
+
+void freeGroup(Group *g) {
+  (void)hipDeviceSynchronize();
+  for (auto e : g->ready) (void)hipEventDestroy(e);
+  (void)hipEventDestroy(g->done);
+  for (auto &p : g->p2p) (void)hipEventDestroy(p.posted);
+  if (g->scratch) (void)hipFree(g->scratch);
+  delete g;
+}
+
+// send / recv between simulated ranks: the later of the two calls performs the
+// copy on its own stream after waiting for the other side's stream, and the
+// other side's stream then waits for the copy.
+flagcxResult_t postP2p(flagcxComm_t comm, bool isSend, const void *sbuf, void *rbuf, size_t count, int dtype, int peer,
+                       flagcxStream_t stream) {
+  if (!comm || !comm->g || !stream) return flagcxInvalidArgument;
+  Group *g = comm->g;
+  const size_t ts = fx_dtype_size(dtype);
+  if (ts == 0 || peer < 0 || peer >= g->n) return flagcxInvalidArgument;
+  if (count && !(isSend ? sbuf : (const void *)rbuf)) return flagcxInvalidArgument;
+  const int src = isSend ? comm->rank : peer, dst = isSend ? peer : comm->rank;
+  const size_t bytes = count * ts;
+  std::lock_guard<std::mutex> lock(g->mu);
+  for (size_t i = 0; i < g->p2p.size(); i++) {
+    PendingP2p &o = g->p2p[i];
+    if (o.isSend == isSend || o.src != src || o.dst != dst) continue;
+    flagcxResult_t res = flagcxSuccess;
+    if (o.bytes != bytes) {
+      res = flagcxInvalidArgument;  // the two sides disagree on the message size
+    } else if (bytes) {
+      hipStream_t s = stream->base;
+      fxSliceDesc d = copyDesc(isSend ? sbuf : o.sbuf, isSend ? o.rbuf : rbuf, bytes);
+      if (o.stream != s && hipStreamWaitEvent(s, o.posted, 0) != hipSuccess) res = flagcxUnhandledDeviceError;
+      if (res == flagcxSuccess) res = R(fx_copy_slices(&d, 1, s));
+      if (res == flagcxSuccess && o.stream != s) {
+        if (hipEventRecord(o.posted, s) != hipSuccess || hipStreamWaitEvent(o.stream, o.posted, 0) != hipSuccess)
+          res = flagcxUnhandledDeviceError;
+      }
+    }
+    (void)hipEventDestroy(o.posted);
+    g->p2p.erase(g->p2p.begin() + (long)i);
+    return res;
+  }
+  PendingP2p p{isSend, src, dst, sbuf, rbuf, bytes, stream->base, nullptr};
+  if (hipEventCreateWithFlags(&p.posted, hipEventDisableTiming) != hipSuccess ||
+      hipEventRecord(p.posted, p.stream) != hipSuccess)
+    return flagcxUnhandledDeviceError;
+  g->p2p.push_back(p);
+  return flagcxSuccess;
+}
+
 void partNode(fxRedNode *n, int step, int rank, size_t slice, int in1, int in2, int out, size_t inOff, size_t outOff,
               size_t cnt) {
   n->step = step;
@@ -465,35 +629,11 @@ extern "C" {
 
 flagcxResult_t fxSimCommInitAll(flagcxComm_t *comms, int nranks) {
   if (!comms || nranks < 1 || nranks > FX_MAX_INPUTS) return flagcxInvalidArgument;
-  Group *g = new (std::nothrow) Group();
-  if (!g) return flagcxSystemError;
-  g->n = nranks;
-  g->posts.resize(nranks);
-  g->ready.assign(nranks, nullptr);
-  if (hipGetDevice(&g->device) != hipSuccess) {
-    delete g;
-    return flagcxUnhandledDeviceError;
-  }
-  bool ok = hipEventCreateWithFlags(&g->done, hipEventDisableTiming) == hipSuccess;
-  for (int r = 0; r < nranks && ok; r++)
-    ok = hipEventCreateWithFlags(&g->ready[r], hipEventDisableTiming) == hipSuccess;
-  if (!ok) {
-    for (auto e : g->ready)
-      if (e) (void)hipEventDestroy(e);
-    if (g->done) (void)hipEventDestroy(g->done);
-    delete g;
-    return flagcxUnhandledDeviceError;
-  }
-  g->nslices = envParam("FLAGCX_UNIRUNNER_NSLICES", 1);
-  g->nredslices = envParam("FLAGCX_UNIRUNNER_NREDSLICES", 0);
-  g->redslicesize = envParam("FLAGCX_UNIRUNNER_REDSLICESIZE", 65536);
-  if (g->nslices < 1) g->nslices = 1;
-  if (g->nredslices < 0) g->nredslices = 0;
-  if (g->redslicesize < 0) g->redslicesize = 0;
-  for (int r = 0; r < nranks; r++) {
-    comms[r] = new (std::nothrow) flagcxComm{g, r};
-    if (!comms[r]) return flagcxSystemError;
-  }
+  Group *g = nullptr;
+  flagcxResult_t rc = newGroup(nranks, &g);
+  if (rc != flagcxSuccess) return rc;
+  g->joined = g->alive = nranks;
+  for (int r = 0; r < nranks; r++) comms[r] = new flagcxComm{g, r};
   return flagcxSuccess;
 }
 
@@ -501,15 +641,51 @@ flagcxResult_t fxSimCommDestroyAll(flagcxComm_t *comms, int nranks) {
   if (!comms || nranks < 1 || !comms[0]) return flagcxInvalidArgument;
   Group *g = comms[0]->g;
   if (g->n != nranks) return flagcxInvalidArgument;
-  (void)hipDeviceSynchronize();
-  for (auto e : g->ready) (void)hipEventDestroy(e);
-  (void)hipEventDestroy(g->done);
-  if (g->scratch) (void)hipFree(g->scratch);
-  delete g;
   for (int r = 0; r < nranks; r++) {
     delete comms[r];
     comms[r] = nullptr;
   }
+  freeGroup(g);
+  return flagcxSuccess;
+}
+
+flagcxResult_t fxSimCommInitRank(flagcxComm_t *comm, int nranks, const void *id, size_t idBytes, int rank) {
+  if (!comm || !id || idBytes == 0 || nranks < 1 || nranks > FX_MAX_INPUTS || rank < 0 || rank >= nranks)
+    return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(gRegistryMu);
+  const std::string key((const char *)id, idBytes);
+  Group *g;
+  auto it = gRegistry.find(key);
+  if (it == gRegistry.end()) {
+    flagcxResult_t rc = newGroup(nranks, &g);
+    if (rc != flagcxSuccess) return rc;
+    g->id = key;
+    gRegistry[key] = g;
+  } else {
+    g = it->second;
+    if (g->n != nranks) return flagcxInvalidArgument;
+  }
+  g->joined++;
+  g->alive++;
+  if (g->joined == nranks) gRegistry.erase(key);  // complete: the id may be reused for a new group
+  *comm = new flagcxComm{g, rank};
+  return flagcxSuccess;
+}
+
+flagcxResult_t fxSimCommDestroy(flagcxComm_t comm) {
+  if (!comm || !comm->g) return flagcxInvalidArgument;
+  Group *g = comm->g;
+  bool last;
+  {
+    std::lock_guard<std::mutex> lock(gRegistryMu);
+    last = (--g->alive == 0);
+    if (last && !g->id.empty()) {
+      auto it = gRegistry.find(g->id);
+      if (it != gRegistry.end() && it->second == g) gRegistry.erase(it);
+    }
+  }
+  delete comm;
+  if (last) freeGroup(g);
   return flagcxSuccess;
 }
 
@@ -595,6 +771,58 @@ flagcxResult_t flagcxAlltoAllv(const void *sendbuff, size_t *sendcounts, size_t 
   if (!sendcounts || !sdispls || !recvcounts || !rdispls) return flagcxInvalidArgument;
   return postAndMaybeRun(comm, kAlltoAllv, sendbuff, recvbuff, 0, datatype, 0, 0, stream, sendcounts, sdispls,
                          recvcounts, rdispls);
+}
+
+flagcxResult_t flagcxGather(const void *sendbuff, void *recvbuff, size_t count, flagcxDataType_t datatype, int root,
+                            flagcxComm_t comm, flagcxStream_t stream) {
+  if (fx_dtype_size(datatype) == 0) return flagcxInvalidArgument;
+  if (!comm || root < 0 || root >= comm->g->n) return flagcxInvalidArgument;
+  if (count && (!sendbuff || (comm->rank == root && !recvbuff))) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kGather, sendbuff, recvbuff, count, datatype, 0, root, stream);
+}
+
+flagcxResult_t flagcxScatter(const void *sendbuff, void *recvbuff, size_t count, flagcxDataType_t datatype, int root,
+                             flagcxComm_t comm, flagcxStream_t stream) {
+  if (fx_dtype_size(datatype) == 0) return flagcxInvalidArgument;
+  if (!comm || root < 0 || root >= comm->g->n) return flagcxInvalidArgument;
+  if (count && (!recvbuff || (comm->rank == root && !sendbuff))) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kScatter, sendbuff, recvbuff, count, datatype, 0, root, stream);
+}
+
+flagcxResult_t flagcxBroadcast(const void *sendbuff, void *recvbuff, size_t count, flagcxDataType_t datatype,
+                               int root, flagcxComm_t comm, flagcxStream_t stream) {
+  if (fx_dtype_size(datatype) == 0) return flagcxInvalidArgument;
+  if (!comm || root < 0 || root >= comm->g->n) return flagcxInvalidArgument;
+  if (count && (!recvbuff || (comm->rank == root && !sendbuff))) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kBroadcast, sendbuff, recvbuff, count, datatype, 0, root, stream);
+}
+
+flagcxResult_t flagcxAlltoAll(const void *sendbuff, void *recvbuff, size_t count, flagcxDataType_t datatype,
+                              flagcxComm_t comm, flagcxStream_t stream) {
+  if (fx_dtype_size(datatype) == 0) return flagcxInvalidArgument;
+  if (count && (!sendbuff || !recvbuff)) return flagcxInvalidArgument;
+  return postAndMaybeRun(comm, kAlltoAll, sendbuff, recvbuff, count, datatype, 0, 0, stream);
+}
+
+flagcxResult_t flagcxSend(const void *sendbuff, size_t count, flagcxDataType_t datatype, int peer, flagcxComm_t comm,
+                          flagcxStream_t stream) {
+  return postP2p(comm, true, sendbuff, nullptr, count, datatype, peer, stream);
+}
+
+flagcxResult_t flagcxRecv(void *recvbuff, size_t count, flagcxDataType_t datatype, int peer, flagcxComm_t comm,
+                          flagcxStream_t stream) {
+  return postP2p(comm, false, nullptr, recvbuff, count, datatype, peer, stream);
+}
+
+// Calls are asynchronous and matched across ranks as they arrive, so a group
+// bracket has nothing to defer.
+flagcxResult_t flagcxGroupStart(flagcxComm_t) { return flagcxSuccess; }
+flagcxResult_t flagcxGroupEnd(flagcxComm_t) { return flagcxSuccess; }
+
+flagcxResult_t fxSimCommDevice(const flagcxComm_t comm, int *device) {
+  if (!comm || !device) return flagcxInvalidArgument;
+  *device = comm->g->device;
+  return flagcxSuccess;
 }
 
 flagcxResult_t fxSimRegisterWindows(flagcxComm_t comm, void *const *windows, size_t bytes) {

@@ -58,7 +58,7 @@ def run_reduce(dev, a):
     dtype, op, k = DT[a.dtype], OP[a.op], a.k
     es = N.DTYPE_SIZE[dtype]
     emax = size(a.max)
-    ins = [dev.malloc(emax + a.misalign * es) for _ in range(k)]
+    ins = [dev.malloc(emax + a.misalign * es + a.in_shift * k) + a.in_shift * i for i in range(k)]
     for i, p in enumerate(ins):
         dev.memset(p, 0x3c + i, emax)
     out = ins[0] if a.inplace else dev.malloc(emax + a.misalign * es)
@@ -173,6 +173,8 @@ def main(argv=None):
     ap.add_argument("--inplace", action="store_true")
     ap.add_argument("--misalign", type=int, default=0, help="shift buffers by this many elements")
     ap.add_argument("--mixed", action="store_true", help="shift only every other input (gather path)")
+    ap.add_argument("--in-shift", type=int, default=0,
+                    help="start input i at byte offset i*IN_SHIFT of its allocation (multiple of 16 keeps vector loads)")
     a = ap.parse_args(argv)
     dev = Device(0)
     {"reduce": run_reduce, "slices": run_slices, "pack": run_pack, "allreduce": run_allreduce}[a.what](dev, a)

@@ -33,6 +33,15 @@ extern "C" {
 flagcxResult_t fxSimCommInitAll(flagcxComm_t *comms, int nranks);
 flagcxResult_t fxSimCommDestroyAll(flagcxComm_t *comms, int nranks);
 
+/* The same group built rank by rank, the way flagcxCommInitRank
+ * (flagcx/include/flagcx.h:296-297) is called: every rank passes the same id
+ * bytes; the group is complete when nranks ranks have joined.  Each
+ * communicator is released with fxSimCommDestroy; the last one frees the group. */
+flagcxResult_t fxSimCommInitRank(flagcxComm_t *comm, int nranks, const void *id,
+                                 size_t idBytes, int rank);
+flagcxResult_t fxSimCommDestroy(flagcxComm_t comm);
+flagcxResult_t fxSimCommDevice(const flagcxComm_t comm, int *device);
+
 /* Configuration keys (defaults come from the same environment variables the
  * reference reads, flagcx/runner/uni_runner_impl.cc:21-26, uni_runner.cc:10-12). */
 enum {
@@ -74,6 +83,31 @@ flagcxResult_t flagcxAlltoAllv(const void *sendbuff, size_t *sendcounts,
                                size_t *recvcounts, size_t *rdispls,
                                flagcxDataType_t datatype, flagcxComm_t comm,
                                flagcxStream_t stream);
+
+/* Byte-moving collectives and point-to-point calls, signatures of
+ * flagcx.h:385-415,468-470,498-516,653-662.  On one GPU they are batched
+ * copies; send/recv pairs are matched as they arrive. */
+flagcxResult_t flagcxGather(const void *sendbuff, void *recvbuff, size_t count,
+                            flagcxDataType_t datatype, int root,
+                            flagcxComm_t comm, flagcxStream_t stream);
+flagcxResult_t flagcxScatter(const void *sendbuff, void *recvbuff, size_t count,
+                             flagcxDataType_t datatype, int root,
+                             flagcxComm_t comm, flagcxStream_t stream);
+flagcxResult_t flagcxBroadcast(const void *sendbuff, void *recvbuff,
+                               size_t count, flagcxDataType_t datatype,
+                               int root, flagcxComm_t comm,
+                               flagcxStream_t stream);
+flagcxResult_t flagcxAlltoAll(const void *sendbuff, void *recvbuff,
+                              size_t count, flagcxDataType_t datatype,
+                              flagcxComm_t comm, flagcxStream_t stream);
+flagcxResult_t flagcxSend(const void *sendbuff, size_t count,
+                          flagcxDataType_t datatype, int peer,
+                          flagcxComm_t comm, flagcxStream_t stream);
+flagcxResult_t flagcxRecv(void *recvbuff, size_t count,
+                          flagcxDataType_t datatype, int peer,
+                          flagcxComm_t comm, flagcxStream_t stream);
+flagcxResult_t flagcxGroupStart(flagcxComm_t comm);
+flagcxResult_t flagcxGroupEnd(flagcxComm_t comm);
 
 /*
  * Custom allreduce hook: this rank's result = k-way reduce over all ranks'

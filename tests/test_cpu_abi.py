@@ -55,6 +55,26 @@ def test_plugin_passes_the_reference_loader_checks():
     assert syms == ["flagcxDeviceAdaptorPlugin_v1"]
 
 
+def test_ccl_plugin_passes_the_reference_loader_checks():
+    from flagcx_amd import ccl_adaptor
+    t = ccl_adaptor.load_plugin()
+    assert t.name == b"MI355X-SIM"
+    # name pointer + 34 function pointers (flagcx_ccl_adaptor.h:42-122), all required (ccl_plugin_load.cc:64-81)
+    assert C.sizeof(ccl_adaptor.CCLAdaptorV1) == 35 * C.sizeof(C.c_void_p)
+    assert len(ccl_adaptor._FIELDS) == 34
+    out = os.popen(f"nm -D --defined-only {ccl_adaptor.CCL_PLUGIN_LIB}").read()
+    syms = [l.split()[-1] for l in out.splitlines() if " D " in l or " T " in l or " B " in l]
+    assert syms == ["flagcxCCLAdaptorPlugin_v1"]          # nothing that could clash with libflagcx.so
+    v = C.c_int()
+    assert t.getVersion(C.byref(v)) == N.SUCCESS and t.getVersion(None) == N.INVALID_ARGUMENT
+    assert t.getErrorString(9) == b"not supported"
+    assert t.commCount(None, C.byref(v)) == N.INVALID_ARGUMENT
+    assert t.commDestroy(None) == N.INVALID_ARGUMENT
+    assert t.allReduce(0x1000, 0x1000, 4, N.DT_FP32, N.OP_SUM, None, None) == N.INVALID_ARGUMENT
+    with pytest.raises(ImportError):
+        ccl_adaptor.load_plugin(N.KERNEL_LIB)
+
+
 def test_loader_rejects_bad_plugins(tmp_path):
     with pytest.raises(ImportError):
         adaptor.load_plugin(str(tmp_path / "nope.so"))

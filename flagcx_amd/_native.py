@@ -67,6 +67,16 @@ _SIGS = {
     "fx_plan_destroy": (_i, [_vp]),
     "fx_pack": (_i, [_vp, _vp, C.POINTER(_sz), C.POINTER(_sz), _i, _i, _vp]),
     "fx_unpack": (_i, [_vp, _vp, C.POINTER(_sz), C.POINTER(_sz), _i, _i, _vp]),
+    "fx_fifo_bytes": (_sz, [_sz]),
+    "fx_fifo_init": (_i, [_vp, _sz]),
+    "fx_fifo_enqueue": (_i, [_vp, C.c_uint64, C.c_uint64, C.c_uint64, _sz, _sz, _i, _i, C.POINTER(_i)]),
+    "fx_fifo_poll_state": (_i, [_vp, _i]),
+    "fx_fifo_set_state": (_i, [_vp, _i, _i]),
+    "fx_fifo_terminate": (_i, [_vp]),
+    "fx_fifo_consumer_create": (_i, [C.POINTER(_vp), _sz]),
+    "fx_fifo_consumer_launch": (_i, [_vp, _vp, _vp, C.c_ulonglong, _vp]),
+    "fx_fifo_consumer_status": (_i, [_vp, C.POINTER(_i), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "fx_fifo_consumer_destroy": (_i, [_vp]),
     "fx_dtype_size": (_sz, [_i]),
     "fx_split": (None, [_sz, _sz, _sz, C.POINTER(_sz), C.POINTER(_sz)]),
     "fx_nredslices": (_sz, [_sz, _i, _sz, _sz, _sz]),

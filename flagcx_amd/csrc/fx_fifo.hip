@@ -1,0 +1,314 @@
+// Reduce-FIFO compatibility mode: a persistent gfx950 kernel that consumes
+// FlagCX's reduce-trigger ring unmodified, plus the host side of that ring.
+//
+// Ring layout and protocol are the reference's
+// (flagcx/include/flagcx_kernel_core.h:44-67,146-162,209-230;
+// flagcx/core/flagcx_reduce_kernel_host.cc:6-98; consumer
+// flagcx/adaptor/kernel/nvidia/flagcx_reduce_kernel_device.cu:53-186):
+//   uint64 words [0] capacity [1] consumed [2] produced [3] terminate, then
+//   `capacity` 32-byte triggers; the producer writes a trigger with state
+//   Enqueued and bumps `produced`; the consumer executes it and ORs state
+//   Complete into value[3]; the producer polls for Complete and resets the slot
+//   to Available; `terminate` = 1 ends the consumer once the ring is drained.
+//
+// What differs from the reference's consumer (one block of 32 threads that
+// dequeues with a CAS and runs the reduce itself): here EVERY workgroup of a
+// full-width grid works on every trigger -- workgroup w takes tiles w, w+G, ...
+// of it -- and the last workgroup to finish marks it Complete.  Workgroup 0
+// alone reads the pinned host ring (over PCIe) and mirrors it into device
+// memory, where the other workgroups poll it.  Nothing waits on another
+// workgroup, so the kernel cannot deadlock on residency; every polling loop is
+// bounded by maxIdlePolls.  Triggers that are in the ring at the same time must
+// be independent of each other, which is how the reference's scheduler uses it
+// (a node is enqueued only after its parents completed,
+// flagcx/runner/uni_runner_impl.cc:1727-1794).
+#include <sched.h>
+
+#include <cstddef>
+#include <cstring>
+#include <new>
+
+#include "flagcx_amd/fx_kernels.h"
+#include "fx_launch.hpp"
+
+using namespace fx;
+
+namespace {
+
+constexpr int kFifoU = 4;
+constexpr uint32_t kMaxCapacity = 1024;
+
+struct FifoMirror {              // device memory, zeroed at creation
+  uint64_t produced;             // triggers mirrored so far (written by workgroup 0)
+  uint64_t terminate;
+  uint64_t completed;            // triggers fully executed
+  uint64_t exitReason;           // FX_FIFO_EXIT_*
+  uint64_t badTriggers;          // triggers skipped because dtype / op is not carried
+  uint64_t pad[3];
+  uint32_t done[kMaxCapacity];   // per slot: workgroups that finished their share
+  uint64_t trig[kMaxCapacity][4];
+};
+
+// Polling uses relaxed atomics (they bypass the non-coherent cache levels on
+// their own); the acquire / release fences are paid only when something changed.
+template <class T>
+__device__ __forceinline__ T pollSys(const T *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+template <class T>
+__device__ __forceinline__ T pollDev(const T *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <class T>
+__device__ __forceinline__ void storeDev(T *p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <class T>
+__device__ __forceinline__ void storeSys(T *p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// This workgroup's share of one two-input trigger.
+template <int DT, int OP>
+__device__ __forceinline__ void runShare(const void *in1, const void *in2, void *out, uint64_t count) {
+  using R = Red<DT, OP>;
+  const void *in[2] = {in1, in2};
+  Seg<2> sg;
+  const TilePlan tp = makeSeg<R::ES, kFifoU>(sg, in, out, count, 2);
+  const uint64_t tiles = tp.tiles();
+  for (uint64_t t = blockIdx.x; t < tiles; t += gridDim.x) reduceTile<R, 2, kFifoU>(sg, tp, (uint32_t)t);
+}
+
+template <int DT>
+__device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b, void *o, uint64_t n) {
+  switch (op) {
+    case flagcxSum: runShare<DT, flagcxSum>(a, b, o, n); return true;
+    case flagcxProd: runShare<DT, flagcxProd>(a, b, o, n); return true;
+    case flagcxMax: runShare<DT, flagcxMax>(a, b, o, n); return true;
+    case flagcxMin: runShare<DT, flagcxMin>(a, b, o, n); return true;
+    default: return false;
+  }
+}
+
+__global__ void __launch_bounds__(kBlock)
+fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uint64_t maxIdlePolls) {
+  __shared__ uint64_t sh[6];  // [0] state, [1..4] trigger words, [5] scratch
+  enum { kWork = 0, kExitTerminate = FX_FIFO_EXIT_TERMINATE, kExitIdle = FX_FIFO_EXIT_IDLE };
+  uint64_t seq = startSeq;
+  uint64_t *hostTrig = host + 4;
+  uint64_t mirrored = startSeq;      // workgroup 0: triggers copied to the mirror so far
+  uint64_t lastPublished = ~0ull;    // workgroup 0: last `completed` written to the host's `consumed`
+  bool hostTermSeen = false;
+  for (;;) {
+    if (threadIdx.x == 0) {
+      uint64_t idle = 0, state;
+      bool termSeen = false;
+      for (;;) {
+        if (blockIdx.x == 0) {
+          const uint64_t hp = pollSys(host + 2), ht = pollSys(host + 3);
+          if (mirrored < hp) {
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // the triggers behind `produced`
+            for (; mirrored < hp; mirrored++) {
+              const uint32_t slot = (uint32_t)(mirrored % cap);
+              for (int w = 0; w < 4; w++) m->trig[slot][w] = pollSys(hostTrig + 4 * slot + w);
+            }
+            storeDev(&m->produced, hp);  // release: the mirrored triggers are visible first
+          }
+          // The host sets terminate after its last enqueue, but two relaxed
+          // polls may be served out of order: act on terminate only on the poll
+          // AFTER the one that first saw it, when `produced` has been re-read.
+          if (ht) {
+            if (hostTermSeen) storeDev(&m->terminate, ht);
+            hostTermSeen = true;
+          }
+          const uint64_t c = pollDev(&m->completed);
+          if (c != lastPublished) {
+            storeSys(host + 1, startSeq + c);  // consumed
+            lastPublished = c;
+          }
+        }
+        const uint64_t term = pollDev(&m->terminate), p = pollDev(&m->produced);
+        if (p > seq) { state = kWork; break; }
+        if (term) {
+          if (termSeen) { state = kExitTerminate; break; }  // same two-step rule as above
+          termSeen = true;
+          continue;
+        }
+        if (++idle > maxIdlePolls) { state = kExitIdle; break; }
+        __builtin_amdgcn_s_sleep(32);
+      }
+      sh[0] = state;
+      if (state == kWork) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const uint32_t slot = (uint32_t)(seq % cap);
+        for (int w = 0; w < 4; w++) sh[1 + w] = m->trig[slot][w];
+      }
+    }
+    __syncthreads();
+    const uint64_t state = sh[0];
+    if (state != kWork) {
+      if (threadIdx.x == 0 && blockIdx.x == 0) {
+        storeSys(host + 1, startSeq + pollDev(&m->completed));
+        storeDev(&m->exitReason, state);
+      }
+      break;
+    }
+    // The trigger's buffers may have been written by other agents since this
+    // kernel last looked: drop stale cache lines before reading them.
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    const void *in1 = (const void *)(uintptr_t)sh[1], *in2 = (const void *)(uintptr_t)sh[2];
+    void *out = (void *)(uintptr_t)sh[3];
+    const uint64_t w3 = sh[4];
+    const uint64_t count = w3 & 0xffffffffull;
+    const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
+    bool ok = true;
+    if (count) {
+      switch (dtype) {
+        case flagcxFloat32: ok = runShareOp<flagcxFloat32>(op, in1, in2, out, count); break;
+        case flagcxInt32: ok = runShareOp<flagcxInt32>(op, in1, in2, out, count); break;
+        case flagcxBfloat16: ok = runShareOp<flagcxBfloat16>(op, in1, in2, out, count); break;
+        case flagcxFloat16: ok = runShareOp<flagcxFloat16>(op, in1, in2, out, count); break;
+        default: ok = false;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const uint32_t slot = (uint32_t)(seq % cap);
+      __threadfence();  // this workgroup's stores are out before it reports in
+      const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      if (prev == gridDim.x - 1) {  // last one out completes the trigger
+        __hip_atomic_store(&m->done[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!ok) __hip_atomic_fetch_add(&m->badTriggers, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence_system();
+        storeSys(hostTrig + 4 * slot + 3, w3 | ((uint64_t)fxTriggerComplete << 56));
+        __hip_atomic_fetch_add(&m->completed, 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    seq++;
+    __syncthreads();
+  }
+}
+
+}  // namespace
+
+struct fxFifoConsumer {
+  FifoMirror *mirror;
+  uint32_t capacity;
+  uint32_t grid;
+};
+
+extern "C" {
+#pragma GCC visibility push(default)
+
+// ---- host side of the ring (flagcx/core/flagcx_reduce_kernel_host.cc) ----
+
+size_t fx_fifo_bytes(size_t capacity) { return (4 + 4 * capacity) * sizeof(uint64_t); }
+
+int fx_fifo_init(uint64_t *fifo, size_t capacity) {
+  if (!fifo || capacity == 0 || capacity > kMaxCapacity) return flagcxInvalidArgument;
+  fifo[0] = capacity;
+  fifo[1] = fifo[2] = fifo[3] = 0;
+  memset(fifo + 4, 0, capacity * sizeof(fxReduceTrigger));
+  __sync_synchronize();
+  return flagcxSuccess;
+}
+
+int fx_fifo_enqueue(uint64_t *fifo, uint64_t in1, uint64_t in2, uint64_t out, size_t count, size_t nthreads,
+                    int dtype, int op, int *idx) {
+  if (!fifo || !idx) return flagcxInvalidArgument;
+  *idx = -1;
+  const uint64_t cap = fifo[0];
+  const uint64_t produced = fifo[2], consumed = __atomic_load_n(&fifo[1], __ATOMIC_ACQUIRE);
+  if (produced - consumed >= cap) {  // ring full: the caller retries
+    sched_yield();
+    return flagcxSuccess;
+  }
+  const uint64_t slot = produced % cap;
+  fxReduceTrigger *t = reinterpret_cast<fxReduceTrigger *>(fifo + 4) + slot;
+  const uint64_t state = (__atomic_load_n(&t->value[3], __ATOMIC_ACQUIRE) >> 56) & 0x3;
+  if (state != fxTriggerAvailable) {  // slot not collected yet
+    sched_yield();
+    return flagcxSuccess;
+  }
+  fxReduceTrigger v;
+  fx_trigger_set(&v, in1, in2, out, count, nthreads, dtype, op, fxTriggerEnqueued);
+  memcpy(t, &v, sizeof(v));
+  __atomic_fetch_add(&fifo[2], 1ull, __ATOMIC_RELEASE);
+  *idx = (int)slot;
+  return flagcxSuccess;
+}
+
+int fx_fifo_poll_state(const uint64_t *fifo, int idx) {
+  if (!fifo || idx < 0 || (uint64_t)idx >= fifo[0]) return -1;
+  const fxReduceTrigger *t = reinterpret_cast<const fxReduceTrigger *>(fifo + 4) + idx;
+  return (int)((__atomic_load_n(&t->value[3], __ATOMIC_ACQUIRE) >> 56) & 0x3);
+}
+
+int fx_fifo_set_state(uint64_t *fifo, int idx, int state) {
+  if (!fifo || idx < 0 || (uint64_t)idx >= fifo[0]) return flagcxInvalidArgument;
+  fxReduceTrigger *t = reinterpret_cast<fxReduceTrigger *>(fifo + 4) + idx;
+  uint64_t v = __atomic_load_n(&t->value[3], __ATOMIC_ACQUIRE);
+  v = (v & ~(0x3ull << 56)) | (((uint64_t)state & 0x3) << 56);
+  __atomic_store_n(&t->value[3], v, __ATOMIC_RELEASE);
+  return flagcxSuccess;
+}
+
+int fx_fifo_terminate(uint64_t *fifo) {
+  if (!fifo) return flagcxInvalidArgument;
+  __atomic_store_n(&fifo[3], 1ull, __ATOMIC_RELEASE);
+  return flagcxSuccess;
+}
+
+// ---- device side ----
+
+int fx_fifo_consumer_create(fxFifoConsumer_t *consumer, size_t capacity) {
+  if (!consumer || capacity == 0 || capacity > kMaxCapacity) return flagcxInvalidArgument;
+  *consumer = nullptr;
+  fxFifoConsumer *c = new (std::nothrow) fxFifoConsumer();
+  if (!c) return flagcxSystemError;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      hipMalloc((void **)&c->mirror, sizeof(FifoMirror)) != hipSuccess) {
+    delete c;
+    return flagcxUnhandledDeviceError;
+  }
+  c->capacity = (uint32_t)capacity;
+  c->grid = (uint32_t)(cus > 0 ? cus : 1);  // one resident workgroup per CU
+  *consumer = c;
+  return flagcxSuccess;
+}
+
+int fx_fifo_consumer_launch(fxFifoConsumer_t c, void *fifoDevicePointer, const uint64_t *fifoHost,
+                            unsigned long long maxIdlePolls, void *stream) {
+  if (!c || !fifoDevicePointer || !fifoHost || maxIdlePolls == 0) return flagcxInvalidArgument;
+  if (fifoHost[0] != c->capacity) return flagcxInvalidArgument;
+  hipStream_t s = (hipStream_t)stream;
+  FX_HIP(hipMemsetAsync(c->mirror, 0, sizeof(FifoMirror), s));
+  const uint64_t startSeq = fifoHost[2];  // triggers produced before this launch are not ours
+  hipLaunchKernelGGL(fifoConsumer, dim3(c->grid), dim3(kBlock), 0, s, (uint64_t *)fifoDevicePointer, c->mirror,
+                     c->capacity, startSeq, (uint64_t)maxIdlePolls);
+  FX_HIP(hipGetLastError());
+  return flagcxSuccess;
+}
+
+int fx_fifo_consumer_status(fxFifoConsumer_t c, int *exitReason, uint64_t *completed, uint64_t *badTriggers) {
+  if (!c) return flagcxInvalidArgument;
+  uint64_t head[8];  // produced, terminate, completed, exitReason, badTriggers, pad
+  static_assert(offsetof(FifoMirror, done) == sizeof(head), "FifoMirror header layout");
+  if (hipMemcpy(head, c->mirror, sizeof(head), hipMemcpyDeviceToHost) != hipSuccess) return flagcxUnhandledDeviceError;
+  if (completed) *completed = head[2];
+  if (exitReason) *exitReason = (int)head[3];
+  if (badTriggers) *badTriggers = head[4];
+  return flagcxSuccess;
+}
+
+int fx_fifo_consumer_destroy(fxFifoConsumer_t c) {
+  if (!c) return flagcxSuccess;
+  (void)hipFree(c->mirror);
+  delete c;
+  return flagcxSuccess;
+}
+
+#pragma GCC visibility pop
+}

@@ -6,6 +6,7 @@ algBw = bytes / 1e9 / t).  Usage:
     python -m flagcx_amd.perf slices            # BASELINE config 2: rank shares in 512 KiB pieces + all-gather copy
     python -m flagcx_amd.perf pack              # BASELINE config 4: alltoallv pack / unpack
     python -m flagcx_amd.perf allreduce -n 8 -d bf16 -b 1M -e 64M
+    python -m flagcx_amd.perf fifo -b 4K -e 256M -f 8   # round trips through the reduce FIFO
 """
 import argparse
 import sys
@@ -143,6 +144,54 @@ def run_pack(dev, a):
         t.ms(lambda: N.check(K.pack(dpk, dbig + 4, big, bd, N.DT_FP32, t.raw))), 2 * sum(big) * 4)
 
 
+def run_fifo(dev, a):
+    """Round trip through the reference's reduce FIFO with the persistent consumer:
+    host enqueue -> kernel executes -> host sees Complete.  Wall-clock on the host."""
+    import ctypes as C
+    import time
+    lib = N.lib
+    cap = 128
+    host = dev.malloc(lib.fx_fifo_bytes(cap), N.MEM_HOST)
+    N.check(lib.fx_fifo_init(host, cap))
+    dptr = C.c_void_p()
+    N.check(dev.t.hostGetDevicePointer(C.byref(dptr), host))
+    stream = dev.stream_create()
+    cons = C.c_void_p()
+    N.check(lib.fx_fifo_consumer_create(C.byref(cons), cap))
+    N.check(lib.fx_fifo_consumer_launch(cons, dptr, host, 20_000_000, dev.raw_stream(stream)))
+    emax = size(a.max)
+    bufs = [dev.malloc(emax) for _ in range(3)]
+    for i, p in enumerate(bufs):
+        dev.memset(p, 0x3c + i, emax)
+    idx = C.c_int()
+
+    def one(n):
+        while True:
+            lib.fx_fifo_enqueue(host, bufs[0], bufs[1], bufs[2], n, 32, N.DT_FP32, N.OP_SUM, C.byref(idx))
+            if idx.value >= 0:
+                break
+        while lib.fx_fifo_poll_state(host, idx.value) != 3:
+            pass
+        lib.fx_fifo_set_state(host, idx.value, 0)
+
+    try:
+        nbytes = size(a.min)
+        while nbytes <= emax:
+            n = nbytes // 4
+            for _ in range(5):
+                one(n)
+            t0 = time.perf_counter()
+            for _ in range(20):
+                one(n)
+            ms = (time.perf_counter() - t0) * 1e3 / 20
+            row("fifo round trip, fp32 sum, 2 inputs", nbytes, ms, 3 * nbytes)
+            nbytes *= a.factor
+    finally:
+        lib.fx_fifo_terminate(host)
+        dev.stream_sync(stream)
+        lib.fx_fifo_consumer_destroy(cons)
+
+
 def run_allreduce(dev, a):
     t = Timer(dev)
     dtype, n = DT[a.dtype], a.nranks
@@ -162,7 +211,7 @@ def run_allreduce(dev, a):
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce"])
+    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo"])
     ap.add_argument("-k", type=int, default=4)
     ap.add_argument("-n", "--nranks", type=int, default=8)
     ap.add_argument("-d", "--dtype", default="fp32", choices=list(DT))
@@ -177,7 +226,8 @@ def main(argv=None):
                     help="start input i at byte offset i*IN_SHIFT of its allocation (multiple of 16 keeps vector loads)")
     a = ap.parse_args(argv)
     dev = Device(0)
-    {"reduce": run_reduce, "slices": run_slices, "pack": run_pack, "allreduce": run_allreduce}[a.what](dev, a)
+    {"reduce": run_reduce, "slices": run_slices, "pack": run_pack, "allreduce": run_allreduce,
+     "fifo": run_fifo}[a.what](dev, a)
 
 
 if __name__ == "__main__":

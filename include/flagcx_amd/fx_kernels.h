@@ -79,6 +79,43 @@ void fx_trigger_get(const fxReduceTrigger *t, uint64_t *in1, uint64_t *in2,
  */
 int fx_reduce_triggers(const fxReduceTrigger *triggers, size_t n, void *stream);
 
+/*
+ * The reference's reduce FIFO, host side (flagcx/core/flagcx_reduce_kernel_host.cc:46-98):
+ * a pinned buffer of uint64 words [capacity, consumed, produced, terminate]
+ * followed by `capacity` triggers.  fx_fifo_enqueue returns idx = -1 when the
+ * ring is full or the slot has not been collected yet (the caller retries);
+ * fx_fifo_poll_state / fx_fifo_set_state are pollState / setState.
+ */
+size_t fx_fifo_bytes(size_t capacity);
+int fx_fifo_init(uint64_t *fifo, size_t capacity);
+int fx_fifo_enqueue(uint64_t *fifo, uint64_t in1, uint64_t in2, uint64_t out,
+                    size_t count, size_t nthreads, int dtype, int op, int *idx);
+int fx_fifo_poll_state(const uint64_t *fifo, int idx);
+int fx_fifo_set_state(uint64_t *fifo, int idx, int state);
+int fx_fifo_terminate(uint64_t *fifo);
+
+/*
+ * FIFO-compatible consumer: the drop-in for flagcxLaunchCollectiveKernel
+ * (flagcx/adaptor/kernel/nvidia/flagcx_reduce_kernel_device.cu:88-192).  A
+ * persistent full-width kernel executes every trigger the host enqueues, for
+ * all four ops and types, and marks it Complete; it returns when `terminate`
+ * is set and the ring is drained, or after maxIdlePolls consecutive empty
+ * polls (so it always ends).  fifoDevicePointer is hostGetDevicePointer() of
+ * the pinned ring, fifoHost the ring itself.  Triggers that sit in the ring at
+ * the same time must not depend on each other.  Capacity <= 1024.
+ */
+typedef struct fxFifoConsumer *fxFifoConsumer_t;
+enum { FX_FIFO_RUNNING = 0, FX_FIFO_EXIT_TERMINATE = 1, FX_FIFO_EXIT_IDLE = 2 };
+int fx_fifo_consumer_create(fxFifoConsumer_t *consumer, size_t capacity);
+int fx_fifo_consumer_launch(fxFifoConsumer_t consumer, void *fifoDevicePointer,
+                            const uint64_t *fifoHost,
+                            unsigned long long maxIdlePolls, void *stream);
+/* after the stream has drained: why the kernel ended, how many triggers it
+ * completed, how many it skipped for an unsupported dtype / op */
+int fx_fifo_consumer_status(fxFifoConsumer_t consumer, int *exitReason,
+                            uint64_t *completed, uint64_t *badTriggers);
+int fx_fifo_consumer_destroy(fxFifoConsumer_t consumer);
+
 /* k-way slice descriptor: up to 8 inputs, `count` elements. */
 typedef struct fxSliceDesc {
   const void *in[FX_MAX_SLICE_INPUTS];

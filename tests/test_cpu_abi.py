@@ -213,3 +213,27 @@ def test_argument_screening_needs_no_gpu():
     assert N.lib.fxSimCommInitAll(comms, 0) == N.INVALID_ARGUMENT
     assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP64, N.OP_SUM, None, None) == N.NOT_SUPPORTED
     assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, None, None) == N.INVALID_ARGUMENT
+
+
+def test_reduce_fifo_host_protocol():
+    """enqueue / full ring / slot-not-collected behaviour of the host side
+    (flagcx_reduce_kernel_host.cc:55-70), with no consumer running."""
+    nbytes = N.lib.fx_fifo_bytes(2)
+    buf = (C.c_uint64 * (nbytes // 8))()
+    N.check(N.lib.fx_fifo_init(buf, 2))
+    idx = C.c_int()
+    for want in (0, 1):
+        N.check(N.lib.fx_fifo_enqueue(buf, 1, 2, 3, 4, 32, N.DT_FP32, N.OP_SUM, C.byref(idx)))
+        assert idx.value == want and N.lib.fx_fifo_poll_state(buf, want) == 1
+    N.check(N.lib.fx_fifo_enqueue(buf, 1, 2, 3, 4, 32, N.DT_FP32, N.OP_SUM, C.byref(idx)))
+    assert idx.value == -1                                           # full: produced - consumed >= capacity
+    buf[1] = 1                                                       # the consumer took one ...
+    N.check(N.lib.fx_fifo_enqueue(buf, 1, 2, 3, 4, 32, N.DT_FP32, N.OP_SUM, C.byref(idx)))
+    assert idx.value == -1                                           # ... but slot 0 is not Available yet
+    N.check(N.lib.fx_fifo_set_state(buf, 0, 3))
+    N.check(N.lib.fx_fifo_set_state(buf, 0, 0))
+    N.check(N.lib.fx_fifo_enqueue(buf, 9, 8, 7, 6, 32, N.DT_BF16, N.OP_MAX, C.byref(idx)))
+    assert idx.value == 0 and buf[2] == 3 and buf[4] == 9 and buf[6] == 7
+    assert (buf[7] >> 48) & 0xf == N.DT_BF16 and (buf[7] >> 52) & 0xf == N.OP_MAX and buf[7] & 0xffffffff == 6
+    assert N.lib.fx_fifo_init(buf, 0) == N.INVALID_ARGUMENT and N.lib.fx_fifo_init(buf, 2000) == N.INVALID_ARGUMENT
+    assert N.lib.fx_fifo_poll_state(buf, 5) == -1

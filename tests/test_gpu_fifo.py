@@ -1,0 +1,130 @@
+"""FIFO-compatible consumer: the reference's reduce-trigger ring
+(flagcx/core/flagcx_reduce_kernel_host.cc:46-98) driven exactly as its
+scheduler drives it -- enqueue, poll for Complete, release the slot, terminate
+-- with the persistent gfx950 kernel on the other end.  Every host wait has a
+deadline and every kernel wait a poll limit, so nothing here can hang."""
+import ctypes as C
+import time
+
+import numpy as np
+import pytest
+
+from flagcx_amd import _native as N
+from oracle import fx_oracle as O
+from tests.util import DevBufs, assert_parity, seeded_inputs
+
+pytestmark = pytest.mark.gpu
+lib = N.lib
+AVAILABLE, ENQUEUED, INPROGRESS, COMPLETE = 0, 1, 2, 3
+POLL_LIMIT = 4_000_000          # kernel-side bound: a few seconds of empty polls
+DEADLINE = 20.0                 # host-side bound per wait, seconds
+
+
+class Ring:
+    """Pinned ring + consumer kernel on its own stream."""
+
+    def __init__(self, dev, capacity, poll_limit=POLL_LIMIT):
+        self.dev, self.cap = dev, capacity
+        self.nbytes = lib.fx_fifo_bytes(capacity)
+        self.host = dev.malloc(self.nbytes, N.MEM_HOST)
+        N.check(lib.fx_fifo_init(self.host, capacity))
+        dptr = C.c_void_p()
+        N.check(dev.t.hostGetDevicePointer(C.byref(dptr), self.host))
+        self.stream = dev.stream_create()
+        self.consumer = C.c_void_p()
+        N.check(lib.fx_fifo_consumer_create(C.byref(self.consumer), capacity))
+        N.check(lib.fx_fifo_consumer_launch(self.consumer, dptr, self.host, poll_limit, dev.raw_stream(self.stream)))
+
+    def words(self):
+        return np.ctypeslib.as_array(C.cast(self.host, C.POINTER(C.c_uint64)), shape=(4,))
+
+    def enqueue(self, in1, in2, out, count, dtype, op):
+        idx = C.c_int(-1)
+        t0 = time.time()
+        while True:
+            N.check(lib.fx_fifo_enqueue(self.host, in1, in2, out, count, 32, dtype, op, C.byref(idx)))
+            if idx.value >= 0:
+                return idx.value
+            assert time.time() - t0 < DEADLINE, "ring never drained"
+
+    def wait(self, idx):
+        t0 = time.time()
+        while lib.fx_fifo_poll_state(self.host, idx) != COMPLETE:
+            assert time.time() - t0 < DEADLINE, f"trigger in slot {idx} never completed"
+        N.check(lib.fx_fifo_set_state(self.host, idx, AVAILABLE))
+
+    def close(self):
+        """terminate -> the kernel drains and exits; returns (exitReason, completed, bad)."""
+        lib.fx_fifo_terminate(self.host)
+        self.dev.stream_sync(self.stream)
+        reason, done, bad = C.c_int(-1), C.c_uint64(), C.c_uint64()
+        N.check(lib.fx_fifo_consumer_status(self.consumer, C.byref(reason), C.byref(done), C.byref(bad)))
+        lib.fx_fifo_consumer_destroy(self.consumer)
+        self.dev.stream_destroy(self.stream)
+        self.dev.free(self.host, N.MEM_HOST)
+        return reason.value, done.value, bad.value
+
+
+def test_triggers_through_the_ring(dev):
+    cases = [(N.DT_FP32, N.OP_SUM, 100003), (N.DT_BF16, N.OP_SUM, 1 << 20), (N.DT_INT32, N.OP_PROD, 7),
+             (N.DT_FP16, N.OP_MAX, 65537), (N.DT_FP32, N.OP_MIN, 3 << 20), (N.DT_BF16, N.OP_PROD, 1),
+             (N.DT_FP32, N.OP_SUM, 0)]
+    ring = Ring(dev, capacity=4)                 # 4 slots, 21 triggers: the ring wraps five times
+    closed = False
+    try:
+        with DevBufs(dev) as b:
+            total = 0
+            for rep in range(3):
+                for dtype, op, n in cases:
+                    a, c = seeded_inputs(dtype, 2, max(n, 1), seed=rep * 10 + op)
+                    da, dc = b.put(a), b.put(c)
+                    do = b.alloc(max(n, 1) * 4)
+                    idx = ring.enqueue(da, dc, do, n, dtype, op)
+                    ring.wait(idx)
+                    total += 1
+                    if n:
+                        got = dev.to_host(do, n, N.NP_DTYPE[dtype])
+                        assert_parity(got, O.reduce2(a[:n], c[:n], dtype, op), dtype, op, f"fifo {dtype} {op} {n}")
+            # several independent triggers in flight at once, collected afterwards
+            a, c = seeded_inputs(N.DT_FP32, 2, 4 * 50000, seed=77)
+            da, dc, do = b.put(a), b.put(c), b.alloc(4 * 50000 * 4)
+            slots = [ring.enqueue(da + q * 200000, dc + q * 200000, do + q * 200000, 50000, N.DT_FP32, N.OP_SUM)
+                     for q in range(4)]
+            for s in slots:
+                ring.wait(s)
+            total += 4
+            assert_parity(dev.to_host(do, 200000, np.float32), O.reduce2(a, c, N.DT_FP32, N.OP_SUM), N.DT_FP32, N.OP_SUM)
+            # a ring reduce-scatter chain: each step's output is the next step's input1 (output == input1)
+            k, n = 5, 300001
+            ins = seeded_inputs(N.DT_FP32, k, n, seed=5)
+            dins = [b.put(x) for x in ins]
+            for p in range(1, k):
+                ring.wait(ring.enqueue(dins[0], dins[p], dins[0], n, N.DT_FP32, N.OP_SUM))
+                total += 1
+            assert_parity(dev.to_host(dins[0], n, np.float32), O.reduce_copy(ins, N.DT_FP32, N.OP_SUM), N.DT_FP32,
+                          N.OP_SUM, "chain")
+            # a type the path does not carry is completed (so the producer is not left waiting) and counted
+            ring.wait(ring.enqueue(dins[0], dins[1], dins[0], 16, N.DT_FP64, N.OP_SUM))
+            total += 1
+            w = ring.words()
+            assert w[0] == 4 and w[2] == total                      # capacity, produced
+            host = ring.host
+            lib.fx_fifo_terminate(host)
+            dev.stream_sync(ring.stream)
+            assert int(w[1]) == total                               # consumed, published by the kernel on its way out
+            reason, done, bad = ring.close()
+            closed = True
+            assert (reason, done, bad) == (N.SUCCESS + 1, total, 1)  # FX_FIFO_EXIT_TERMINATE
+    finally:
+        if not closed:
+            ring.close()
+
+
+def test_consumer_ends_by_itself_when_idle(dev):
+    """No trigger, no terminate: the poll limit ends the kernel."""
+    ring = Ring(dev, capacity=8, poll_limit=2000)
+    t0 = time.time()
+    dev.stream_sync(ring.stream)
+    assert time.time() - t0 < DEADLINE
+    reason, done, bad = ring.close()
+    assert (reason, done, bad) == (2, 0, 0)                          # FX_FIFO_EXIT_IDLE

@@ -238,12 +238,57 @@ flagcxResult_t runAllReduce(const Ctx &c) {
   return R(fx_copy_slices(descs.data(), descs.size(), c.s));
 }
 
+// Receive steps of tree rank a (uni_runner_impl.cc:1314-1326): the root takes
+// ceil(log2 n); others ctz(a), clipped so that a + 2^i stays below n.
+int treeSteps(int a, int n) {
+  int total = 0;
+  while ((1 << total) < n) total++;
+  if (a == 0) return total;
+  int st = __builtin_ctz((unsigned)a);
+  if (st && n - a <= (1 << (st - 1))) {
+    int rest = n - a - 1;
+    for (st = 0; rest; rest >>= 1) st++;
+  }
+  return st;
+}
+
 flagcxResult_t runReduce(const Ctx &c) {
   Group *g = c.g;
-  if (g->count == 0) return flagcxSuccess;
-  std::vector<const void *> in(c.n);
-  for (int j = 0; j < c.n; j++) in[j] = c.send(j);
-  return R(fx_reduce_copy(c.recv(g->root), in.data(), c.n, g->count, g->dtype, g->op, 0, c.s));
+  const int n = c.n, root = g->root;
+  const size_t count = g->count, ts = c.ts;
+  if (count == 0) return flagcxSuccess;
+  if (g->order != FX_ORDER_TREE || n == 1) {
+    std::vector<const void *> in(n);
+    for (int j = 0; j < n; j++) in[j] = c.send(j);
+    return R(fx_reduce_copy(c.recv(root), in.data(), n, count, g->dtype, g->op, 0, c.s));
+  }
+  // Tree order: round i, every tree rank a with more than i receive steps
+  // computes partial(a) = partial(a + 2^i) (op) partial(a).  Partials live in a
+  // per-rank scratch row; the root's last round writes recvbuff.
+  flagcxResult_t rc = ensureScratch(g, (size_t)n * count * ts);
+  if (rc != flagcxSuccess) return rc;
+  const int total = treeSteps(0, n);
+  auto rankOf = [&](int a) { return mod(a + root, n); };
+  auto partial = [&](int a, int round) -> const void * {   // where tree rank a's partial is before `round`
+    return (round == 0 || treeSteps(a, n) == 0) ? c.send(rankOf(a)) : madd(g->scratch, (size_t)a * count * ts);
+  };
+  std::vector<fxSliceDesc> descs;
+  for (int i = 0; i < total; i++) {
+    for (int a = 0; a < n; a++) {
+      if (treeSteps(a, n) <= i) continue;
+      fxSliceDesc d;
+      memset(&d, 0, sizeof(d));
+      d.in[0] = partial(a + (1 << i), i);   // received
+      d.in[1] = partial(a, i);              // own
+      d.out = (a == 0 && i == total - 1) ? c.recv(root) : madd(g->scratch, (size_t)a * count * ts);
+      d.count = count;
+      descs.push_back(d);
+    }
+    rc = R(fx_reduce_slices(descs.data(), descs.size(), 2, g->dtype, g->op, c.s));
+    descs.clear();
+    if (rc != flagcxSuccess) return rc;
+  }
+  return flagcxSuccess;
 }
 
 flagcxResult_t runReduceScatter(const Ctx &c) {
@@ -699,7 +744,7 @@ flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
       g->algo = value;
       break;
     case FX_SIM_ORDER:
-      if (value != FX_ORDER_RANK && value != FX_ORDER_RING) return flagcxInvalidArgument;
+      if (value != FX_ORDER_RANK && value != FX_ORDER_RING && value != FX_ORDER_TREE) return flagcxInvalidArgument;
       g->order = value;
       break;
     case FX_SIM_NSLICES:

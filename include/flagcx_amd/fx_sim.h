@@ -57,7 +57,10 @@ enum {
 };
 enum {
   FX_ORDER_RANK = 0, /* rank 0,1,..,n-1: the custom allreduce's peer loop    */
-  FX_ORDER_RING = 1  /* the rotated order a ring yields for each chunk       */
+  FX_ORDER_RING = 1, /* the rotated order a ring yields for each chunk       */
+  FX_ORDER_TREE = 2  /* flagcxReduce only: the binomial tree of
+                        initUniRunnerStateTreeRed (uni_runner_impl.cc:1266-1557),
+                        ceil(log2 n) rounds of two-input reduces               */
 };
 flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value);
 

@@ -25,6 +25,8 @@
  *       acc*=x left to right and checked against numpy only.
  *   oracle_split / plans ...................... tiling invariants + closed
  *       forms of the reference's divisible cases.
+ *   oracle_tree_reduce ........................ hand-derived associations for
+ *       n = 3, 5, 6, 8 on non-associative values + the reference's closed forms.
  *   oracle_pack / oracle_unpack ............... round-trip identity and the
  *       displacement arithmetic of service/bootstrap.cc:1253-1258.
  *   trigger encode/decode ..................... bit constants of
@@ -460,6 +462,60 @@ int oracle_ring_allreduce(void *const *recv, const void *const *send,
   }
   free(wire);
   return RC_OK;
+}
+
+/*
+ * Binomial ("halving doubling") tree reduce to `root`, hop by hop
+ * (runner/uni_runner_impl.cc:1266-1557).  With a = (rank - root) mod n, rank a
+ * receives from a + 2^i for i = 0 .. steps(a)-1 and each time computes
+ * partial = received (op) partial (the reduce node's input1 is the received
+ * data, :1448-1457); steps(0) = ceil(log2 n), otherwise ctz(a) clipped so that
+ * a + 2^i < n (:1316-1326).  For n = 8, root 0:
+ * ((x7+x6)+(x5+x4)) + ((x3+x2)+(x1+x0)).
+ */
+static int tree_steps(int a, int n) {
+  int total = 0;
+  while ((1 << total) < n) total++; /* 8*sizeof(int) - clz(n-1) for n >= 2 */
+  if (a == 0) return total;
+  int st = __builtin_ctz((unsigned)a);
+  if (st && n - a <= (1 << (st - 1))) {
+    int rest = n - a - 1;
+    st = 0;
+    while (rest) {
+      st++;
+      rest >>= 1;
+    }
+  }
+  return st;
+}
+
+int oracle_tree_steps(int algo_rank, int nranks) { return tree_steps(algo_rank, nranks); }
+
+static int tree_value(void *acc, const void *const *send, int n, int root, int a, size_t count, int dtype, int op) {
+  size_t bytes = count * oracle_dtype_size(dtype);
+  memcpy(acc, send[(a + root) % n], bytes);
+  int st = tree_steps(a, n);
+  for (int i = 0; i < st; i++) {
+    void *peer = malloc(bytes ? bytes : 1);
+    if (!peer) return RC_INVALID;
+    int rc = tree_value(peer, send, n, root, a + (1 << i), count, dtype, op);
+    if (!rc) rc = oracle_reduce2(acc, peer, acc, count, dtype, op); /* received (op) own */
+    free(peer);
+    if (rc) return rc;
+  }
+  return RC_OK;
+}
+
+int oracle_tree_reduce(void *recv_root, const void *const *send, int nranks, int root, size_t count, int dtype,
+                       int op) {
+  int rc = check_args(dtype, op);
+  if (rc) return rc;
+  if (nranks < 1 || root < 0 || root >= nranks) return RC_INVALID;
+  if (nranks == 1) {
+    if (count && recv_root != send[0]) memmove(recv_root, send[0], count * oracle_dtype_size(dtype));
+    return RC_OK;
+  }
+  return tree_value(recv_root, send, nranks, root, 0, count, dtype, op);
 }
 
 /* ------------------------------------------------------------- alltoallv */

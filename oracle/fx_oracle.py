@@ -44,6 +44,10 @@ lib.oracle_plan_locred.restype = _sz
 lib.oracle_plan_locred.argtypes = [_sz, _i, _i, _sz, C.POINTER(RedNode)]
 lib.oracle_ring_allreduce.restype = _i
 lib.oracle_ring_allreduce.argtypes = [C.POINTER(_vp), C.POINTER(_vp), _i, _sz, _i, _i]
+lib.oracle_tree_reduce.restype = _i
+lib.oracle_tree_reduce.argtypes = [_vp, C.POINTER(_vp), _i, _i, _sz, _i, _i]
+lib.oracle_tree_steps.restype = _i
+lib.oracle_tree_steps.argtypes = [_i, _i]
 lib.oracle_pack.restype = None
 lib.oracle_pack.argtypes = [_vp, _vp, C.POINTER(_sz), C.POINTER(_sz), _i, _sz]
 lib.oracle_unpack.restype = None
@@ -133,6 +137,16 @@ def ring_allreduce(sends, dtype, op):
     if rc:
         raise ValueError(f"oracle_ring_allreduce rc={rc}")
     return recvs
+
+
+def tree_reduce(sends, root, dtype, op):
+    """Result at `root` of the reference's binomial-tree reduce."""
+    sends = [np.ascontiguousarray(a) for a in sends]
+    out = np.empty_like(sends[0])
+    rc = lib.oracle_tree_reduce(out.ctypes.data, _ptrs(sends), len(sends), root, sends[0].size, dtype, op)
+    if rc:
+        raise ValueError(f"oracle_tree_reduce rc={rc}")
+    return out
 
 
 def _szs(v):

@@ -333,6 +333,49 @@ def test_ring_allreduce_order_is_the_rotated_left_fold():
             assert np.array_equal(recvs[r][off:off + cnt].view(np.uint32), want.view(np.uint32))
 
 
+# ---- binomial tree reduce (uni_runner_impl.cc:1266-1557) -----------------------------------------
+def test_tree_reduce_associations_derived_by_hand():
+    """Receive steps: root ceil(log2 n); others ctz(a) clipped to a + 2^i < n.  Each
+    hop computes received + own.  Values chosen so that every association differs."""
+    f = np.float32
+    steps = lambda n: [O.lib.oracle_tree_steps(a, n) for a in range(n)]
+    assert steps(8) == [3, 0, 1, 0, 2, 0, 1, 0]
+    assert steps(5) == [3, 0, 1, 0, 0]
+    assert steps(6) == [3, 0, 1, 0, 1, 0]
+    assert steps(3) == [2, 0, 0] and steps(2) == [1, 0] and steps(7) == [3, 0, 1, 0, 2, 0, 0]
+    rng = np.random.default_rng(11)
+    x = [(rng.standard_normal(4000) * 10.0 ** rng.integers(-6, 7, 4000)).astype(f) for _ in range(8)]
+    add = lambda a, b: (a + b).astype(f)
+    want = {
+        3: add(x[2], add(x[1], x[0])),
+        5: add(x[4], add(add(x[3], x[2]), add(x[1], x[0]))),
+        6: add(add(x[5], x[4]), add(add(x[3], x[2]), add(x[1], x[0]))),
+        8: add(add(add(x[7], x[6]), add(x[5], x[4])), add(add(x[3], x[2]), add(x[1], x[0]))),
+    }
+    for n, w in want.items():
+        got = O.tree_reduce(x[:n], 0, F32, SUM)
+        assert np.array_equal(got.view(np.uint32), w.view(np.uint32)), n
+        # a different order would not have matched (n = 3 is the left fold up to commutativity)
+        if n > 3:
+            assert not np.array_equal(got.view(np.uint32), O.reduce_copy(x[:n], F32, SUM).view(np.uint32)), n
+    # root r renumbers ranks: tree rank a is rank (a + r) % n
+    got = O.tree_reduce(x[:5], 2, F32, SUM)
+    y = [x[(a + 2) % 5] for a in range(5)]
+    assert np.array_equal(got, add(y[4], add(add(y[3], y[2]), add(y[1], y[0]))))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 7, 8])
+def test_tree_reduce_closed_forms(n):
+    # test/unittest/runner/coll_reduce.cpp uses the allreduce pattern at the root
+    count = 999
+    i = np.arange(count)
+    sends = [(r * 1000 + i % 10).astype(np.float32) for r in range(n)]
+    for root in {0, n - 1}:
+        assert np.array_equal(O.tree_reduce(sends, root, F32, SUM), (n * (n - 1) // 2 * 1000 + n * (i % 10)).astype(np.float32))
+    ints = [np.full(count, r + 1, np.int32) for r in range(n)]
+    assert (O.tree_reduce(ints, 0, I32, MAX) == n).all() and (O.tree_reduce(ints, 0, I32, MIN) == 1).all()
+
+
 # ---- alltoallv pack / unpack ----------------------------------------------------------------------
 def test_pack_unpack_round_trip_and_layout():
     rng = np.random.default_rng(8)

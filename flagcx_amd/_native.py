@@ -18,9 +18,11 @@ OP_SUM, OP_PROD, OP_MAX, OP_MIN, OP_AVG = 0, 1, 2, 3, 4
 MEMCPY_H2D, MEMCPY_D2H, MEMCPY_D2D = 0, 1, 2
 MEM_HOST, MEM_DEVICE, MEM_MANAGED = 0, 1, 2
 
-DTYPE_SIZE = {DT_INT32: 4, DT_FP32: 4, DT_FP16: 2, DT_BF16: 2}
+DTYPE_SIZE = {DT_INT8: 1, DT_UINT8: 1, DT_INT32: 4, DT_UINT32: 4, DT_INT64: 8, DT_UINT64: 8,
+              DT_FP16: 2, DT_FP32: 4, DT_FP64: 8, DT_BF16: 2}
 # host-side container dtypes: 16-bit floats travel as raw uint16 bit patterns
-NP_DTYPE = {DT_INT32: np.int32, DT_FP32: np.float32, DT_FP16: np.uint16, DT_BF16: np.uint16}
+NP_DTYPE = {DT_INT8: np.int8, DT_UINT8: np.uint8, DT_INT32: np.int32, DT_UINT32: np.uint32, DT_INT64: np.int64,
+            DT_UINT64: np.uint64, DT_FP16: np.uint16, DT_FP32: np.float32, DT_FP64: np.float64, DT_BF16: np.uint16}
 
 
 class FlagcxError(RuntimeError):

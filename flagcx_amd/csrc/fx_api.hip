@@ -30,6 +30,12 @@ const KernelSet *setFor(int dtype, int op) {
     case flagcxInt32: return &kernelSetsI32()[op];
     case flagcxBfloat16: return &kernelSetsBF16()[op];
     case flagcxFloat16: return &kernelSetsF16()[op];
+    case flagcxUint32: return &kernelSetsU32()[op];
+    case flagcxInt8: return &kernelSetsI8()[op];
+    case flagcxUint8: return &kernelSetsU8()[op];
+    case flagcxInt64: return &kernelSetsI64()[op];
+    case flagcxUint64: return &kernelSetsU64()[op];
+    case flagcxFloat64: return &kernelSetsF64()[op];
     default: return nullptr;
   }
 }

@@ -16,10 +16,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __host__ __device__ inline size_t dtypeSize(int dt) {
   switch (dt) {
-    case flagcxInt32:
-    case flagcxFloat32: return 4;
+    case flagcxInt8:
+    case flagcxUint8: return 1;
     case flagcxFloat16:
     case flagcxBfloat16: return 2;
+    case flagcxInt32:
+    case flagcxUint32:
+    case flagcxFloat32: return 4;
+    case flagcxInt64:
+    case flagcxUint64:
+    case flagcxFloat64: return 8;
     default: return 0;
   }
 }

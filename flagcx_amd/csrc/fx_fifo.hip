@@ -168,6 +168,12 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
         case flagcxInt32: ok = runShareOp<flagcxInt32>(op, in1, in2, out, count); break;
         case flagcxBfloat16: ok = runShareOp<flagcxBfloat16>(op, in1, in2, out, count); break;
         case flagcxFloat16: ok = runShareOp<flagcxFloat16>(op, in1, in2, out, count); break;
+        case flagcxUint32: ok = runShareOp<flagcxUint32>(op, in1, in2, out, count); break;
+        case flagcxInt8: ok = runShareOp<flagcxInt8>(op, in1, in2, out, count); break;
+        case flagcxUint8: ok = runShareOp<flagcxUint8>(op, in1, in2, out, count); break;
+        case flagcxInt64: ok = runShareOp<flagcxInt64>(op, in1, in2, out, count); break;
+        case flagcxUint64: ok = runShareOp<flagcxUint64>(op, in1, in2, out, count); break;
+        case flagcxFloat64: ok = runShareOp<flagcxFloat64>(op, in1, in2, out, count); break;
         default: ok = false;
       }
     }

@@ -121,6 +121,12 @@ const KernelSet *kernelSetsF32();
 const KernelSet *kernelSetsI32();
 const KernelSet *kernelSetsBF16();
 const KernelSet *kernelSetsF16();
+const KernelSet *kernelSetsU32();
+const KernelSet *kernelSetsI8();
+const KernelSet *kernelSetsU8();
+const KernelSet *kernelSetsI64();
+const KernelSet *kernelSetsU64();
+const KernelSet *kernelSetsF64();
 const KernelSet *kernelSetsCopy();  // index log2(ES): 0 -> 1 byte, 1 -> 2, 2 -> 4
 
 }  // namespace fx

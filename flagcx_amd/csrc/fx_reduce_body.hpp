@@ -3,7 +3,10 @@
 // Arithmetic contract (order follows FlagCX's peer loop,
 // flagcx/adaptor/kernel/nvidia/custom_allreduce.cu:345-359):
 //   acc = in[0]; acc = acc (op) in[p] for p = 1..k-1, left to right.
-//   fp32: plain IEEE single arithmetic.  int32: sum/prod wrap modulo 2^32.
+//   fp32 / fp64: plain IEEE arithmetic.  Integers of every width: sum/prod
+//   wrap modulo 2^width (the host loops of flagcx/service/include/utils.h:664-725
+//   on the types FlagCX dispatches there: char = signed 8-bit on x86-64,
+//   unsigned char, int32_t, uint32_t, int64_t, uint64_t, float, double).
 //   bf16/fp16 sum and prod: every input widened to fp32, accumulated in fp32,
 //   rounded to nearest even once.  max = (acc < x) ? x : acc and
 //   min = (x < acc) ? x : acc (the std::max / std::min of
@@ -100,6 +103,141 @@ struct Red<flagcxInt32, OP> {
     u32x4 r;
 #pragma unroll
     for (int i = 0; i < 4; i++) r[i] = c.a[i];
+    return r;
+  }
+};
+
+// uint32: as int32 with unsigned comparisons.
+template <int OP>
+struct Red<flagcxUint32, OP> {
+  static constexpr int ES = 4;
+  struct Acc {
+    uint32_t a[4];
+  };
+  static __device__ __forceinline__ uint32_t op(uint32_t a, uint32_t b) {
+    if (OP == flagcxSum) return a + b;
+    if (OP == flagcxProd) return a * b;
+    if (OP == flagcxMax) return (a < b) ? b : a;
+    return (b < a) ? b : a;
+  }
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) c.a[i] = v[i];
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) c.a[i] = op(c.a[i], v[i]);
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = c.a[i];
+    return r;
+  }
+};
+
+// 8-bit integers: sixteen per vector, each kept in a 32-bit accumulator
+// (sign- or zero-extended).  The low byte of a 32-bit sum or product is the
+// 8-bit result modulo 256; max/min compare the extended values.
+template <bool SIGNED, int OP>
+struct Red8 {
+  static constexpr int ES = 1;
+  struct Acc {
+    int32_t a[16];
+  };
+  static __device__ __forceinline__ int32_t lane(uint32_t w, int b) {
+    return SIGNED ? ((int32_t)(w << (24 - 8 * b)) >> 24) : (int32_t)((w >> (8 * b)) & 0xffu);
+  }
+  static __device__ __forceinline__ int32_t op(int32_t a, int32_t b) {
+    if (OP == flagcxSum) return (int32_t)((uint32_t)a + (uint32_t)b);
+    if (OP == flagcxProd) return (int32_t)((uint32_t)a * (uint32_t)b);
+    if (OP == flagcxMax) return (a < b) ? b : a;
+    return (b < a) ? b : a;
+  }
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) c.a[i] = lane(v[i / 4], i & 3);
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) c.a[i] = op(c.a[i], lane(v[i / 4], i & 3));
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      r[i] = ((uint32_t)c.a[4 * i] & 0xffu) | (((uint32_t)c.a[4 * i + 1] & 0xffu) << 8) |
+             (((uint32_t)c.a[4 * i + 2] & 0xffu) << 16) | ((uint32_t)c.a[4 * i + 3] << 24);
+    return r;
+  }
+};
+template <int OP>
+struct Red<flagcxInt8, OP> : Red8<true, OP> {};
+template <int OP>
+struct Red<flagcxUint8, OP> : Red8<false, OP> {};
+
+// 64-bit integers and doubles: two per vector.
+template <bool SIGNED, int OP>
+struct RedI64 {
+  static constexpr int ES = 8;
+  struct Acc {
+    uint64_t a[2];
+  };
+  static __device__ __forceinline__ uint64_t op(uint64_t a, uint64_t b) {
+    if (OP == flagcxSum) return a + b;
+    if (OP == flagcxProd) return a * b;
+    const bool lt = SIGNED ? ((int64_t)a < (int64_t)b) : (a < b);
+    const bool gt = SIGNED ? ((int64_t)b < (int64_t)a) : (b < a);
+    if (OP == flagcxMax) return lt ? b : a;
+    return gt ? b : a;
+  }
+  static __device__ __forceinline__ uint64_t word(u32x4 v, int i) {
+    return (uint64_t)v[2 * i] | ((uint64_t)v[2 * i + 1] << 32);
+  }
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+    c.a[0] = word(v, 0);
+    c.a[1] = word(v, 1);
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+    c.a[0] = op(c.a[0], word(v, 0));
+    c.a[1] = op(c.a[1], word(v, 1));
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    u32x4 r = {(uint32_t)c.a[0], (uint32_t)(c.a[0] >> 32), (uint32_t)c.a[1], (uint32_t)(c.a[1] >> 32)};
+    return r;
+  }
+};
+template <int OP>
+struct Red<flagcxInt64, OP> : RedI64<true, OP> {};
+template <int OP>
+struct Red<flagcxUint64, OP> : RedI64<false, OP> {};
+
+template <int OP>
+struct Red<flagcxFloat64, OP> {
+  static constexpr int ES = 8;
+  struct Acc {
+    double a[2];
+  };
+  static __device__ __forceinline__ double op(double a, double b) {
+    if (OP == flagcxSum) return a + b;
+    if (OP == flagcxProd) return a * b;
+    if (OP == flagcxMax) return (a < b) ? b : a;
+    return (b < a) ? b : a;
+  }
+  static __device__ __forceinline__ double word(u32x4 v, int i) {
+    return __longlong_as_double((long long)((uint64_t)v[2 * i] | ((uint64_t)v[2 * i + 1] << 32)));
+  }
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+    c.a[0] = word(v, 0);
+    c.a[1] = word(v, 1);
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+    c.a[0] = op(c.a[0], word(v, 0));
+    c.a[1] = op(c.a[1], word(v, 1));
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+    const uint64_t x = (uint64_t)__double_as_longlong(c.a[0]), y = (uint64_t)__double_as_longlong(c.a[1]);
+    u32x4 r = {(uint32_t)x, (uint32_t)(x >> 32), (uint32_t)y, (uint32_t)(y >> 32)};
     return r;
   }
 };
@@ -299,9 +437,13 @@ __device__ __forceinline__ u32x4 gatherElems(const char *base, uint64_t e0, int 
 #pragma unroll
   for (int s = 0; s < VE; s++) {
     if (s >= lo && s < hi) {
-      if (ES == 4) {
+      if constexpr (ES == 8) {
+        const uint64_t w = *reinterpret_cast<const uint64_t *>(base + (e0 + s) * 8);
+        r[2 * s] = (uint32_t)w;
+        r[2 * s + 1] = (uint32_t)(w >> 32);
+      } else if constexpr (ES == 4) {
         r[s] = *reinterpret_cast<const uint32_t *>(base + (e0 + s) * 4);
-      } else if (ES == 2) {
+      } else if constexpr (ES == 2) {
         uint32_t h = *reinterpret_cast<const uint16_t *>(base + (e0 + s) * 2);
         r[s / 2] |= h << (16 * (s & 1));
       } else {
@@ -319,9 +461,11 @@ __device__ __forceinline__ void scatterElems(char *base, uint64_t e0, int lo, in
 #pragma unroll
   for (int s = 0; s < VE; s++) {
     if (s >= lo && s < hi) {
-      if (ES == 4)
+      if constexpr (ES == 8)
+        *reinterpret_cast<uint64_t *>(base + (e0 + s) * 8) = (uint64_t)v[2 * s] | ((uint64_t)v[2 * s + 1] << 32);
+      else if constexpr (ES == 4)
         *reinterpret_cast<uint32_t *>(base + (e0 + s) * 4) = v[s];
-      else if (ES == 2)
+      else if constexpr (ES == 2)
         *reinterpret_cast<uint16_t *>(base + (e0 + s) * 2) = (uint16_t)(v[s / 2] >> (16 * (s & 1)));
       else
         *reinterpret_cast<uint8_t *>(base + e0 + s) = (uint8_t)(v[s / 4] >> (8 * (s & 3)));

@@ -567,8 +567,6 @@ flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, v
 // kernel layer (unsupported-but-known -> flagcxNotSupported).
 flagcxResult_t screenReduce(int dtype, int op) {
   if (dtype < 0 || dtype >= flagcxNumTypes || op < 0 || op >= flagcxNumRedOps) return flagcxInvalidArgument;
-  if (dtype != flagcxInt32 && dtype != flagcxFloat32 && dtype != flagcxFloat16 && dtype != flagcxBfloat16)
-    return flagcxNotSupported;
   if (op > flagcxMin) return flagcxNotSupported;
   return flagcxSuccess;
 }

@@ -97,7 +97,7 @@ def split(total, parts, idx):
 
 def synth(n, dtype, dist, a, b, seed, stream=0, threads=8):
     """Host array of n synthetic elements (16-bit floats as uint16 bit patterns)."""
-    np_dt = {N.DT_FP64: np.float64}.get(dtype) or N.NP_DTYPE[dtype]
+    np_dt = N.NP_DTYPE[dtype]
     out = np.empty(n, dtype=np_dt)
     N.check(lib.fx_synth_fill(out.ctypes.data, n, dtype, dist, a, b, seed, stream, threads), "fx_synth_fill")
     return out

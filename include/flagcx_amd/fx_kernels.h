@@ -6,8 +6,11 @@
  * 9 = not supported -- callers fall through on 9 exactly as FlagCX does,
  * flagcx/flagcx.cc:2673-2680).  `stream` is a raw hipStream_t (NULL = the
  * default stream); all launches are enqueue-only.  dtype / op are FlagCX enum
- * values (flagcx/include/flagcx.h:36-66): int32 = 2, fp16 = 6, fp32 = 7,
- * bf16 = 9; sum = 0, prod = 1, max = 2, min = 3.
+ * values (flagcx/include/flagcx.h:36-66): int8 = 0, uint8 = 1, int32 = 2,
+ * uint32 = 3, int64 = 4, uint64 = 5, fp16 = 6, fp32 = 7, fp64 = 8, bf16 = 9;
+ * sum = 0, prod = 1, max = 2, min = 3.  All ten types are carried; avg = 4 is
+ * answered with 9.  Integer sum / prod wrap modulo 2^width, as the host loops
+ * of flagcx/service/include/utils.h:664-725 do.
  */
 #ifndef FLAGCX_AMD_FX_KERNELS_H_
 #define FLAGCX_AMD_FX_KERNELS_H_
@@ -29,7 +32,8 @@ extern "C" {
  * tail the reference drops (:383-384) and unaligned buffers it rejects
  * (:633-635).  bf16/fp16 sum/prod accumulate in fp32 and round once.
  * `in` is a host array of k device pointers; out may equal any in[p]
- * (in-place), partial overlap is undefined.  first = 0 is the reference order;
+ * (in-place), partial overlap is undefined.  Pointers must be aligned to the
+ * element size.  first = 0 is the reference order;
  * another value gives the rotated order a ring produces for that chunk.
  */
 int fx_reduce_copy(void *out, const void *const *in, int k, size_t count,

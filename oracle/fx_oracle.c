@@ -15,6 +15,9 @@
  *   oracle_reduce2 sum/min/max on fp32/int32 .. reference KATs
  *       (test/unittest/service/test_reduction_ops.cpp:11-75) + numpy float32 /
  *       int32 arithmetic (independent correctly-rounded implementation).
+ *   the other host types (int8, uint8, uint32, int64, uint64, fp64) ....
+ *       numpy arithmetic of the same width (wrapping integers, IEEE double),
+ *       extreme values and ties included.
  *   oracle_reduce_copy order ................... brute force over parenthesis-
  *       ations on non-associative tuples + numpy left fold.
  *   bf16 / fp16 widening and rounding ......... exhaustive tables against
@@ -42,7 +45,10 @@
 #endif
 
 /* FlagCX enum values (include/flagcx.h:36-66). */
-enum { DT_INT32 = 2, DT_FP16 = 6, DT_FP32 = 7, DT_BF16 = 9 };
+enum {
+  DT_INT8 = 0, DT_UINT8 = 1, DT_INT32 = 2, DT_UINT32 = 3, DT_INT64 = 4, DT_UINT64 = 5,
+  DT_FP16 = 6, DT_FP32 = 7, DT_FP64 = 8, DT_BF16 = 9
+};
 enum { OP_SUM = 0, OP_PROD = 1, OP_MAX = 2, OP_MIN = 3 };
 enum { RC_OK = 0, RC_INVALID = 4, RC_UNSUPPORTED = 9 };
 
@@ -53,14 +59,13 @@ static int g_threads = 1;
 void oracle_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
 int oracle_get_threads(void) { return g_threads; }
 
-/* flagcx.cc:35-66 (getFlagcxDataTypeSize), restricted to the four types of
- * the device path. */
+/* flagcx.cc:35-66 (getFlagcxDataTypeSize). */
 size_t oracle_dtype_size(int dtype) {
   switch (dtype) {
-    case DT_INT32: return 4;
-    case DT_FP32: return 4;
-    case DT_FP16: return 2;
-    case DT_BF16: return 2;
+    case DT_INT8: case DT_UINT8: return 1;
+    case DT_FP16: case DT_BF16: return 2;
+    case DT_INT32: case DT_UINT32: case DT_FP32: return 4;
+    case DT_INT64: case DT_UINT64: case DT_FP64: return 8;
     default: return 0;
   }
 }
@@ -158,6 +163,42 @@ static inline int32_t op_i32(int32_t a, int32_t b, int op) {
   }
 }
 
+/*
+ * The remaining element types of the host dispatch (utils.h:664-695): char
+ * (signed on x86-64), unsigned char, uint32_t, int64_t, uint64_t, double.
+ * T is the element type, W the unsigned type of the same width in which sum
+ * and prod are computed so that they wrap instead of overflowing; for char the
+ * reference's int promotion followed by the narrowing store gives the same
+ * modulo-256 value.  max/min compare as T.
+ */
+#define ORACLE_INT_LOOP(T, W)                                                  \
+  do {                                                                         \
+    T *o = (T *)out;                                                           \
+    _Pragma("omp parallel for num_threads(nt) schedule(static) if (nt > 1)")   \
+    for (long long i = 0; i < n; i++) {                                        \
+      T acc = ((const T *)in[first])[i];                                       \
+      for (int j = 1; j < k; j++) {                                            \
+        T x = ((const T *)in[(first + j) % k])[i];                             \
+        switch (op) {                                                          \
+          case OP_SUM: acc = (T)(W)((W)acc + (W)x); break;                     \
+          case OP_PROD: acc = (T)(W)((W)acc * (W)x); break;                    \
+          case OP_MAX: acc = (acc < x) ? x : acc; break;                       \
+          default: acc = (x < acc) ? x : acc; break;                           \
+        }                                                                      \
+      }                                                                        \
+      o[i] = acc;                                                              \
+    }                                                                          \
+  } while (0)
+
+static inline double op_f64(double a, double b, int op) {
+  switch (op) {
+    case OP_SUM: return a + b;
+    case OP_PROD: return a * b;
+    case OP_MAX: return (a < b) ? b : a;
+    default: return (b < a) ? b : a;
+  }
+}
+
 static int check_args(int dtype, int op) {
   if (oracle_dtype_size(dtype) == 0) return RC_INVALID; /* utils.h:690-694 */
   if (op < OP_SUM || op > OP_MIN) return RC_INVALID;    /* bootstrap.cc:872-874 */
@@ -195,6 +236,25 @@ int oracle_reduce_copy(void *out, const void *const *in, int k, size_t count,
       int32_t acc = ((const int32_t *)in[first])[i];
       for (int j = 1; j < k; j++)
         acc = op_i32(acc, ((const int32_t *)in[(first + j) % k])[i], op);
+      o[i] = acc;
+    }
+  } else if (dtype == DT_INT8) {
+    ORACLE_INT_LOOP(int8_t, uint8_t);
+  } else if (dtype == DT_UINT8) {
+    ORACLE_INT_LOOP(uint8_t, uint8_t);
+  } else if (dtype == DT_UINT32) {
+    ORACLE_INT_LOOP(uint32_t, uint32_t);
+  } else if (dtype == DT_INT64) {
+    ORACLE_INT_LOOP(int64_t, uint64_t);
+  } else if (dtype == DT_UINT64) {
+    ORACLE_INT_LOOP(uint64_t, uint64_t);
+  } else if (dtype == DT_FP64) {
+    double *o = (double *)out;
+#pragma omp parallel for num_threads(nt) schedule(static) if (nt > 1)
+    for (long long i = 0; i < n; i++) {
+      double acc = ((const double *)in[first])[i];
+      for (int j = 1; j < k; j++)
+        acc = op_f64(acc, ((const double *)in[(first + j) % k])[i], op);
       o[i] = acc;
     }
   } else {

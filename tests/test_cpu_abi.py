@@ -190,9 +190,9 @@ def test_argument_screening_needs_no_gpu():
     p = 0x1000
     rc = lambda **kw: K.reduce_copy(kw.get("out", p), kw.get("ins", [p, p]), kw.get("n", 4), kw.get("dtype", N.DT_FP32),
                                     kw.get("op", N.OP_SUM), kw.get("first", 0))
-    assert rc(dtype=N.DT_FP64) == N.NOT_SUPPORTED
-    assert rc(dtype=N.DT_UINT8) == N.NOT_SUPPORTED
     assert rc(op=N.OP_AVG) == N.NOT_SUPPORTED
+    assert rc(dtype=N.DT_FP64, op=N.OP_AVG) == N.NOT_SUPPORTED
+    assert rc(dtype=N.DT_INT64, out=p + 4) == N.INVALID_ARGUMENT      # 8-byte elements need 8-byte alignment
     assert rc(dtype=10) == N.INVALID_ARGUMENT and rc(dtype=-1) == N.INVALID_ARGUMENT
     assert rc(op=5) == N.INVALID_ARGUMENT
     assert rc(first=2) == N.INVALID_ARGUMENT and rc(first=-1) == N.INVALID_ARGUMENT
@@ -211,7 +211,7 @@ def test_argument_screening_needs_no_gpu():
     assert N.lib.fxSimCommInitAll(None, 2) == N.INVALID_ARGUMENT
     comms = (C.c_void_p * 2)()
     assert N.lib.fxSimCommInitAll(comms, 0) == N.INVALID_ARGUMENT
-    assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP64, N.OP_SUM, None, None) == N.NOT_SUPPORTED
+    assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP64, N.OP_AVG, None, None) == N.NOT_SUPPORTED
     assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, None, None) == N.INVALID_ARGUMENT
 
 

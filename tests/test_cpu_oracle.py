@@ -222,9 +222,72 @@ def test_host_ring_passes_equal_kway_for_exact_types():
 
 def test_unsupported_arguments_are_rejected():
     a = np.zeros(4, np.float32)
-    for dtype, op in ((8, SUM), (0, SUM), (F32, 4), (F32, -1)):   # fp64 / int8 / avg: utils.h:690-694, bootstrap.cc:872-874
+    for dtype, op in ((10, SUM), (-1, SUM), (F32, 4), (F32, -1)):   # outside the enum / avg: bootstrap.cc:872-874
         with pytest.raises(ValueError):
             O.reduce2(a, a, dtype, op)
+
+
+# ---- the other element types of the host dispatch (utils.h:664-695) --------------------------
+_HOST_INTS = {0: np.int8, 1: np.uint8, 3: np.uint32, 4: np.int64, 5: np.uint64}
+
+
+@pytest.mark.parametrize("dtype", sorted(_HOST_INTS))
+def test_host_integer_types_match_numpy_of_the_same_width(dtype):
+    """numpy's fixed-width integer arrays wrap on overflow like the C loops do;
+    extremes and equal values are planted so that wrap and ties are exercised."""
+    t = np.dtype(_HOST_INTS[dtype])
+    lo, hi = np.iinfo(t).min, np.iinfo(t).max
+    rng = np.random.default_rng(dtype)
+    for k in (1, 2, 3, 8):
+        ins = [rng.integers(lo, hi, 4000, dtype=t, endpoint=True) for _ in range(k)]
+        for a in ins:
+            a[:4] = [hi, lo, hi, 0]
+        ins[-1][4:8] = ins[0][4:8]
+        with np.errstate(over="ignore"):
+            want = {SUM: ins[0].copy(), PROD: ins[0].copy(), MAX: ins[0].copy(), MIN: ins[0].copy()}
+            for x in ins[1:]:
+                want[SUM] = (want[SUM] + x).astype(t)
+                want[PROD] = (want[PROD] * x).astype(t)
+                want[MAX] = np.maximum(want[MAX], x)
+                want[MIN] = np.minimum(want[MIN], x)
+        for op in (SUM, PROD, MAX, MIN):
+            assert np.array_equal(O.reduce_copy(ins, dtype, op), want[op]), (dtype, k, op)
+    # closed forms: hi + 1 wraps to lo; 2^(bits-1) * 2 wraps to 0; big-int arithmetic modulo 2^bits
+    one, top = np.array([1], t), np.array([hi], t)
+    assert O.reduce_copy([top, one], dtype, SUM)[0] == lo
+    bits = 8 * t.itemsize
+    vals = [int(x) for x in rng.integers(lo, hi, 5, dtype=t, endpoint=True)]
+    p = 1
+    for v in vals:
+        p *= v
+    p %= 1 << bits
+    if lo < 0 and p >= 1 << (bits - 1):
+        p -= 1 << bits
+    assert int(O.reduce_copy([np.array([v], t) for v in vals], dtype, PROD)[0]) == p
+
+
+def test_fp64_left_fold_matches_numpy():
+    rng = np.random.default_rng(8)
+    for k in (1, 2, 5, 8):
+        ins = [rng.uniform(-1, 1, 3000) * 10.0 ** rng.integers(-20, 20, 3000) for _ in range(k)]
+        ins[0][:4] = [0.0, -0.0, np.nan, 1.0]
+        if k > 1:
+            ins[1][:4] = [-0.0, 0.0, 1.0, np.nan]
+        acc = {op: ins[0].copy() for op in (SUM, PROD, MAX, MIN)}
+        with np.errstate(all="ignore"):
+            for x in ins[1:]:
+                acc[SUM] = acc[SUM] + x
+                acc[PROD] = acc[PROD] * x
+                acc[MAX] = np.where(acc[MAX] < x, x, acc[MAX])
+                acc[MIN] = np.where(x < acc[MIN], x, acc[MIN])
+            for op in (SUM, PROD, MAX, MIN):
+                got = O.reduce_copy(ins, 8, op)
+                nan = np.isnan(acc[op])
+                assert np.array_equal(np.isnan(got), nan)
+                assert np.array_equal(got.view(np.uint64)[~nan], acc[op].view(np.uint64)[~nan]), (k, op)
+    # order: a triple whose left fold differs from the right fold in double precision
+    a, b, c = np.array([1e16]), np.array([1.0]), np.array([-1e16])
+    assert O.reduce_copy([a, b, c], 8, SUM)[0] == 0.0 and O.reduce_copy([a, c, b], 8, SUM)[0] == 1.0
 
 
 # ---- partition arithmetic ------------------------------------------------------------------

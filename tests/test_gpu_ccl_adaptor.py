@@ -117,7 +117,7 @@ def test_reducing_collectives_closed_forms(dev, ccl, stream):
         wantb = O.reduce_copy(bf, N.DT_BF16, N.OP_SUM)
         for r in (0, 7):
             assert np.array_equal(dev.to_host(dr[r], 300001, np.uint16), wantb)
-        assert ccl.allReduce(ds[0], dr[0], count, N.DT_FP64, N.OP_SUM, comms[0], stream) == N.NOT_SUPPORTED
+        assert ccl.allReduce(ds[0], dr[0], count, N.DT_FP32, N.OP_AVG, comms[0], stream) == N.NOT_SUPPORTED
     destroy(ccl, comms)
 
 

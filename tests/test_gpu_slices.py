@@ -95,7 +95,7 @@ def test_triggers_ring_step_semantics(dev):
         assert_parity(dev.to_host(di[0], n, np.int32), O.reduce2(i[0], i[1], N.DT_INT32, N.OP_PROD), N.DT_INT32,
                       N.OP_PROD)
         assert_parity(dev.to_host(dh[0], n, np.uint16), O.reduce2(h[0], h[1], N.DT_FP16, N.OP_MAX), N.DT_FP16, N.OP_MAX)
-        bad = [K.make_trigger(df[0], df[1], df[0], 4, 32, N.DT_FP64, N.OP_SUM)]
+        bad = [K.make_trigger(df[0], df[1], df[0], 4, 32, N.DT_FP32, N.OP_AVG)]
         assert K.reduce_triggers(bad) == N.NOT_SUPPORTED
 
 
@@ -104,7 +104,7 @@ def test_reduce2_all_types(dev):
         a, c = seeded_inputs(dtype, 2, 12345, seed=9)
         for op in OPS.values():
             with DevBufs(dev) as b:
-                da, dc, do = b.put(a), b.put(c), b.alloc(12345 * 4)
+                da, dc, do = b.put(a), b.put(c), b.alloc(12345 * N.DTYPE_SIZE[dtype])
                 N.check(K.reduce2(do, da, dc, 12345, dtype, op), "fx_reduce2")
                 dev.sync()
                 got = dev.to_host(do, 12345, N.NP_DTYPE[dtype])

@@ -4,16 +4,27 @@ import numpy as np
 from flagcx_amd import _native as N
 from flagcx_amd import kernels as K
 
-DTYPES = {"fp32": N.DT_FP32, "int32": N.DT_INT32, "bf16": N.DT_BF16, "fp16": N.DT_FP16}
+DTYPES = {"fp32": N.DT_FP32, "int32": N.DT_INT32, "bf16": N.DT_BF16, "fp16": N.DT_FP16,
+          "uint32": N.DT_UINT32, "int8": N.DT_INT8, "uint8": N.DT_UINT8, "int64": N.DT_INT64, "uint64": N.DT_UINT64,
+          "fp64": N.DT_FP64}
 OPS = {"sum": N.OP_SUM, "prod": N.OP_PROD, "max": N.OP_MAX, "min": N.OP_MIN}
 
 
 def seeded_inputs(dtype, k, n, seed, dist=None):
     """k host arrays of n elements in the distribution BASELINE's configs name
-    for the type: fp32 uniform[-1,1), 16-bit N(0,1), int32 uniform[-2^20,2^20]."""
+    for the type: fp32 uniform[-1,1), 16-bit N(0,1), int32 uniform[-2^20,2^20].
+    The other host types of the reference (8/64-bit and unsigned integers over
+    their whole range so that sums and products wrap, fp64 uniform[-1,1)) come
+    from numpy's seeded generator."""
     out = []
     for p in range(k):
-        if dtype == N.DT_FP32:
+        if dtype in (N.DT_INT8, N.DT_UINT8, N.DT_UINT32, N.DT_INT64, N.DT_UINT64):
+            t = np.dtype(N.NP_DTYPE[dtype])
+            rng = np.random.default_rng([seed, p, dtype])
+            out.append(rng.integers(np.iinfo(t).min, np.iinfo(t).max, n, dtype=t, endpoint=True))
+        elif dtype == N.DT_FP64:
+            out.append(np.random.default_rng([seed, p, dtype]).uniform(-1.0, 1.0, n))
+        elif dtype == N.DT_FP32:
             out.append(K.synth(n, dtype, K.SYNTH_UNIFORM, -1.0, 1.0, seed, p))
         elif dtype == N.DT_INT32:
             out.append(K.synth(n, dtype, K.SYNTH_UNIFORM_INT, -(1 << 20), 1 << 20, seed, p))
@@ -55,7 +66,7 @@ def assert_parity(got, want, dtype, op, what=""):
 
 
 def _uint(a):
-    return {2: np.uint16, 4: np.uint32}[a.itemsize]
+    return {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.itemsize]
 
 
 class DevBufs:

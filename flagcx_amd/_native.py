@@ -101,6 +101,12 @@ _SIGS.update({
     "fxSimCommInitRank": (_i, [C.POINTER(_vp), _i, _vp, _sz, _i]),
     "fxSimCommDestroy": (_i, [_vp]),
     "fxSimCommDevice": (_i, [_vp, C.POINTER(_i)]),
+    "flagcxGetVersion": (_i, [C.POINTER(_i)]),
+    "flagcxGetUniqueId": (_i, [_vp]),
+    "flagcxCommInitRank": (_i, [C.POINTER(_vp), _i, _vp, _i]),
+    "flagcxCommDestroy": (_i, [_vp]),
+    "flagcxGetErrorString": (C.c_char_p, [_i]),
+    "flagcxBarrier": (_i, [_vp, _vp]),
     "flagcxGather": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
     "flagcxScatter": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
     "flagcxBroadcast": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),

@@ -214,37 +214,39 @@ int fx_reduce_slices(const fxSliceDesc *slices, size_t n, int k, int dtype, int 
   if (k < 1 || k > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
   if (n == 0) return flagcxSuccess;
   if (!slices) return flagcxInvalidArgument;
-  return launchSliceBatches(setFor(dtype, op), slices, n, k, (hipStream_t)stream);
+  return guarded([&] { return (int)launchSliceBatches(setFor(dtype, op), slices, n, k, (hipStream_t)stream); });
 }
 
 int fx_reduce_triggers(const fxReduceTrigger *triggers, size_t n, void *stream) {
   if (n == 0) return flagcxSuccess;
   if (!triggers) return flagcxInvalidArgument;
-  std::vector<fxSliceDesc> run;
-  size_t i = 0;
-  while (i < n) {
-    int dtype, op;
-    fx_trigger_get(&triggers[i], nullptr, nullptr, nullptr, nullptr, nullptr, &dtype, &op, nullptr);
-    run.clear();
-    size_t j = i;
-    for (; j < n; j++) {
-      uint64_t a, b, o, c;
-      int dt, rop;
-      fx_trigger_get(&triggers[j], &a, &b, &o, &c, nullptr, &dt, &rop, nullptr);
-      if (dt != dtype || rop != op) break;
-      fxSliceDesc d;
-      memset(&d, 0, sizeof(d));
-      d.in[0] = (const void *)(uintptr_t)a;
-      d.in[1] = (const void *)(uintptr_t)b;
-      d.out = (void *)(uintptr_t)o;
-      d.count = c;
-      run.push_back(d);
+  return guarded([&]() -> int {
+    std::vector<fxSliceDesc> run;
+    size_t i = 0;
+    while (i < n) {
+      int dtype, op;
+      fx_trigger_get(&triggers[i], nullptr, nullptr, nullptr, nullptr, nullptr, &dtype, &op, nullptr);
+      run.clear();
+      size_t j = i;
+      for (; j < n; j++) {
+        uint64_t a, b, o, c;
+        int dt, rop;
+        fx_trigger_get(&triggers[j], &a, &b, &o, &c, nullptr, &dt, &rop, nullptr);
+        if (dt != dtype || rop != op) break;
+        fxSliceDesc d;
+        memset(&d, 0, sizeof(d));
+        d.in[0] = (const void *)(uintptr_t)a;
+        d.in[1] = (const void *)(uintptr_t)b;
+        d.out = (void *)(uintptr_t)o;
+        d.count = c;
+        run.push_back(d);
+      }
+      int rc = fx_reduce_slices(run.data(), run.size(), 2, dtype, op, stream);
+      if (rc != flagcxSuccess) return rc;
+      i = j;
     }
-    int rc = fx_reduce_slices(run.data(), run.size(), 2, dtype, op, stream);
-    if (rc != flagcxSuccess) return rc;
-    i = j;
-  }
-  return flagcxSuccess;
+    return flagcxSuccess;
+  });
 }
 
 int fx_copy_slices(const fxSliceDesc *slices, size_t n, void *stream) {
@@ -252,10 +254,12 @@ int fx_copy_slices(const fxSliceDesc *slices, size_t n, void *stream) {
   if (!slices) return flagcxInvalidArgument;
   for (size_t i = 0; i < n; i++)
     if (slices[i].count && (!slices[i].in[0] || !slices[i].out)) return flagcxInvalidArgument;
-  const int es = copyGranularity(slices, n);
-  std::vector<fxSliceDesc> el(slices, slices + n);
-  for (auto &d : el) d.count /= (uint64_t)es;
-  return launchSliceBatches(copySetFor(es), el.data(), n, 1, (hipStream_t)stream);
+  return guarded([&]() -> int {
+    const int es = copyGranularity(slices, n);
+    std::vector<fxSliceDesc> el(slices, slices + n);
+    for (auto &d : el) d.count /= (uint64_t)es;
+    return launchSliceBatches(copySetFor(es), el.data(), n, 1, (hipStream_t)stream);
+  });
 }
 
 int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, int dtype, int op) {
@@ -263,66 +267,68 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
   *plan = nullptr;
   if (n && !slices) return flagcxInvalidArgument;
   if (n > 0x7fffffffull) return flagcxInvalidArgument;
-  const KernelSet *ks;
-  uint64_t div = 1;
-  if (op == -1) {
-    k = 1;
-    for (size_t i = 0; i < n; i++)
-      if (slices[i].count && (!slices[i].in[0] || !slices[i].out)) return flagcxInvalidArgument;
-    int es = copyGranularity(slices, n);
-    ks = copySetFor(es);
-    div = (uint64_t)es;
-  } else {
-    flagcxResult_t rc = screen(dtype, op);
-    if (rc != flagcxSuccess) return rc;
-    if (k < 1 || k > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
-    ks = setFor(dtype, op);
-  }
-  const int U = unrollFor(k);
-  std::vector<SliceDescDev> desc;
-  std::vector<uint32_t> start(1, 0u);
-  std::vector<fxSliceDesc> scaled(slices, slices + n);
-  for (auto &d : scaled) {
-    if (d.count && !d.out) return flagcxInvalidArgument;
-    for (int p = 0; p < k; p++)
-      if (d.count && !d.in[p]) return flagcxInvalidArgument;
-    d.count /= div;
-  }
-  const std::vector<fxSliceDesc> merged = mergeAdjacent(scaled.data(), scaled.size(), k, (size_t)ks->elemSize);
-  for (size_t i = 0; i < merged.size(); i++) {
-    fxSliceDesc s = merged[i];
-    uint64_t tiles;
-    flagcxResult_t rc = sliceTiles(s, k, ks->elemSize, U, &tiles);
-    if (rc != flagcxSuccess) return rc;
-    if (tiles == 0) continue;
-    if ((uint64_t)start.back() + tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
-    SliceDescDev d;
-    for (int p = 0; p < kMaxFixedK; p++) d.in[p] = (p < k) ? s.in[p] : nullptr;
-    d.out = s.out;
-    d.count = s.count;
-    desc.push_back(d);
-    start.push_back(start.back() + (uint32_t)tiles);
-  }
-  fxPlan *pl = new (std::nothrow) fxPlan();
-  if (!pl) return flagcxSystemError;
-  pl->ks = ks;
-  pl->k = k;
-  pl->n = (uint32_t)desc.size();
-  pl->grid = start.back();
-  pl->dDesc = nullptr;
-  pl->dTileStart = nullptr;
-  if (pl->n) {
-    if (hipMalloc((void **)&pl->dDesc, desc.size() * sizeof(SliceDescDev)) != hipSuccess ||
-        hipMalloc((void **)&pl->dTileStart, start.size() * sizeof(uint32_t)) != hipSuccess ||
-        hipMemcpy(pl->dDesc, desc.data(), desc.size() * sizeof(SliceDescDev), hipMemcpyHostToDevice) != hipSuccess ||
-        hipMemcpy(pl->dTileStart, start.data(), start.size() * sizeof(uint32_t), hipMemcpyHostToDevice) !=
-            hipSuccess) {
-      fx_plan_destroy(pl);
-      return flagcxUnhandledDeviceError;
+  return guarded([&]() -> int {
+    const KernelSet *ks;
+    uint64_t div = 1;
+    if (op == -1) {
+      k = 1;
+      for (size_t i = 0; i < n; i++)
+        if (slices[i].count && (!slices[i].in[0] || !slices[i].out)) return flagcxInvalidArgument;
+      int es = copyGranularity(slices, n);
+      ks = copySetFor(es);
+      div = (uint64_t)es;
+    } else {
+      flagcxResult_t rc = screen(dtype, op);
+      if (rc != flagcxSuccess) return rc;
+      if (k < 1 || k > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
+      ks = setFor(dtype, op);
     }
-  }
-  *plan = pl;
-  return flagcxSuccess;
+    const int U = unrollFor(k);
+    std::vector<SliceDescDev> desc;
+    std::vector<uint32_t> start(1, 0u);
+    std::vector<fxSliceDesc> scaled(slices, slices + n);
+    for (auto &d : scaled) {
+      if (d.count && !d.out) return flagcxInvalidArgument;
+      for (int p = 0; p < k; p++)
+        if (d.count && !d.in[p]) return flagcxInvalidArgument;
+      d.count /= div;
+    }
+    const std::vector<fxSliceDesc> merged = mergeAdjacent(scaled.data(), scaled.size(), k, (size_t)ks->elemSize);
+    for (size_t i = 0; i < merged.size(); i++) {
+      fxSliceDesc s = merged[i];
+      uint64_t tiles;
+      flagcxResult_t rc = sliceTiles(s, k, ks->elemSize, U, &tiles);
+      if (rc != flagcxSuccess) return rc;
+      if (tiles == 0) continue;
+      if ((uint64_t)start.back() + tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+      SliceDescDev d;
+      for (int p = 0; p < kMaxFixedK; p++) d.in[p] = (p < k) ? s.in[p] : nullptr;
+      d.out = s.out;
+      d.count = s.count;
+      desc.push_back(d);
+      start.push_back(start.back() + (uint32_t)tiles);
+    }
+    fxPlan *pl = new (std::nothrow) fxPlan();
+    if (!pl) return flagcxSystemError;
+    pl->ks = ks;
+    pl->k = k;
+    pl->n = (uint32_t)desc.size();
+    pl->grid = start.back();
+    pl->dDesc = nullptr;
+    pl->dTileStart = nullptr;
+    if (pl->n) {
+      if (hipMalloc((void **)&pl->dDesc, desc.size() * sizeof(SliceDescDev)) != hipSuccess ||
+          hipMalloc((void **)&pl->dTileStart, start.size() * sizeof(uint32_t)) != hipSuccess ||
+          hipMemcpy(pl->dDesc, desc.data(), desc.size() * sizeof(SliceDescDev), hipMemcpyHostToDevice) != hipSuccess ||
+          hipMemcpy(pl->dTileStart, start.data(), start.size() * sizeof(uint32_t), hipMemcpyHostToDevice) !=
+              hipSuccess) {
+        fx_plan_destroy(pl);
+        return flagcxUnhandledDeviceError;
+      }
+    }
+    *plan = pl;
+    return flagcxSuccess;
+  });
 }
 
 int fx_plan_launch(fxPlan_t plan, void *stream) {
@@ -346,26 +352,28 @@ static int packOrUnpack(bool pack, void *a, const void *b, const size_t *counts,
   if (es == 0) return flagcxInvalidArgument;
   if (npeers == 0) return flagcxSuccess;
   if (!counts || !displs) return flagcxInvalidArgument;
-  std::vector<fxSliceDesc> sl;
-  size_t slot = 0;
-  for (int i = 0; i < npeers; i++) {
-    if (counts[i]) {
-      if (!a || !b) return flagcxInvalidArgument;
-      fxSliceDesc d;
-      memset(&d, 0, sizeof(d));
-      if (pack) {  // a = packed, b = sendbuff
-        d.in[0] = (const char *)b + displs[i] * es;
-        d.out = (char *)a + slot * es;
-      } else {     // a = recvbuff, b = packed
-        d.in[0] = (const char *)b + slot * es;
-        d.out = (char *)a + displs[i] * es;
+  return guarded([&]() -> int {
+    std::vector<fxSliceDesc> sl;
+    size_t slot = 0;
+    for (int i = 0; i < npeers; i++) {
+      if (counts[i]) {
+        if (!a || !b) return flagcxInvalidArgument;
+        fxSliceDesc d;
+        memset(&d, 0, sizeof(d));
+        if (pack) {  // a = packed, b = sendbuff
+          d.in[0] = (const char *)b + displs[i] * es;
+          d.out = (char *)a + slot * es;
+        } else {     // a = recvbuff, b = packed
+          d.in[0] = (const char *)b + slot * es;
+          d.out = (char *)a + displs[i] * es;
+        }
+        d.count = counts[i] * es;
+        sl.push_back(d);
       }
-      d.count = counts[i] * es;
-      sl.push_back(d);
+      slot += counts[i];
     }
-    slot += counts[i];
-  }
-  return fx_copy_slices(sl.data(), sl.size(), stream);
+    return fx_copy_slices(sl.data(), sl.size(), stream);
+  });
 }
 
 int fx_pack(void *packed, const void *sendbuff, const size_t *sendcounts, const size_t *sdispls, int npeers,

@@ -47,21 +47,7 @@ flagcxResult_t cclGetUniqueId(flagcxInnerUniqueId_t *uniqueId) {
   return flagcxSuccess;
 }
 
-const char *cclGetErrorString(flagcxResult_t r) {
-  switch (r) {
-    case flagcxSuccess: return "no error";
-    case flagcxUnhandledDeviceError: return "unhandled device error";
-    case flagcxSystemError: return "unhandled system error";
-    case flagcxInternalError: return "internal error";
-    case flagcxInvalidArgument: return "invalid argument";
-    case flagcxInvalidUsage: return "invalid usage";
-    case flagcxRemoteError: return "remote process exited or there was a network error";
-    case flagcxInProgress: return "operation in progress";
-    case flagcxUnhandledCCLError: return "unhandled ccl error";
-    case flagcxNotSupported: return "not supported";
-    default: return "unknown result code";
-  }
-}
+const char *cclGetErrorString(flagcxResult_t r) { return flagcxGetErrorString(r); }
 
 const char *cclGetLastError(flagcxInnerComm_t) { return ""; }
 

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <new>
 
 #include "flagcx_amd/fx_types.h"
 
@@ -37,6 +38,19 @@ inline bool opSupported(int op) { return op >= flagcxSum && op <= flagcxMin; }
     hipError_t e_ = (call);                                                    \
     if (e_ != hipSuccess) return flagcxUnhandledDeviceError;                   \
   } while (0)
+
+// No C++ exception may cross the C ABI: host entry points that allocate run
+// their body through this.
+template <class F>
+inline int guarded(F body) noexcept {
+  try {
+    return body();
+  } catch (const std::bad_alloc &) {
+    return flagcxSystemError;
+  } catch (...) {
+    return flagcxInternalError;
+  }
+}
 
 // 128-bit streaming accesses: every byte is touched once, so keep it out of
 // the caches' way (nontemporal).

@@ -90,6 +90,12 @@ __device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b,
   }
 }
 
+// Clears the mirror before a consumer launch.  A kernel rather than a memset
+// node so that the launch sequence stays safe to record into a HIP graph.
+__global__ void __launch_bounds__(kBlock) clearMirror(uint64_t *words, uint32_t n) {
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += gridDim.x * kBlock) words[i] = 0;
+}
+
 __global__ void __launch_bounds__(kBlock)
 fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uint64_t maxIdlePolls) {
   __shared__ uint64_t sh[6];  // [0] state, [1..4] trigger words, [5] scratch
@@ -290,7 +296,10 @@ int fx_fifo_consumer_launch(fxFifoConsumer_t c, void *fifoDevicePointer, const u
   if (!c || !fifoDevicePointer || !fifoHost || maxIdlePolls == 0) return flagcxInvalidArgument;
   if (fifoHost[0] != c->capacity) return flagcxInvalidArgument;
   hipStream_t s = (hipStream_t)stream;
-  FX_HIP(hipMemsetAsync(c->mirror, 0, sizeof(FifoMirror), s));
+  static_assert(sizeof(FifoMirror) % sizeof(uint64_t) == 0, "FifoMirror is cleared in 8-byte words");
+  const uint32_t words = (uint32_t)(sizeof(FifoMirror) / sizeof(uint64_t));
+  hipLaunchKernelGGL(clearMirror, dim3((words + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (uint64_t *)c->mirror, words);
+  FX_HIP(hipGetLastError());
   const uint64_t startSeq = fifoHost[2];  // triggers produced before this launch are not ours
   hipLaunchKernelGGL(fifoConsumer, dim3(c->grid), dim3(kBlock), 0, s, (uint64_t *)fifoDevicePointer, c->mirror,
                      c->capacity, startSeq, (uint64_t)maxIdlePolls);

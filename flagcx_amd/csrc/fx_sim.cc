@@ -12,6 +12,8 @@
 // the reference would receive a copy of it.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -22,6 +24,7 @@
 
 #include "flagcx_amd/fx_kernels.h"
 #include "flagcx_amd/fx_sim.h"
+#include "fx_common.hpp"
 
 struct flagcxStream {
   hipStream_t base;
@@ -31,7 +34,7 @@ namespace {
 
 enum Kind {
   kNone = 0, kReduce, kAllReduce, kReduceScatter, kAllGather, kAlltoAllv, kCustomAllReduce,
-  kGather, kScatter, kBroadcast, kAlltoAll
+  kGather, kScatter, kBroadcast, kAlltoAll, kBarrier
 };
 
 struct Post {
@@ -491,9 +494,21 @@ struct flagcxComm {
 
 namespace {
 
+flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *send, void *recv, size_t count, int dtype,
+                                   int op, int root, flagcxStream_t stream, const size_t *sc, const size_t *sd,
+                                   const size_t *rc_, const size_t *rd);
+
 flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, void *recv, size_t count, int dtype,
                                int op, int root, flagcxStream_t stream, const size_t *sc, const size_t *sd,
                                const size_t *rc_, const size_t *rd) {
+  return R(fx::guarded([&]() -> int {
+    return postAndMaybeRunImpl(comm, kind, send, recv, count, dtype, op, root, stream, sc, sd, rc_, rd);
+  }));
+}
+
+flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *send, void *recv, size_t count, int dtype,
+                                   int op, int root, flagcxStream_t stream, const size_t *sc, const size_t *sd,
+                                   const size_t *rc_, const size_t *rd) {
   if (!comm || !comm->g || !stream) return flagcxInvalidArgument;
   Group *g = comm->g;
   const int rank = comm->rank;
@@ -546,6 +561,7 @@ flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, v
       case kScatter: res = runScatter(c); break;
       case kBroadcast: res = runBroadcast(c); break;
       case kAlltoAll: res = runAlltoAll(c); break;
+      case kBarrier: break;  // the event waits around this switch are the barrier
       default: res = flagcxInternalError;
     }
   }
@@ -578,8 +594,13 @@ flagcxResult_t newGroup(int nranks, Group **out) {
   Group *g = new (std::nothrow) Group();
   if (!g) return flagcxSystemError;
   g->n = nranks;
-  g->posts.resize(nranks);
-  g->ready.assign(nranks, nullptr);
+  try {
+    g->posts.resize(nranks);
+    g->ready.assign(nranks, nullptr);
+  } catch (...) {
+    delete g;
+    throw;
+  }
   bool ok = hipGetDevice(&g->device) == hipSuccess;
   ok = ok && hipEventCreateWithFlags(&g->done, hipEventDisableTiming) == hipSuccess;
   for (int r = 0; r < nranks && ok; r++)
@@ -614,8 +635,16 @@ void freeGroup(Group *g) {
 // send / recv between simulated ranks: the later of the two calls performs the
 // copy on its own stream after waiting for the other side's stream, and the
 // other side's stream then waits for the copy.
+flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, void *rbuf, size_t count, int dtype,
+                           int peer, flagcxStream_t stream);
+
 flagcxResult_t postP2p(flagcxComm_t comm, bool isSend, const void *sbuf, void *rbuf, size_t count, int dtype, int peer,
                        flagcxStream_t stream) {
+  return R(fx::guarded([&]() -> int { return postP2pImpl(comm, isSend, sbuf, rbuf, count, dtype, peer, stream); }));
+}
+
+flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, void *rbuf, size_t count, int dtype,
+                           int peer, flagcxStream_t stream) {
   if (!comm || !comm->g || !stream) return flagcxInvalidArgument;
   Group *g = comm->g;
   const size_t ts = fx_dtype_size(dtype);
@@ -672,12 +701,21 @@ extern "C" {
 
 flagcxResult_t fxSimCommInitAll(flagcxComm_t *comms, int nranks) {
   if (!comms || nranks < 1 || nranks > FX_MAX_INPUTS) return flagcxInvalidArgument;
-  Group *g = nullptr;
-  flagcxResult_t rc = newGroup(nranks, &g);
-  if (rc != flagcxSuccess) return rc;
-  g->joined = g->alive = nranks;
-  for (int r = 0; r < nranks; r++) comms[r] = new flagcxComm{g, r};
-  return flagcxSuccess;
+  return R(fx::guarded([&]() -> int {
+    Group *g = nullptr;
+    flagcxResult_t rc = newGroup(nranks, &g);
+    if (rc != flagcxSuccess) return rc;
+    g->joined = g->alive = nranks;
+    int made = 0;
+    for (; made < nranks; made++)
+      if (!(comms[made] = new (std::nothrow) flagcxComm{g, made})) break;
+    if (made < nranks) {
+      for (int r = 0; r < made; r++) delete comms[r];
+      freeGroup(g);
+      return flagcxSystemError;
+    }
+    return flagcxSuccess;
+  }));
 }
 
 flagcxResult_t fxSimCommDestroyAll(flagcxComm_t *comms, int nranks) {
@@ -695,24 +733,40 @@ flagcxResult_t fxSimCommDestroyAll(flagcxComm_t *comms, int nranks) {
 flagcxResult_t fxSimCommInitRank(flagcxComm_t *comm, int nranks, const void *id, size_t idBytes, int rank) {
   if (!comm || !id || idBytes == 0 || nranks < 1 || nranks > FX_MAX_INPUTS || rank < 0 || rank >= nranks)
     return flagcxInvalidArgument;
-  std::lock_guard<std::mutex> lock(gRegistryMu);
-  const std::string key((const char *)id, idBytes);
-  Group *g;
-  auto it = gRegistry.find(key);
-  if (it == gRegistry.end()) {
-    flagcxResult_t rc = newGroup(nranks, &g);
-    if (rc != flagcxSuccess) return rc;
-    g->id = key;
-    gRegistry[key] = g;
-  } else {
-    g = it->second;
-    if (g->n != nranks) return flagcxInvalidArgument;
-  }
-  g->joined++;
-  g->alive++;
-  if (g->joined == nranks) gRegistry.erase(key);  // complete: the id may be reused for a new group
-  *comm = new flagcxComm{g, rank};
-  return flagcxSuccess;
+  return R(fx::guarded([&]() -> int {
+    std::lock_guard<std::mutex> lock(gRegistryMu);
+    const std::string key((const char *)id, idBytes);
+    flagcxComm *c = new flagcxComm{nullptr, rank};
+    Group *g;
+    auto it = gRegistry.find(key);
+    if (it == gRegistry.end()) {
+      flagcxResult_t rc = newGroup(nranks, &g);
+      if (rc != flagcxSuccess) {
+        delete c;
+        return rc;
+      }
+      g->id = key;
+      try {
+        gRegistry[key] = g;
+      } catch (...) {
+        delete c;
+        freeGroup(g);
+        throw;
+      }
+    } else {
+      g = it->second;
+      if (g->n != nranks) {
+        delete c;
+        return flagcxInvalidArgument;
+      }
+    }
+    g->joined++;
+    g->alive++;
+    if (g->joined == nranks) gRegistry.erase(key);  // complete: the id may be reused for a new group
+    c->g = g;
+    *comm = c;
+    return flagcxSuccess;
+  }));
 }
 
 flagcxResult_t fxSimCommDestroy(flagcxComm_t comm) {
@@ -730,6 +784,49 @@ flagcxResult_t fxSimCommDestroy(flagcxComm_t comm) {
   delete comm;
   if (last) freeGroup(g);
   return flagcxSuccess;
+}
+
+flagcxResult_t flagcxGetVersion(int *version) {
+  if (!version) return flagcxInvalidArgument;
+  *version = FX_SIM_VERSION;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxGetUniqueId(flagcxUniqueId_t uniqueId) {
+  if (!uniqueId) return flagcxInvalidArgument;
+  static std::atomic<uint64_t> counter{0};
+  const uint64_t words[3] = {(uint64_t)std::chrono::steady_clock::now().time_since_epoch().count(), ++counter,
+                             (uint64_t)(uintptr_t)&counter};
+  memset(uniqueId->internal, 0, sizeof(uniqueId->internal));
+  memcpy(uniqueId->internal, words, sizeof(words));
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxCommInitRank(flagcxComm_t *comm, int nranks, flagcxUniqueId_t commId, int rank) {
+  if (!commId) return flagcxInvalidArgument;
+  return fxSimCommInitRank(comm, nranks, commId->internal, sizeof(commId->internal), rank);
+}
+
+flagcxResult_t flagcxCommDestroy(flagcxComm_t comm) { return fxSimCommDestroy(comm); }
+
+const char *flagcxGetErrorString(flagcxResult_t result) {
+  switch (result) {
+    case flagcxSuccess: return "no error";
+    case flagcxUnhandledDeviceError: return "unhandled device error";
+    case flagcxSystemError: return "unhandled system error";
+    case flagcxInternalError: return "internal error";
+    case flagcxInvalidArgument: return "invalid argument";
+    case flagcxInvalidUsage: return "invalid usage";
+    case flagcxRemoteError: return "remote process exited or there was a network error";
+    case flagcxInProgress: return "operation in progress";
+    case flagcxUnhandledCCLError: return "unhandled ccl error";
+    case flagcxNotSupported: return "not supported";
+    default: return "unknown result code";
+  }
+}
+
+flagcxResult_t flagcxBarrier(flagcxComm_t comm, flagcxStream_t stream) {
+  return postAndMaybeRun(comm, kBarrier, nullptr, nullptr, 0, 0, 0, 0, stream);
 }
 
 flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
@@ -763,7 +860,7 @@ flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
 }
 
 flagcxResult_t flagcxCommCount(const flagcxComm_t comm, int *count) {
-  if (!comm || !count) return flagcxInvalidArgument;
+  if (!comm || !comm->g || !count) return flagcxInvalidArgument;
   *count = comm->g->n;
   return flagcxSuccess;
 }
@@ -863,7 +960,7 @@ flagcxResult_t flagcxGroupStart(flagcxComm_t) { return flagcxSuccess; }
 flagcxResult_t flagcxGroupEnd(flagcxComm_t) { return flagcxSuccess; }
 
 flagcxResult_t fxSimCommDevice(const flagcxComm_t comm, int *device) {
-  if (!comm || !device) return flagcxInvalidArgument;
+  if (!comm || !comm->g || !device) return flagcxInvalidArgument;
   *device = comm->g->device;
   return flagcxSuccess;
 }
@@ -871,15 +968,17 @@ flagcxResult_t fxSimCommDevice(const flagcxComm_t comm, int *device) {
 flagcxResult_t fxSimRegisterWindows(flagcxComm_t comm, void *const *windows, size_t bytes) {
   if (!comm || !comm->g) return flagcxInvalidArgument;
   Group *g = comm->g;
-  std::lock_guard<std::mutex> lock(g->mu);
-  g->windows.clear();
-  g->windowBytes = 0;
-  if (!windows) return flagcxSuccess;
-  for (int r = 0; r < g->n; r++)
-    if (!windows[r]) return flagcxInvalidArgument;
-  g->windows.assign(windows, windows + g->n);
-  g->windowBytes = bytes;
-  return flagcxSuccess;
+  return R(fx::guarded([&]() -> int {
+    std::lock_guard<std::mutex> lock(g->mu);
+    g->windows.clear();
+    g->windowBytes = 0;
+    if (!windows) return flagcxSuccess;
+    for (int r = 0; r < g->n; r++)
+      if (!windows[r]) return flagcxInvalidArgument;
+    g->windows.assign(windows, windows + g->n);
+    g->windowBytes = bytes;
+    return flagcxSuccess;
+  }));
 }
 
 flagcxResult_t flagcxCustomAllReduceImpl(const void *sendbuff, void *recvbuff, size_t count,
@@ -890,9 +989,13 @@ flagcxResult_t flagcxCustomAllReduceImpl(const void *sendbuff, void *recvbuff, s
   if (rc != flagcxSuccess) return flagcxNotSupported;  // the hook only ever declines
   Group *g = comm->g;
   const size_t bytes = count * fx_dtype_size(datatype);
-  if (g->windows.empty() || bytes > g->windowBytes) return flagcxNotSupported;
+  void *win;
+  {
+    std::lock_guard<std::mutex> lock(g->mu);
+    if (g->windows.empty() || bytes > g->windowBytes) return flagcxNotSupported;
+    win = g->windows[comm->rank];
+  }
   if (count && (!sendbuff || !recvbuff)) return flagcxInvalidArgument;
-  void *win = g->windows[comm->rank];
   if (bytes && sendbuff != win &&
       hipMemcpyAsync(win, sendbuff, bytes, hipMemcpyDeviceToDevice, stream->base) != hipSuccess)
     return flagcxUnhandledDeviceError;

@@ -42,6 +42,28 @@ flagcxResult_t fxSimCommInitRank(flagcxComm_t *comm, int nranks, const void *id,
 flagcxResult_t fxSimCommDestroy(flagcxComm_t comm);
 flagcxResult_t fxSimCommDevice(const flagcxComm_t comm, int *device);
 
+/*
+ * The communicator life cycle under its reference names and signatures
+ * (flagcx/include/flagcx.h:282-321,358), so that a harness written against
+ * libflagcx -- e.g. the ctypes table of plugin/interservice/flagcx_wrapper.py:
+ * 244-330 -- binds to this library unchanged for the calls of this path.
+ * flagcxGetUniqueId fills the 256 bytes with a value unique in the process;
+ * flagcxCommInitRank joins the in-process group carrying that id (no
+ * bootstrap network: all ranks of a group live in one process on one GPU);
+ * flagcxCommDestroy releases one rank.  flagcxGetVersion reports
+ * FX_SIM_VERSION.  flagcxGetErrorString names the code (the reference returns
+ * "Not implemented." for every code, flagcx.cc:1586-1589).  flagcxBarrier makes
+ * every rank's stream wait for all the others'.
+ */
+#define FX_SIM_VERSION 100
+flagcxResult_t flagcxGetVersion(int *version);
+flagcxResult_t flagcxGetUniqueId(flagcxUniqueId_t uniqueId);
+flagcxResult_t flagcxCommInitRank(flagcxComm_t *comm, int nranks,
+                                  flagcxUniqueId_t commId, int rank);
+flagcxResult_t flagcxCommDestroy(flagcxComm_t comm);
+const char *flagcxGetErrorString(flagcxResult_t result);
+flagcxResult_t flagcxBarrier(flagcxComm_t comm, flagcxStream_t stream);
+
 /* Configuration keys (defaults come from the same environment variables the
  * reference reads, flagcx/runner/uni_runner_impl.cc:21-26, uni_runner.cc:10-12). */
 enum {
@@ -117,8 +139,7 @@ flagcxResult_t flagcxGroupEnd(flagcxComm_t comm);
  * registered send windows, in rank order, written to recvbuff.  sendbuff is
  * first staged into this rank's window unless it already is the window.
  * Returns flagcxNotSupported (caller falls through, flagcx.cc:2673-2680) for
- * avg, for types outside {fp16, bf16, fp32, int32}, when no window is
- * registered or when the message exceeds it.  Unlike the reference it accepts
+ * avg, when no window is registered or when the message exceeds it.  Unlike the reference it accepts
  * every op on every type, odd counts and unaligned recvbuff.
  */
 flagcxResult_t flagcxCustomAllReduceImpl(const void *sendbuff, void *recvbuff,

@@ -58,6 +58,13 @@ typedef enum {
   flagcxEventDisableTiming = 1
 } flagcxEventType_t;
 
+/* flagcx/include/flagcx.h:112-116 */
+#define FLAGCX_UNIQUE_ID_BYTES 256
+typedef struct {
+  char internal[FLAGCX_UNIQUE_ID_BYTES];
+} flagcxUniqueId;
+typedef flagcxUniqueId *flagcxUniqueId_t;
+
 typedef struct flagcxComm *flagcxComm_t;
 typedef struct flagcxStream *flagcxStream_t;
 typedef struct flagcxEvent *flagcxEvent_t;

@@ -206,3 +206,57 @@ def test_cfg5_large_bf16_sum(dev, stream):
         N.check(K.reduce_copy(dins[0], dins, n, c["dtype"], N.OP_SUM, 0, raw))
         dev.stream_sync(stream)
         assert W.digest(dev.to_host(dins[0], n, np.uint16)) == gold["out_sha256"], "in-place"
+
+
+@pytest.mark.parametrize("dname,dtype,count", [("int8", N.DT_INT8, (1 << 32) + (3 << 20) + 12345),   # > 2^32 elements
+                                               ("fp32", N.DT_FP32, (1 << 31) + 777)])             # > 2^33 bytes
+def test_counts_beyond_32_bit_offsets(dev, dname, dtype, count):
+    """Maximum sizes: element counts and byte offsets that do not fit 32 bits.
+    Inputs are a byte pattern with seeded random patches planted at the start,
+    across the 2^32-byte boundary and at the end, so that an index truncated to
+    32 bits would read the wrong patch.  The whole output is downloaded and
+    compared piecewise with the oracle; the bytes behind it must be untouched."""
+    es = N.DTYPE_SIZE[dtype]
+    npdt = N.NP_DTYPE[dtype]
+    nbytes = count * es
+    patch_el = (1 << 20) // es
+    starts = sorted({0, ((1 << 32) - (1 << 19)) // es, count - patch_el})          # element offsets of the patches
+    assert all(s + patch_el <= count for s in starts)
+    rng = np.random.default_rng(count % 1000)
+    fill = (0x01, 0x02)
+    with DevBufs(dev) as b:
+        dins, patches = [], []
+        for p in range(2):
+            d = b.alloc(nbytes + 256)
+            dev.memset(d, fill[p], nbytes)
+            mine = {}
+            for s in starts:
+                raw = rng.integers(0, 256, patch_el * es, dtype=np.uint8)
+                if dtype == N.DT_FP32:                                                # finite values only
+                    with np.errstate(all="ignore"):
+                        f = raw.view(np.float32) % np.float32(1e6)
+                    raw = np.nan_to_num(f, nan=1.5).view(np.uint8)
+                mine[s] = raw.view(npdt)
+                dev.upload(d + s * es, mine[s])
+            dins.append(d)
+            patches.append(mine)
+        dout = b.alloc(nbytes + 256)
+        dev.memset(dout, 0xEE, nbytes + 256)
+        N.check(K.reduce_copy(dout, dins, count, dtype, N.OP_SUM), "fx_reduce_copy")
+        dev.sync()
+        base = [np.full(1, f, np.uint8).repeat(es).view(npdt)[0] for f in fill]
+        plain = O.reduce2(np.full(4, base[0], npdt), np.full(4, base[1], npdt), dtype, N.OP_SUM)[0]
+        step = (1 << 28) // es                                                        # 256 MiB per download
+        for off in range(0, count, step):
+            n = min(step, count - off)
+            got = dev.to_host(dout + off * es, n, npdt)
+            want = np.full(n, plain, npdt)
+            for s in starts:
+                lo, hi = max(s, off), min(s + patch_el, off + n)
+                if lo < hi:
+                    a = [np.full(hi - lo, base[p], npdt) for p in range(2)]
+                    for p in range(2):
+                        a[p][:] = patches[p][s][lo - s:hi - s]
+                    want[lo - off:hi - off] = O.reduce2(a[0], a[1], dtype, N.OP_SUM)
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), f"{dname}: window at element {off}"
+        assert (dev.to_host(dout + nbytes, 256, np.uint8) == 0xEE).all(), "wrote past the end"

@@ -179,6 +179,10 @@ class Device:
     def sync(self):
         N.check(self.t.deviceSynchronize(), "deviceSynchronize")
 
+    def set_device(self):
+        """Make this GPU current for the calling host thread."""
+        N.check(self.t.setDevice(self.index), "setDevice")
+
     def event_create(self, timing=True):
         e = _vp()
         N.check(self.t.eventCreate(C.byref(e), 0 if timing else 1), "eventCreate")

@@ -271,3 +271,49 @@ def test_ranks_on_different_streams(dev):
     finally:
         for s in streams:
             dev.stream_destroy(s)
+
+
+def test_one_host_thread_per_rank(dev):
+    """FlagCX applications drive each rank from its own thread on its own stream.
+    Eight threads post 30 all-reduces each (alternating op), never synchronising
+    with one another on the host; every result must equal the oracle's."""
+    import threading
+    n, count, rounds = 8, 100003, 30
+    sends = seeded_inputs(N.DT_FP32, n, count, seed=21)
+    want = {op: O.reduce_copy(sends, N.DT_FP32, op) for op in (N.OP_SUM, N.OP_MAX)}
+    errors = []
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        ds = [b.put(a) for a in sends]
+        dr = [[b.alloc(count * 4) for _ in range(n)] for _ in range(2)]
+        streams = [dev.stream_create() for _ in range(n)]
+
+        def rank_main(r):
+            try:
+                dev.set_device()
+                for it in range(rounds):
+                    op = (N.OP_SUM, N.OP_MAX)[it % 2]
+                    # a collective is matched by arrival order, so a rank may only post round it
+                    # once every rank has posted round it-1: the barrier models the application's own
+                    # per-step structure and involves no device synchronisation
+                    gate.wait()
+                    rc = N.lib.flagcxAllReduce(ds[r], dr[it % 2][r], count, N.DT_FP32, op, g.comms[r], streams[r])
+                    if rc != N.SUCCESS:
+                        errors.append((r, it, rc))
+                dev.stream_sync(streams[r])
+            except Exception as e:                      # noqa: BLE001 - reported below
+                errors.append((r, repr(e)))
+                gate.abort()
+
+        gate = threading.Barrier(n)
+        threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=60)
+        assert not errors, errors
+        assert not any(t.is_alive() for t in threads)
+        for r in range(n):
+            assert_parity(dev.to_host(dr[1][r], count, np.float32), want[N.OP_MAX], N.DT_FP32, N.OP_MAX, f"rank {r}")
+            assert_parity(dev.to_host(dr[0][r], count, np.float32), want[N.OP_SUM], N.DT_FP32, N.OP_SUM, f"rank {r}")
+        for s in streams:
+            dev.stream_destroy(s)

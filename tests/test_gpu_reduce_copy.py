@@ -199,3 +199,39 @@ def test_error_paths(dev):
         dev.sync()
     finally:
         dev.free(p)
+
+
+def test_concurrent_host_threads(dev):
+    """The C ABI is enqueue-only and thread-safe: four host threads launch on
+    their own streams at the same time (ctypes drops the GIL around each call)."""
+    import threading
+    jobs = [(N.DT_BF16, N.OP_SUM, 8, 300007), (N.DT_FP32, N.OP_MAX, 3, 70001), (N.DT_INT64, N.OP_PROD, 2, 65537),
+            (N.DT_UINT8, N.OP_SUM, 5, 1 << 20)]
+    errors, results = [], {}
+    with DevBufs(dev) as b:
+        prepared = []
+        for dtype, op, k, n in jobs:
+            ins = seeded_inputs(dtype, k, n, seed=k)
+            prepared.append((dtype, op, n, ins, [b.put(a) for a in ins], b.alloc(n * N.DTYPE_SIZE[dtype])))
+
+        def work(i):
+            try:
+                dev.set_device()
+                dtype, op, n, _, dins, dout = prepared[i]
+                s = dev.stream_create()
+                for _ in range(50):
+                    N.check(K.reduce_copy(dout, dins, n, dtype, op, 0, dev.raw_stream(s)), "fx_reduce_copy")
+                dev.stream_sync(s)
+                results[i] = dev.to_host(dout, n, N.NP_DTYPE[dtype])
+                dev.stream_destroy(s)
+            except Exception as e:                      # noqa: BLE001 - reported below
+                errors.append((i, repr(e)))
+
+        threads = [threading.Thread(target=work, args=(i,)) for i in range(len(jobs))]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=60)
+        assert not errors, errors
+        for i, (dtype, op, n, ins, _, _) in enumerate(prepared):
+            assert_parity(results[i], O.reduce_copy(ins, dtype, op), dtype, op, f"thread {i}")

@@ -237,3 +237,55 @@ def test_reduce_fifo_host_protocol():
     assert (buf[7] >> 48) & 0xf == N.DT_BF16 and (buf[7] >> 52) & 0xf == N.OP_MAX and buf[7] & 0xffffffff == 6
     assert N.lib.fx_fifo_init(buf, 0) == N.INVALID_ARGUMENT and N.lib.fx_fifo_init(buf, 2000) == N.INVALID_ARGUMENT
     assert N.lib.fx_fifo_poll_state(buf, 5) == -1
+
+
+def test_headers_are_plain_c_and_a_c_client_links(tmp_path):
+    """The boundary is a C ABI: every header compiles as strict C11, a C program
+    links against the kernel library and the host-only entry points answer."""
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "client.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "flagcx_amd/fx_types.h"
+#include "flagcx_amd/fx_kernels.h"
+#include "flagcx_amd/fx_sim.h"
+#include "flagcx_amd/fx_synth.h"
+#include "flagcx_amd/fx_device_adaptor.h"
+#include "flagcx_amd/fx_ccl_adaptor.h"
+_Static_assert(sizeof(fxReduceTrigger) == 32, "trigger is 32 bytes");
+_Static_assert(sizeof(struct flagcxDeviceAdaptor_v1) == 32 + 48 * sizeof(void *), "v1 device adaptor layout");
+_Static_assert(sizeof(struct flagcxCCLAdaptor_v1) == 35 * sizeof(void *), "v1 ccl adaptor layout");
+_Static_assert(sizeof(flagcxUniqueId) == 256, "unique id");
+int main(void) {
+  size_t cnt, off;
+  fxReduceTrigger t;
+  int dt, op, st, version;
+  uint64_t c;
+  flagcxUniqueId a, b;
+  fx_split(10, 3, 0, &cnt, &off);
+  if (cnt != 4 || off != 0) return 1;
+  fx_trigger_set(&t, 1, 2, 3, 77, 32, flagcxBfloat16, flagcxMax, fxTriggerEnqueued);
+  fx_trigger_get(&t, NULL, NULL, NULL, &c, NULL, &dt, &op, &st);
+  if (c != 77 || dt != flagcxBfloat16 || op != flagcxMax || st != fxTriggerEnqueued) return 2;
+  if (fx_dtype_size(flagcxFloat64) != 8 || fx_dtype_size(99) != 0) return 3;
+  if (fx_reduce_copy(NULL, NULL, 2, 4, flagcxFloat32, flagcxAvg, 0, NULL) != flagcxNotSupported) return 4;
+  if (strcmp(flagcxGetErrorString(flagcxInvalidArgument), "invalid argument")) return 5;
+  if (flagcxGetVersion(&version) != flagcxSuccess || version != FX_SIM_VERSION) return 6;
+  if (flagcxGetUniqueId(&a) != flagcxSuccess || flagcxGetUniqueId(&b) != flagcxSuccess) return 7;
+  if (!memcmp(&a, &b, sizeof(a))) return 8;
+  printf("%s\n", fx_version());
+  return 0;
+}
+''')
+    exe = tmp_path / "client"
+    libdir = os.path.join(root, "flagcx_amd", "lib")
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{root}/include", str(src), "-o",
+                    str(exe), f"-L{libdir}", "-lflagcx_amd", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"],
+                   check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert "flagcx_amd" in out

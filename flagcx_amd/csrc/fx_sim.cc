@@ -14,6 +14,7 @@
 
 #include <atomic>
 #include <chrono>
+#include <condition_variable>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -54,6 +55,7 @@ struct PendingP2p {
   size_t bytes;
   hipStream_t stream;
   hipEvent_t posted;       // recorded on `stream` when the call was made
+  uint64_t id;             // names this half for a sleeping poster (rendezvous mode)
 };
 
 struct Group {
@@ -63,6 +65,8 @@ struct Group {
   std::string id;          // non-empty when created rank by rank (fxSimCommInitRank)
   int joined = 0, alive = 0;
   std::vector<PendingP2p> p2p;
+  uint64_t nextP2pId = 1;
+  std::map<uint64_t, flagcxResult_t> p2pMatched;  // rendezvous mode: verdicts awaiting their sleeping poster
   // pending collective
   Kind kind = kNone;
   size_t count = 0;
@@ -70,7 +74,13 @@ struct Group {
   std::vector<Post> posts;
   std::vector<hipEvent_t> ready;
   hipEvent_t done = nullptr;
+  // rendezvous mode: posters sleep here until the collective they joined is launched
+  std::condition_variable cv;
+  uint64_t launched = 0;       // collectives launched (or abandoned) so far
+  flagcxResult_t lastResult = flagcxSuccess;
+  long long timeoutMs = 30000;
   // configuration
+  long long sync = FX_SYNC_GROUP;
   long long algo = FX_ALGO_DIRECT, order = FX_ORDER_RANK;
   long long nslices = 1, nredslices = 0, redslicesize = 65536;
   // scratch: ring reduce-scatter partials / alltoallv staging
@@ -480,6 +490,15 @@ void resetPending(Group *g) {
   for (auto &p : g->posts) p = Post();
 }
 
+// Drop the pending collective because of a caller error; ranks asleep in a
+// rendezvous get the same verdict.
+void abandonPending(Group *g, flagcxResult_t why) {
+  resetPending(g);
+  g->lastResult = why;
+  g->launched++;
+  g->cv.notify_all();
+}
+
 // Record one rank's call; the last rank to arrive launches the collective.
 flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, void *recv, size_t count, int dtype,
                                int op, int root, flagcxStream_t stream, const size_t *sc = nullptr,
@@ -512,7 +531,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   if (!comm || !comm->g || !stream) return flagcxInvalidArgument;
   Group *g = comm->g;
   const int rank = comm->rank;
-  std::lock_guard<std::mutex> lock(g->mu);
+  std::unique_lock<std::mutex> lock(g->mu);
   if (g->nposted == 0) {
     g->kind = kind;
     g->count = count;
@@ -520,13 +539,13 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
     g->op = op;
     g->root = root;
   } else if (g->kind != kind || g->count != count || g->dtype != dtype || g->op != op || g->root != root) {
-    resetPending(g);
-    return flagcxInvalidArgument;  // ranks disagree on the collective
+    abandonPending(g, flagcxInvalidArgument);  // ranks disagree on the collective
+    return flagcxInvalidArgument;
   }
   Post &p = g->posts[rank];
   if (p.posted) {
-    resetPending(g);
-    return flagcxInvalidUsage;  // same rank called twice before the others arrived
+    abandonPending(g, flagcxInvalidUsage);  // same rank called twice before the others arrived
+    return flagcxInvalidUsage;
   }
   p.posted = true;
   p.send = send;
@@ -538,17 +557,33 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
     p.recvcounts.assign(rc_, rc_ + g->n);
     p.rdispls.assign(rd, rd + g->n);
   }
-  if (hipEventRecord(g->ready[rank], p.stream) != hipSuccess) {
-    resetPending(g);
-    return flagcxUnhandledDeviceError;
+  if (++g->nposted < g->n) {
+    if (g->sync != FX_SYNC_RENDEZVOUS) return flagcxSuccess;
+    // Sleep until the last rank has launched this collective (it also makes this
+    // rank's stream wait for the result before it wakes us).
+    const uint64_t mine = g->launched;
+    if (!g->cv.wait_for(lock, std::chrono::milliseconds(g->timeoutMs), [&] { return g->launched != mine; })) {
+      resetPending(g);  // a rank never arrived: give up for everybody
+      g->lastResult = flagcxInternalError;
+      g->launched++;
+      g->cv.notify_all();
+    }
+    return g->lastResult;
   }
-  if (++g->nposted < g->n) return flagcxSuccess;
 
+  // Last rank in: order the launch after everything the other ranks' streams
+  // hold right now (their calls are already made, so that covers all they
+  // enqueued before calling).  One event per distinct foreign stream.
   Ctx c{g, p.stream, g->n, fx_dtype_size(dtype)};
   flagcxResult_t res = flagcxSuccess;
-  for (int r = 0; r < g->n && res == flagcxSuccess; r++)
-    if (g->posts[r].stream != c.s && hipStreamWaitEvent(c.s, g->ready[r], 0) != hipSuccess)
+  for (int r = 0; r < g->n && res == flagcxSuccess; r++) {
+    hipStream_t s = g->posts[r].stream;
+    bool seen = (s == c.s);
+    for (int q = 0; q < r && !seen; q++) seen = (g->posts[q].stream == s);
+    if (seen) continue;
+    if (hipEventRecord(g->ready[r], s) != hipSuccess || hipStreamWaitEvent(c.s, g->ready[r], 0) != hipSuccess)
       res = flagcxUnhandledDeviceError;
+  }
   if (res == flagcxSuccess) {
     switch (kind) {
       case kAllReduce: res = runAllReduce(c); break;
@@ -570,12 +605,18 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
     for (int r = 0; r < g->n; r++) others = others || (g->posts[r].stream != c.s);
     if (others) {
       if (hipEventRecord(g->done, c.s) != hipSuccess) res = flagcxUnhandledDeviceError;
-      for (int r = 0; r < g->n && res == flagcxSuccess; r++)
-        if (g->posts[r].stream != c.s && hipStreamWaitEvent(g->posts[r].stream, g->done, 0) != hipSuccess)
-          res = flagcxUnhandledDeviceError;
+      for (int r = 0; r < g->n && res == flagcxSuccess; r++) {
+        hipStream_t s = g->posts[r].stream;
+        bool seen = (s == c.s);
+        for (int q = 0; q < r && !seen; q++) seen = (g->posts[q].stream == s);
+        if (!seen && hipStreamWaitEvent(s, g->done, 0) != hipSuccess) res = flagcxUnhandledDeviceError;
+      }
     }
   }
   resetPending(g);
+  g->lastResult = res;
+  g->launched++;
+  g->cv.notify_all();
   return res;
 }
 
@@ -619,6 +660,10 @@ flagcxResult_t newGroup(int nranks, Group **out) {
   if (g->nslices < 1) g->nslices = 1;
   if (g->nredslices < 0) g->nredslices = 0;
   if (g->redslicesize < 0) g->redslicesize = 0;
+  const char *sync = getenv("FX_SIM_SYNC");
+  if (sync && !strcmp(sync, "rendezvous")) g->sync = FX_SYNC_RENDEZVOUS;
+  g->timeoutMs = envParam("FX_SIM_RENDEZVOUS_TIMEOUT_MS", 30000);
+  if (g->timeoutMs < 1) g->timeoutMs = 1;
   *out = g;
   return flagcxSuccess;
 }
@@ -652,7 +697,7 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
   if (count && !(isSend ? sbuf : (const void *)rbuf)) return flagcxInvalidArgument;
   const int src = isSend ? comm->rank : peer, dst = isSend ? peer : comm->rank;
   const size_t bytes = count * ts;
-  std::lock_guard<std::mutex> lock(g->mu);
+  std::unique_lock<std::mutex> lock(g->mu);
   for (size_t i = 0; i < g->p2p.size(); i++) {
     PendingP2p &o = g->p2p[i];
     if (o.isSend == isSend || o.src != src || o.dst != dst) continue;
@@ -670,15 +715,37 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
       }
     }
     (void)hipEventDestroy(o.posted);
+    if (g->sync == FX_SYNC_RENDEZVOUS) {
+      g->p2pMatched[o.id] = res;
+      g->cv.notify_all();
+    }
     g->p2p.erase(g->p2p.begin() + (long)i);
     return res;
   }
-  PendingP2p p{isSend, src, dst, sbuf, rbuf, bytes, stream->base, nullptr};
-  if (hipEventCreateWithFlags(&p.posted, hipEventDisableTiming) != hipSuccess ||
-      hipEventRecord(p.posted, p.stream) != hipSuccess)
+  PendingP2p p{isSend, src, dst, sbuf, rbuf, bytes, stream->base, nullptr, g->nextP2pId++};
+  if (hipEventCreateWithFlags(&p.posted, hipEventDisableTiming) != hipSuccess) return flagcxUnhandledDeviceError;
+  if (hipEventRecord(p.posted, p.stream) != hipSuccess) {
+    (void)hipEventDestroy(p.posted);
     return flagcxUnhandledDeviceError;
+  }
   g->p2p.push_back(p);
-  return flagcxSuccess;
+  if (g->sync != FX_SYNC_RENDEZVOUS) return flagcxSuccess;
+  // Sleep until the partner has made its call and enqueued the copy.
+  const uint64_t id = p.id;
+  const bool matched = g->cv.wait_for(lock, std::chrono::milliseconds(g->timeoutMs),
+                                      [&] { return g->p2pMatched.count(id) != 0; });
+  if (!matched) {  // the partner never came: withdraw this half
+    for (size_t i = 0; i < g->p2p.size(); i++)
+      if (g->p2p[i].id == id) {
+        (void)hipEventDestroy(g->p2p[i].posted);
+        g->p2p.erase(g->p2p.begin() + (long)i);
+        break;
+      }
+    return flagcxInternalError;
+  }
+  const flagcxResult_t res = g->p2pMatched[id];
+  g->p2pMatched.erase(id);
+  return res;
 }
 
 void partNode(fxRedNode *n, int step, int rank, size_t slice, int in1, int in2, int out, size_t inOff, size_t outOff,
@@ -853,6 +920,11 @@ flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
     case FX_SIM_REDSLICESIZE:
       if (value < 0) return flagcxInvalidArgument;
       g->redslicesize = value;
+      break;
+    case FX_SIM_SYNC:
+      if (value != FX_SYNC_GROUP && value != FX_SYNC_RENDEZVOUS) return flagcxInvalidArgument;
+      if (g->nposted) return flagcxInvalidUsage;  // not while a collective is half posted
+      g->sync = value;
       break;
     default: return flagcxInvalidArgument;
   }

@@ -6,9 +6,10 @@ from . import _native as N
 
 lib = N.lib
 
-ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE = 0, 1, 2, 3, 4
+ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE, SYNC = 0, 1, 2, 3, 4, 5
 ALGO_DIRECT, ALGO_RING = 0, 1
-ORDER_RANK, ORDER_RING = 0, 1
+ORDER_RANK, ORDER_RING, ORDER_TREE = 0, 1, 2
+SYNC_GROUP, SYNC_RENDEZVOUS = 0, 1
 
 
 def _szs(v):
@@ -22,9 +23,9 @@ class SimGroup:
         N.check(lib.fxSimCommInitAll(self.comms, nranks), "fxSimCommInitAll")
         self.configure(**config)
 
-    def configure(self, algo=None, order=None, nslices=None, nredslices=None, redslicesize=None):
+    def configure(self, algo=None, order=None, nslices=None, nredslices=None, redslicesize=None, sync=None):
         for key, val in ((ALGO, algo), (ORDER, order), (NSLICES, nslices), (NREDSLICES, nredslices),
-                         (REDSLICESIZE, redslicesize)):
+                         (REDSLICESIZE, redslicesize), (SYNC, sync)):
             if val is not None:
                 N.check(lib.fxSimCommConfig(self.comms[0], key, val), f"fxSimCommConfig({key})")
 

@@ -11,12 +11,24 @@
  * "peer IPC buffers" are ordinary allocations in the same GPU's HBM.  No
  * inter-GPU transport exists here.
  *
- * Calling convention (single-process multi-rank, like a grouped launch): every
- * rank of the group calls the same collective once; calls are enqueue-only
- * (flagcx.h:345-346).  The work is launched when the last rank has posted, on
- * that caller's stream, after waiting for the other ranks' streams; those
- * streams in turn wait for the result.  In-place rules are FlagCX's
- * (flagcx.h:369,423,439,454).
+ * Calling convention (single-process multi-rank): every rank of the group
+ * calls the same collective once; the work is launched when the last rank has
+ * posted, on that caller's stream, after waiting for what the other ranks'
+ * streams held at that moment; those streams in turn wait for the result.
+ * In-place rules are FlagCX's (flagcx.h:369,423,439,454).
+ *
+ * Two synchronisation modes (FX_SIM_SYNC):
+ *   FX_SYNC_GROUP (default)  every call returns at once (flagcx.h:345-346).
+ *     Like the calls of one ncclGroupStart/End bracket, a collective is ordered
+ *     after work a rank enqueued BEFORE the last rank posted and before work
+ *     enqueued AFTER it: a single host thread that loops over the ranks, on one
+ *     stream or several, needs nothing else.
+ *   FX_SYNC_RENDEZVOUS       for one host thread per rank, each on its own
+ *     stream, the way separate FlagCX processes behave: a call blocks its host
+ *     thread until every rank has posted and the work is enqueued, so whatever
+ *     the rank enqueues after the call returns is ordered after the collective.
+ *     A rank that never arrives makes the others return flagcxInternalError
+ *     after FX_SIM_RENDEZVOUS_TIMEOUT_MS (environment, default 30000).
  */
 #ifndef FLAGCX_AMD_FX_SIM_H_
 #define FLAGCX_AMD_FX_SIM_H_
@@ -71,7 +83,12 @@ enum {
   FX_SIM_ORDER = 1,        /* FX_ORDER_*                                  */
   FX_SIM_NSLICES = 2,      /* FLAGCX_UNIRUNNER_NSLICES (default 1)        */
   FX_SIM_NREDSLICES = 3,   /* FLAGCX_UNIRUNNER_NREDSLICES (0 = automatic) */
-  FX_SIM_REDSLICESIZE = 4  /* FLAGCX_UNIRUNNER_REDSLICESIZE (65536 elems) */
+  FX_SIM_REDSLICESIZE = 4, /* FLAGCX_UNIRUNNER_REDSLICESIZE (65536 elems) */
+  FX_SIM_SYNC = 5          /* FX_SYNC_*; environment FX_SIM_SYNC=group|rendezvous */
+};
+enum {
+  FX_SYNC_GROUP = 0,
+  FX_SYNC_RENDEZVOUS = 1
 };
 enum {
   FX_ALGO_DIRECT = 0, /* one k-way reduce per slice, then all-gather copies */

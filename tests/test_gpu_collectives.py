@@ -317,3 +317,82 @@ def test_one_host_thread_per_rank(dev):
             assert_parity(dev.to_host(dr[0][r], count, np.float32), want[N.OP_SUM], N.DT_FP32, N.OP_SUM, f"rank {r}")
         for s in streams:
             dev.stream_destroy(s)
+
+
+def test_rendezvous_mode_orders_later_work_after_the_collective(dev):
+    """One host thread per rank, each on its own stream, written the way the
+    reference's per-process tests are (coll_allreduce.cpp:9-37): upload, all-reduce,
+    download on the same stream right after the call, synchronise, check -- with
+    no host barrier between ranks.  Only a call that returns after the collective
+    is enqueued makes the download see the result."""
+    import threading
+    n, count, rounds = 8, 50001, 12
+    idx = np.arange(count)
+    errors = []
+    with DevBufs(dev) as b, S.SimGroup(n, sync=S.SYNC_RENDEZVOUS) as g:
+        dbuf = [b.alloc(count * 4) for _ in range(n)]
+        dtmp = [b.alloc(count * 4) for _ in range(n)]
+
+        def rank_main(r):
+            try:
+                dev.set_device()
+                s = dev.stream_create()
+                host = np.empty(count, np.float32)
+                for it in range(rounds):
+                    src = ((r + it) * 1000 + idx % 10).astype(np.float32)      # kept alive until the stream is drained
+                    dev.upload(dbuf[r], src, s)
+                    N.check(N.lib.flagcxAllReduce(dbuf[r], dbuf[r], count, N.DT_FP32, N.OP_SUM, g.comms[r], s))
+                    dev.download(host, dbuf[r], s)
+                    dev.stream_sync(s)
+                    want = (sum(q + it for q in range(n)) * 1000 + n * (idx % 10)).astype(np.float32)
+                    if not np.array_equal(host, want):
+                        errors.append((r, it, "allreduce", host[:4].tolist(), want[:4].tolist()))
+                    # ring shift: send own block to the right neighbour, receive from the left one
+                    src = np.full(count, r * 100 + it, np.float32)
+                    dev.upload(dbuf[r], src, s)
+                    if r % 2 == 0:      # even ranks send first, odd ranks receive first: no cyclic wait
+                        N.check(N.lib.flagcxSend(dbuf[r], count, N.DT_FP32, (r + 1) % n, g.comms[r], s))
+                        N.check(N.lib.flagcxRecv(dtmp[r], count, N.DT_FP32, (r - 1) % n, g.comms[r], s))
+                    else:
+                        N.check(N.lib.flagcxRecv(dtmp[r], count, N.DT_FP32, (r - 1) % n, g.comms[r], s))
+                        N.check(N.lib.flagcxSend(dbuf[r], count, N.DT_FP32, (r + 1) % n, g.comms[r], s))
+                    dev.download(host, dtmp[r], s)
+                    dev.stream_sync(s)
+                    if not (host == ((r - 1) % n) * 100 + it).all():
+                        errors.append((r, it, "sendrecv", host[:4].tolist()))
+                    N.check(N.lib.flagcxBarrier(g.comms[r], s))     # nobody overwrites dbuf while a neighbour reads it
+                    dev.stream_sync(s)
+                dev.stream_destroy(s)
+            except Exception as e:                      # noqa: BLE001 - reported below
+                errors.append((r, repr(e)))
+
+        threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=100)
+        assert not any(t.is_alive() for t in threads)
+        assert not errors, errors[:4]
+
+
+def test_rendezvous_times_out_when_a_rank_never_arrives(dev, stream, monkeypatch):
+    import threading
+    monkeypatch.setenv("FX_SIM_RENDEZVOUS_TIMEOUT_MS", "200")
+    n = 4
+    codes = {}
+    with DevBufs(dev) as b, S.SimGroup(n, sync=S.SYNC_RENDEZVOUS) as g:
+        p = b.alloc(1024)
+
+        def rank_main(r):
+            codes[r] = N.lib.flagcxAllReduce(p, p, 16, N.DT_FP32, N.OP_SUM, g.comms[r], stream)
+
+        threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(n - 1)]    # rank 3 stays away
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=20)
+        assert codes == {0: N.INTERNAL_ERROR, 1: N.INTERNAL_ERROR, 2: N.INTERNAL_ERROR}
+        # nothing was enqueued and the group is usable again
+        g.configure(sync=S.SYNC_GROUP)
+        N.check(g.all_reduce([p] * n, [p] * n, 0, N.DT_FP32, N.OP_SUM, stream))
+        dev.stream_sync(stream)

@@ -41,6 +41,10 @@ class ReduceTrigger(C.Structure):
     _fields_ = [("value", C.c_uint64 * 4)]
 
 
+class BcastDesc(C.Structure):
+    _fields_ = [("inp", C.c_void_p * 8), ("out", C.c_void_p * 8), ("count", C.c_uint64)]
+
+
 class SliceDesc(C.Structure):
     _fields_ = [("in_", C.c_void_p * 8), ("out", C.c_void_p), ("count", C.c_uint64)]
 
@@ -63,6 +67,7 @@ _SIGS = {
     "fx_trigger_get": (None, [C.POINTER(ReduceTrigger)] + [C.POINTER(C.c_uint64)] * 5 + [C.POINTER(_i)] * 3),
     "fx_reduce_triggers": (_i, [C.POINTER(ReduceTrigger), _sz, _vp]),
     "fx_reduce_slices": (_i, [C.POINTER(SliceDesc), _sz, _i, _i, _i, _vp]),
+    "fx_reduce_bcast_slices": (_i, [C.POINTER(BcastDesc), _sz, _i, _i, _i, _i, _vp]),
     "fx_copy_slices": (_i, [C.POINTER(SliceDesc), _sz, _vp]),
     "fx_plan_create": (_i, [C.POINTER(_vp), C.POINTER(SliceDesc), _sz, _i, _i, _i]),
     "fx_plan_launch": (_i, [_vp, _vp]),

@@ -262,6 +262,112 @@ int fx_copy_slices(const fxSliceDesc *slices, size_t n, void *stream) {
   });
 }
 
+int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout, int dtype, int op, void *stream) {
+  const bool copy = (op == -1);
+  if (copy) {
+    k = 1;
+  } else {
+    flagcxResult_t rc = screen(dtype, op);
+    if (rc != flagcxSuccess) return rc;
+  }
+  if (k < 1 || k > FX_MAX_SLICE_INPUTS || nout < 1 || nout > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
+  if (n == 0) return flagcxSuccess;
+  if (!slices) return flagcxInvalidArgument;
+  return guarded([&]() -> int {
+    hipStream_t s = (hipStream_t)stream;
+    // element size: the dtype's, or for copies the widest unit every pointer and count allows
+    uintptr_t bits = 0;
+    for (size_t i = 0; i < n; i++) {
+      if (slices[i].count == 0) continue;
+      for (int p = 0; p < k; p++) {
+        if (!slices[i].in[p]) return flagcxInvalidArgument;
+        bits |= (uintptr_t)slices[i].in[p];
+      }
+      for (int o = 0; o < nout; o++) {
+        if (!slices[i].out[o]) return flagcxInvalidArgument;
+        bits |= (uintptr_t)slices[i].out[o];
+      }
+      if (copy) bits |= (uintptr_t)slices[i].count;
+    }
+    const int es = copy ? ((bits & 1) ? 1 : ((bits & 2) ? 2 : 4)) : (int)dtypeSize(dtype);
+    if (!copy && (bits & (uintptr_t)(es - 1))) return flagcxInvalidArgument;
+    const KernelSet *ks = copy ? copySetFor(es) : setFor(dtype, op);
+    const int U = unrollFor(k);
+    // merge slices that continue each other in every stream
+    std::vector<fxBcastDesc> merged;
+    merged.reserve(n);
+    for (size_t i = 0; i < n; i++) {
+      fxBcastDesc d = slices[i];
+      if (d.count == 0) continue;
+      if (copy) d.count /= (uint64_t)es;
+      if (!merged.empty()) {
+        fxBcastDesc &l = merged.back();
+        const size_t bytes = l.count * (size_t)es;
+        bool cont = true;
+        for (int p = 0; p < k && cont; p++) cont = (const char *)d.in[p] == (const char *)l.in[p] + bytes;
+        for (int o = 0; o < nout && cont; o++) cont = (const char *)d.out[o] == (const char *)l.out[o] + bytes;
+        if (cont) {
+          l.count += d.count;
+          continue;
+        }
+      }
+      merged.push_back(d);
+    }
+    std::vector<fxSliceDesc> plainReduce, plainCopy;  // slices whose outputs are not co-aligned
+    InlineBcastTable t;
+    t.n = 0;
+    t.tileStart[0] = 0;
+    auto flush = [&]() -> flagcxResult_t {
+      if (t.n == 0) return flagcxSuccess;
+      flagcxResult_t rc = ks->bcastInline[k](t, s);
+      t.n = 0;
+      return rc;
+    };
+    for (const fxBcastDesc &d : merged) {
+      bool same = true;
+      for (int o = 1; o < nout; o++) same = same && (((uintptr_t)d.out[o] & 15u) == ((uintptr_t)d.out[0] & 15u));
+      if (!same) {
+        fxSliceDesc r;
+        memset(&r, 0, sizeof(r));
+        for (int p = 0; p < k; p++) r.in[p] = d.in[p];
+        r.out = d.out[0];
+        r.count = d.count;
+        plainReduce.push_back(r);
+        for (int o = 1; o < nout; o++) {
+          fxSliceDesc c;
+          memset(&c, 0, sizeof(c));
+          c.in[0] = d.out[0];
+          c.out = d.out[o];
+          c.count = d.count * (uint64_t)es;
+          plainCopy.push_back(c);
+        }
+        continue;
+      }
+      const uint64_t tiles = tilesFor(d.out[0], d.in, k, d.count, es, U);
+      if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+      if (t.n == (uint32_t)kInlineBcast || (uint64_t)t.tileStart[t.n] + tiles > 0x7ffffff0ull) {
+        flagcxResult_t rc = flush();
+        if (rc != flagcxSuccess) return rc;
+      }
+      BcastDescDev &dd = t.d[t.n];
+      for (int p = 0; p < kMaxFixedK; p++) dd.in[p] = (p < k) ? d.in[p] : nullptr;
+      for (int o = 0; o < kMaxFixedK; o++) dd.out[o] = (o < nout) ? d.out[o] : nullptr;
+      dd.count = d.count;
+      dd.nout = (uint32_t)nout;
+      t.tileStart[t.n + 1] = t.tileStart[t.n] + (uint32_t)tiles;
+      t.n++;
+    }
+    flagcxResult_t rc = flush();
+    if (rc != flagcxSuccess) return rc;
+    if (!plainReduce.empty()) {
+      rc = launchSliceBatches(ks, plainReduce.data(), plainReduce.size(), k, s);
+      if (rc != flagcxSuccess) return rc;
+      return fx_copy_slices(plainCopy.data(), plainCopy.size(), stream);
+    }
+    return flagcxSuccess;
+  });
+}
+
 int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, int dtype, int op) {
   if (!plan) return flagcxInvalidArgument;
   *plan = nullptr;

@@ -19,6 +19,7 @@ struct KernelSet {
   flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const InlineSliceTable &t, hipStream_t s);
   flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
                                                 uint32_t grid, hipStream_t s);
+  flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const InlineBcastTable &t, hipStream_t s);
   int elemSize;
 };
 
@@ -73,14 +74,27 @@ flagcxResult_t launchSlicesTable(const SliceDescDev *d, const uint32_t *tileStar
 }
 
 template <class R, int K>
+flagcxResult_t launchBcastInline(const InlineBcastTable &t, hipStream_t s) {
+  constexpr int U = unrollFor(K);
+  uint32_t grid = t.tileStart[t.n];
+  if (grid == 0) return flagcxSuccess;
+  hipLaunchKernelGGL((reduceBcastInline<R, K, U>), dim3(grid), dim3(kBlock), 0, s, t);
+  FX_HIP(hipGetLastError());
+  return flagcxSuccess;
+}
+
+template <class R, int K, bool BCAST = true>
 void fillSet(KernelSet &ks) {
   ks.direct[K] = &launchDirect<R, K>;
   if (K > 0) {
     ks.slicesInline[K] = &launchSlicesInline<R, (K > 0 ? K : 1)>;
     ks.slicesTable[K] = &launchSlicesTable<R, (K > 0 ? K : 1)>;
+    if constexpr (BCAST) ks.bcastInline[K] = &launchBcastInline<R, (K > 0 ? K : 1)>;
+    else ks.bcastInline[K] = nullptr;
   } else {
     ks.slicesInline[0] = nullptr;
     ks.slicesTable[0] = nullptr;
+    ks.bcastInline[0] = nullptr;
   }
 }
 
@@ -104,7 +118,7 @@ KernelSet makeSet() {
 template <int ES>
 KernelSet makeCopySet() {
   KernelSet ks = {};
-  fillSet<CopyRed<ES>, 1>(ks);
+  fillSet<CopyRed<ES>, 1, true>(ks);
   ks.elemSize = ES;
   return ks;
 }

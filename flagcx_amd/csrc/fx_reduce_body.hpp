@@ -473,6 +473,39 @@ __device__ __forceinline__ void scatterElems(char *base, uint64_t e0, int lo, in
   }
 }
 
+// Segment with several outputs: the result of every vector is stored to out
+// and to each of more[0..nmore-1] (the software form of a multicast store: one
+// read of the k inputs serves every rank's receive buffer).  All outputs share
+// out's misalignment within 16 bytes; the host checks that.
+template <int K>
+struct SegB : Seg<K> {
+  char *more[kMaxFixedK - 1];
+  int nmore;
+};
+
+template <int K>
+__device__ __forceinline__ void storeVector(const Seg<K> &sg, uint64_t byteOff, u32x4 v) {
+  stg_stream(sg.out + byteOff, v);
+}
+template <int K>
+__device__ __forceinline__ void storeVector(const SegB<K> &sg, uint64_t byteOff, u32x4 v) {
+  stg_stream(sg.out + byteOff, v);
+#pragma unroll
+  for (int o = 0; o < kMaxFixedK - 1; o++)   // constant indices keep the pointers in scalar registers
+    if (o < sg.nmore) stg_stream(sg.more[o] + byteOff, v);
+}
+template <int ES, int K>
+__device__ __forceinline__ void storeElems(const Seg<K> &sg, uint64_t e0, int lo, int hi, u32x4 v) {
+  scatterElems<ES>(sg.out, e0, lo, hi, v);
+}
+template <int ES, int K>
+__device__ __forceinline__ void storeElems(const SegB<K> &sg, uint64_t e0, int lo, int hi, u32x4 v) {
+  scatterElems<ES>(sg.out, e0, lo, hi, v);
+#pragma unroll
+  for (int o = 0; o < kMaxFixedK - 1; o++)
+    if (o < sg.nmore) scatterElems<ES>(sg.more[o], e0, lo, hi, v);
+}
+
 // A whole 16-byte vector from an address that is only element-aligned: aligned
 // dword loads plus a funnel shift.  The dword holding the first (last) byte may
 // start before (end after) the vector, but never leaves the 4-byte word that
@@ -496,8 +529,8 @@ __device__ __forceinline__ u32x4 loadVectorUnaligned(const char *p) {
 }
 
 // Reduce vector j of the segment with full bounds / alignment handling.
-template <class R, int K>
-__device__ __forceinline__ void reduceVectorChecked(const Seg<K> &sg, uint64_t j) {
+template <class R, int K, class SG>
+__device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
   constexpr int VE = 16 / R::ES;
   const uint64_t e0 = j * VE;
   if (e0 >= sg.end || e0 + VE <= sg.lead) return;
@@ -514,15 +547,15 @@ __device__ __forceinline__ void reduceVectorChecked(const Seg<K> &sg, uint64_t j
   for (int p = 1; p < k; p++) R::fold(acc, fetch(p));
   u32x4 r = R::finish(acc);
   if (full)
-    stg_stream(sg.out + j * 16, r);
+    storeVector(sg, j * 16, r);
   else
-    scatterElems<R::ES>(sg.out, e0, lo, hi, r);
+    storeElems<R::ES>(sg, e0, lo, hi, r);
 }
 
 // Branch-free body: lane handles U whole vectors at byte offsets off + u*ustride
 // of every stream, all K*U loads in flight before the first use.
-template <class R, int K, int U>
-__device__ __forceinline__ void reduceVectorsFast(const Seg<K> &sg, uint64_t off, uint64_t ustride) {
+template <class R, int K, int U, class SG>
+__device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, uint64_t ustride) {
   if (K > 0) {
     u32x4 v[U][K > 0 ? K : 1];
 #pragma unroll
@@ -535,7 +568,7 @@ __device__ __forceinline__ void reduceVectorsFast(const Seg<K> &sg, uint64_t off
       R::init(acc, v[u][0]);
 #pragma unroll
       for (int p = 1; p < K; p++) R::fold(acc, v[u][p]);
-      stg_stream(sg.out + off + u * ustride, R::finish(acc));
+      storeVector(sg, off + u * ustride, R::finish(acc));
     }
   } else {
     typename R::Acc acc[U];
@@ -550,13 +583,13 @@ __device__ __forceinline__ void reduceVectorsFast(const Seg<K> &sg, uint64_t off
       for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
     }
 #pragma unroll
-    for (int u = 0; u < U; u++) stg_stream(sg.out + off + u * ustride, R::finish(acc[u]));
+    for (int u = 0; u < U; u++) storeVector(sg, off + u * ustride, R::finish(acc[u]));
   }
 }
 
 // Tile `tile` of the segment: striped zone first, then head, then tail.
-template <class R, int K, int U>
-__device__ __forceinline__ void reduceTile(const Seg<K> &sg, const TilePlan &tp, uint32_t tile) {
+template <class R, int K, int U, class SG>
+__device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uint32_t tile) {
   constexpr uint64_t V = (uint64_t)U * kBlock;
   if (tile < tp.zoneTiles) {
     // tile i of region r owns vectors zs + r*RV + row*kRowVecs + i*kPieceVecs + [0, kPieceVecs)
@@ -688,6 +721,37 @@ template <class R, int K, int U>
 __global__ void __launch_bounds__(kBlock)
 reduceSlicesTable(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n) {
   reduceSlicesBody<R, K, U>(d, tileStart, n);
+}
+
+// One read of the inputs, several outputs: slices whose result goes to up to
+// kMaxFixedK buffers at once.
+struct BcastDescDev {
+  const void *in[kMaxFixedK];
+  void *out[kMaxFixedK];
+  uint64_t count;
+  uint32_t nout;
+};
+
+constexpr int kInlineBcast = 16;
+
+struct InlineBcastTable {
+  BcastDescDev d[kInlineBcast];
+  uint32_t tileStart[kInlineBcast + 1];
+  uint32_t n;
+};
+
+template <class R, int K, int U>
+__global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable t) {
+  const uint32_t b = blockIdx.x;
+  const uint32_t i = findSlice(t.tileStart, t.n, b);
+  const BcastDescDev &d = t.d[i];
+  SegB<K> sg;
+  const TilePlan tp = makeSeg<R::ES, U>(static_cast<Seg<K> &>(sg), d.in, d.out[0], d.count, K);
+  const uint64_t mis = (uint64_t)(uintptr_t)d.out[0] & 15u;
+  sg.nmore = (int)d.nout - 1;
+#pragma unroll
+  for (int o = 0; o < kMaxFixedK - 1; o++) sg.more[o] = (o < sg.nmore) ? (char *)d.out[o + 1] - mis : nullptr;
+  reduceTile<R, K, U>(sg, tp, b - t.tileStart[i]);
 }
 
 }  // namespace fx

@@ -156,6 +156,10 @@ flagcxResult_t flushKway(const Ctx &c, std::vector<fxSliceDesc> &descs) {
   return rc;
 }
 
+// One read, n stores: usable when both the inputs and the outputs of a
+// descriptor fit its eight slots.
+inline bool canBroadcast(const Ctx &c) { return c.n <= FX_MAX_SLICE_INPUTS; }
+
 // Visit the (slice, red-slice) pieces of a chunk of ccnt elements at element
 // offset coff, exactly as the reference nests its three splits.
 template <class F>
@@ -226,7 +230,30 @@ flagcxResult_t runAllReduce(const Ctx &c) {
     }
     return flagcxSuccess;
   }
-  // direct: chunk ch is reduced k-way into the rank the ring would leave it
+  // direct, up to eight ranks: every piece is reduced k-way once and stored to
+  // all n receive buffers by the same workgroup -- (k + n) * size bytes of
+  // traffic instead of the (k + 1 + 2 (n - 1)) * size of reduce-then-copy.
+  if (canBroadcast(c)) {
+    std::vector<fxBcastDesc> bd;
+    for (int ch = 0; ch < n; ch++) {
+      size_t ccnt, coff;
+      fx_split(count, n, ch, &ccnt, &coff);
+      const int first = (g->order == FX_ORDER_RING) ? ch : 0;
+      flagcxResult_t rc = forPieces(g, ccnt, coff, nred, [&](size_t off, size_t, size_t cnt) {
+        if (cnt == 0) return flagcxSuccess;
+        fxBcastDesc d;
+        memset(&d, 0, sizeof(d));
+        for (int j = 0; j < n; j++) d.in[j] = cadd(c.send(mod(first + j, n)), off * ts);
+        for (int r = 0; r < n; r++) d.out[r] = madd(c.recv(r), off * ts);
+        d.count = cnt;
+        bd.push_back(d);
+        return flagcxSuccess;
+      });
+      if (rc != flagcxSuccess) return rc;
+    }
+    return R(fx_reduce_bcast_slices(bd.data(), bd.size(), n, n, g->dtype, g->op, c.s));
+  }
+  // more ranks: chunk ch is reduced k-way into the rank the ring would leave it
   // on, (ch-1)%n, then copied to everyone else.
   for (int ch = 0; ch < n; ch++) {
     size_t ccnt, coff;
@@ -358,6 +385,16 @@ flagcxResult_t runReduceScatter(const Ctx &c) {
 flagcxResult_t runAllGather(const Ctx &c) {
   const size_t bytes = c.g->count * c.ts;
   if (bytes == 0) return flagcxSuccess;
+  if (canBroadcast(c)) {  // each rank's block is read once and stored to every receive buffer
+    std::vector<fxBcastDesc> bd(c.n);
+    for (int r = 0; r < c.n; r++) {
+      memset(&bd[r], 0, sizeof(fxBcastDesc));
+      bd[r].in[0] = c.send(r);
+      for (int j = 0; j < c.n; j++) bd[r].out[j] = madd(c.recv(j), (size_t)r * bytes);
+      bd[r].count = bytes;
+    }
+    return R(fx_reduce_bcast_slices(bd.data(), bd.size(), 1, c.n, 0, -1, c.s));
+  }
   std::vector<fxSliceDesc> descs;
   for (int r = 0; r < c.n; r++)
     for (int j = 0; j < c.n; j++) {
@@ -428,6 +465,14 @@ flagcxResult_t runScatter(const Ctx &c) {
 
 flagcxResult_t runBroadcast(const Ctx &c) {
   const size_t bytes = c.g->count * c.ts;
+  if (bytes && canBroadcast(c)) {
+    fxBcastDesc b;
+    memset(&b, 0, sizeof(b));
+    b.in[0] = c.send(c.g->root);
+    for (int r = 0; r < c.n; r++) b.out[r] = c.recv(r);
+    b.count = bytes;
+    return R(fx_reduce_bcast_slices(&b, 1, 1, c.n, 0, -1, c.s));
+  }
   std::vector<fxSliceDesc> d;
   for (int r = 0; r < c.n && bytes; r++)
     if (c.recv(r) != c.send(c.g->root)) d.push_back(copyDesc(c.send(c.g->root), c.recv(r), bytes));
@@ -466,6 +511,14 @@ flagcxResult_t runAlltoAll(const Ctx &c) {
 flagcxResult_t runCustomAllReduce(const Ctx &c) {
   Group *g = c.g;
   if (g->count == 0) return flagcxSuccess;
+  if (canBroadcast(c)) {  // every rank's result is the same fold of the windows: compute it once
+    fxBcastDesc b;
+    memset(&b, 0, sizeof(b));
+    for (int j = 0; j < c.n; j++) b.in[j] = g->windows[j];
+    for (int r = 0; r < c.n; r++) b.out[r] = c.recv(r);
+    b.count = g->count;
+    return R(fx_reduce_bcast_slices(&b, 1, c.n, c.n, g->dtype, g->op, c.s));
+  }
   std::vector<fxSliceDesc> descs;
   for (int r = 0; r < c.n; r++) {
     if (c.n <= FX_MAX_SLICE_INPUTS) {

@@ -37,6 +37,19 @@ def reduce_slices(descs, k, dtype, op, stream=None):
     return lib.fx_reduce_slices(arr, n, k, dtype, op, stream)
 
 
+def reduce_bcast_slices(descs, k, nout, dtype, op, stream=None):
+    """descs: iterable of (ins, outs, count); op = -1 broadcasts in[0] (count in bytes)."""
+    descs = list(descs)
+    arr = (N.BcastDesc * max(len(descs), 1))()
+    for i, (ins, outs, count) in enumerate(descs):
+        for p, ptr in enumerate(ins):
+            arr[i].inp[p] = ptr
+        for o, ptr in enumerate(outs):
+            arr[i].out[o] = ptr
+        arr[i].count = count
+    return lib.fx_reduce_bcast_slices(arr, len(descs), k, nout, dtype, op, stream)
+
+
 def copy_slices(descs, stream=None):
     """descs: iterable of (src, dst, nbytes)."""
     arr, n = make_slices(([s], d, b) for s, d, b in descs)

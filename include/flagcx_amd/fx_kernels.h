@@ -137,6 +137,26 @@ int fx_reduce_slices(const fxSliceDesc *slices, size_t n, int k, int dtype,
                      int op, void *stream);
 
 /*
+ * Slices whose result goes to several buffers at once: out[0..nout-1] all
+ * receive in[0] (op) ... (op) in[k-1].  One pass reads the k inputs once and
+ * stores nout times -- what the reference gets from multicast stores
+ * (multimem.st in flagcx/adaptor/kernel/nvidia/custom_allreduce.cu, the NVLS
+ * variants of the allreduce kernel) and what an all-reduce over n ranks on one
+ * GPU needs: (k + nout) * size bytes of traffic instead of the
+ * (k + 1 + 2 * (nout - 1)) * size of reduce-then-copy.  op = -1 makes it a
+ * broadcast copy (k = 1, count in bytes, dtype ignored).  Every out[j] may
+ * alias one in[p] exactly.  Outputs that do not share out[0]'s alignment
+ * within 16 bytes are served by a reduce into out[0] plus copies.
+ */
+typedef struct fxBcastDesc {
+  const void *in[FX_MAX_SLICE_INPUTS];
+  void *out[FX_MAX_SLICE_INPUTS];
+  uint64_t count;
+} fxBcastDesc;
+int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
+                           int dtype, int op, void *stream);
+
+/*
  * Copy n independent byte ranges (in[0] -> out, `count` = BYTES): the Cpy node
  * and the all-gather landing copies (uni_runner_impl.cc:322-344,1649-1662;
  * flagcx/core/p2p.cc:257-283) as one launch.

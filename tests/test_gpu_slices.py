@@ -172,3 +172,63 @@ def test_pack_unpack_random_displacements(dev, dname, np_t):
         assert np.array_equal(recv, O.unpack(np.zeros(rlen, np_t), O.pack(send, counts, sdispls), counts, rdispls))
         for c, sd, rd in zip(counts, sdispls, rdispls):           # the identity, segment by segment
             assert np.array_equal(recv[rd:rd + c], send[sd:sd + c])
+
+
+@pytest.mark.parametrize("dname", ["bf16", "fp32", "int8", "fp64"])
+def test_reduce_to_several_outputs_at_once(dev, dname):
+    """fx_reduce_bcast_slices: every output equals the oracle's fold; covers 1..8
+    outputs, in-place outputs (out[j] == in[j]), odd lengths, unaligned but
+    co-aligned buffers, outputs of differing alignment (reduce + copy fallback),
+    several slices per launch and more slices than one launch carries."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    npdt = N.NP_DTYPE[dtype]
+    for k, nout, n, off_el, inplace in [(8, 8, 300001, 0, True), (2, 3, 5, 0, False), (3, 1, 70001, 1, False),
+                                        (4, 8, (1 << 20) + 3, 3, False), (8, 2, 4 << 20, 0, False),
+                                        (5, 4, 1000, None, False)]:
+        ins = seeded_inputs(dtype, k, n, seed=k * 10 + nout)
+        for op in (N.OP_SUM, N.OP_MIN):
+            want = O.reduce_copy(ins, dtype, op)
+            with DevBufs(dev) as b:
+                pad = (off_el or 0) * es
+                dins = [b.put(a, pad_before=pad) for a in ins]
+                if inplace:
+                    douts = dins[:nout]
+                elif off_el is None:            # each output at its own misalignment
+                    douts = [b.alloc(n * es + 64) + (j % (16 // es)) * es for j in range(nout)]
+                else:
+                    douts = [b.alloc(n * es + pad + 64) + pad for _ in range(nout)]
+                N.check(K.reduce_bcast_slices([(dins, douts, n)], k, nout, dtype, op), "fx_reduce_bcast_slices")
+                dev.sync()
+                for j, d in enumerate(douts):
+                    assert_parity(dev.to_host(d, n, npdt), want, dtype, op, f"{dname} k={k} nout={nout} n={n} out {j}")
+    # 40 slices of uneven length cut from one pair of buffers, three outputs, one call
+    k, nout, total = 2, 3, 500000
+    ins = seeded_inputs(dtype, k, total, seed=3)
+    want = O.reduce_copy(ins, dtype, N.OP_SUM)
+    cuts = np.unique(np.random.default_rng(5).integers(0, total, 39))
+    edges = [0] + cuts.tolist() + [total]
+    with DevBufs(dev) as b:
+        dins = [b.put(a) for a in ins]
+        douts = [b.alloc(total * es) for _ in range(nout)]
+        for d in douts:
+            dev.memset(d, 0x5A, total * es)
+        descs = [([p + lo * es for p in dins], [p + lo * es for p in douts], hi - lo)
+                 for lo, hi in zip(edges[:-1], edges[1:]) if (lo // 7) % 5]            # leave some gaps untouched
+        N.check(K.reduce_bcast_slices(descs, k, nout, dtype, N.OP_SUM), "fx_reduce_bcast_slices")
+        dev.sync()
+        expect = np.frombuffer(bytes([0x5A]) * (total * es), dtype=npdt).copy()
+        for lo, hi in zip(edges[:-1], edges[1:]):
+            if (lo // 7) % 5:
+                expect[lo:hi] = want[lo:hi]
+        for d in douts:
+            assert np.array_equal(dev.to_host(d, total, npdt).view(np.uint8), expect.view(np.uint8))
+    # broadcast copy: one source, five destinations, byte granular
+    src = np.random.default_rng(6).integers(0, 256, 100003, dtype=np.uint8)
+    with DevBufs(dev) as b:
+        dsrc = b.put(src, pad_before=3)
+        dd = [b.alloc(src.size + 64) + 3 for _ in range(5)]
+        N.check(K.reduce_bcast_slices([([dsrc], dd, src.size)], 1, 5, 0, -1), "broadcast copy")
+        dev.sync()
+        for d in dd:
+            assert np.array_equal(dev.to_host(d, src.size, np.uint8), src)

@@ -404,22 +404,45 @@ flagcxResult_t runAllGather(const Ctx &c) {
   return R(fx_copy_slices(descs.data(), descs.size(), c.s));
 }
 
-// pack every rank's segments into its contiguous staging slots, then unpack
-// from the peers' slots: two batched launches, safe for send == recv.
+// When no receive segment overlaps any send segment, every segment goes
+// straight from the sender's buffer to the receiver's: one batched launch.
+// Otherwise (in-place use) every rank's segments are packed into contiguous
+// staging slots and unpacked from the peers' slots: two launches.
 flagcxResult_t runAlltoAllv(const Ctx &c) {
   Group *g = c.g;
   const int n = c.n;
   const size_t ts = c.ts;
   std::vector<size_t> base(n + 1, 0);
+  struct Range {
+    uintptr_t lo, hi;
+  };
+  std::vector<Range> sendR, recvR;
   for (int r = 0; r < n; r++) {
     size_t tot = 0;
     for (int i = 0; i < n; i++) {
-      if (g->posts[r].sendcounts[i] != g->posts[i].recvcounts[r]) return flagcxInvalidArgument;
-      tot += g->posts[r].sendcounts[i];
+      const size_t cnt = g->posts[r].sendcounts[i];
+      if (cnt != g->posts[i].recvcounts[r]) return flagcxInvalidArgument;
+      tot += cnt;
+      if (cnt) {
+        const uintptr_t s = (uintptr_t)c.send(r) + g->posts[r].sdispls[i] * ts;
+        const uintptr_t d = (uintptr_t)c.recv(i) + g->posts[i].rdispls[r] * ts;
+        sendR.push_back({s, s + cnt * ts});
+        recvR.push_back({d, d + cnt * ts});
+      }
     }
     base[r + 1] = base[r] + ((tot * ts + 255) & ~(size_t)255);
   }
   if (base[n] == 0) return flagcxSuccess;
+  bool overlap = false;
+  for (size_t a = 0; a < recvR.size() && !overlap; a++)
+    for (size_t b = 0; b < sendR.size() && !overlap; b++)
+      overlap = recvR[a].lo < sendR[b].hi && sendR[b].lo < recvR[a].hi;
+  if (!overlap) {
+    std::vector<fxSliceDesc> direct;
+    for (size_t a = 0; a < recvR.size(); a++)
+      direct.push_back(copyDesc((const void *)sendR[a].lo, (void *)recvR[a].lo, recvR[a].hi - recvR[a].lo));
+    return R(fx_copy_slices(direct.data(), direct.size(), c.s));
+  }
   flagcxResult_t rc = ensureScratch(g, base[n]);
   if (rc != flagcxSuccess) return rc;
   std::vector<fxSliceDesc> pack, unpack;

@@ -197,6 +197,18 @@ def test_alltoallv_matches_oracle(dev, stream):
         bad = counts.T.copy()
         bad[0, 1] += 1                                             # receiver expects more than is sent
         assert g.all_to_allv(ds, counts, sd, dr, bad, rd, N.DT_FP32, stream) == N.INVALID_ARGUMENT
+        # in place (send == recv, uneven blocks laid out back to back): goes through the staging slots
+        blk = np.array([[1000 + 37 * ((r + i) % n) for i in range(n)] for r in range(n)], np.int64)   # symmetric
+        disp = np.concatenate([np.zeros((n, 1), np.int64), np.cumsum(blk, axis=1)[:, :-1]], axis=1)
+        bufs = [rng.integers(0, 2**32, int(blk[r].sum()), dtype=np.uint64).astype(np.uint32) for r in range(n)]
+        dbuf = [b.put(a) for a in bufs]
+        N.check(g.all_to_allv(dbuf, blk, disp, dbuf, blk.T, disp, N.DT_FP32, stream))
+        dev.stream_sync(stream)
+        for i in range(n):
+            got = dev.to_host(dbuf[i], bufs[i].size, np.uint32)
+            for r in range(n):
+                src = bufs[r][disp[r, i]:disp[r, i] + blk[r, i]]
+                assert np.array_equal(got[disp[i, r]:disp[i, r] + blk[r, i]], src), (i, r)
 
 
 def test_custom_allreduce_hook(dev, stream):

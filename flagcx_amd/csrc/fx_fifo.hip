@@ -90,6 +90,21 @@ __device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b,
   }
 }
 
+// Workgroups that take part in one trigger: one per tile, at most the grid,
+// at least one (which completes empty and unsupported triggers).  Every
+// workgroup computes the same number from the trigger words alone, so the ones
+// left out neither work nor report in -- a small trigger costs a few counter
+// updates instead of one per workgroup.
+__device__ __forceinline__ uint32_t participants(const void *in1, const void *in2, void *out, uint64_t count, int dtype,
+                                                 int op) {
+  const int es = (int)dtypeSize(dtype);
+  if (es == 0 || count == 0 || op < flagcxSum || op > flagcxMin) return 1;
+  const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
+  const bool co = (((uint64_t)(uintptr_t)in1 & 15u) == mis) && (((uint64_t)(uintptr_t)in2 & 15u) == mis);
+  const uint64_t tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, co).tiles();
+  return (uint32_t)(tiles < gridDim.x ? (tiles ? tiles : 1) : gridDim.x);
+}
+
 // Clears the mirror before a consumer launch.  A kernel rather than a memset
 // node so that the launch sequence stays safe to record into a HIP graph.
 __global__ void __launch_bounds__(kBlock) clearMirror(uint64_t *words, uint32_t n) {
@@ -168,6 +183,12 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
     const uint64_t count = w3 & 0xffffffffull;
     const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
     bool ok = true;
+    const uint32_t takers = participants(in1, in2, out, count, dtype, op);
+    if (blockIdx.x >= takers) {  // not needed for this trigger
+      seq++;
+      __syncthreads();
+      continue;
+    }
     if (count) {
       switch (dtype) {
         case flagcxFloat32: ok = runShareOp<flagcxFloat32>(op, in1, in2, out, count); break;
@@ -188,7 +209,7 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       const uint32_t slot = (uint32_t)(seq % cap);
       __threadfence();  // this workgroup's stores are out before it reports in
       const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-      if (prev == gridDim.x - 1) {  // last one out completes the trigger
+      if (prev == takers - 1) {  // last one out completes the trigger
         __hip_atomic_store(&m->done[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (!ok) __hip_atomic_fetch_add(&m->badTriggers, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __threadfence_system();
@@ -286,7 +307,11 @@ int fx_fifo_consumer_create(fxFifoConsumer_t *consumer, size_t capacity) {
     return flagcxUnhandledDeviceError;
   }
   c->capacity = (uint32_t)capacity;
-  c->grid = (uint32_t)(cus > 0 ? cus : 1);  // one resident workgroup per CU
+  int perCu = 1;  // resident workgroups per CU
+  if (const char *e = getenv("FX_FIFO_WGS_PER_CU")) perCu = atoi(e);
+  if (perCu < 1) perCu = 1;
+  if (perCu > 8) perCu = 8;
+  c->grid = (uint32_t)((cus > 0 ? cus : 1) * perCu);
   *consumer = c;
   return flagcxSuccess;
 }

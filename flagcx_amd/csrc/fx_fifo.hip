@@ -12,11 +12,12 @@
 //   to Available; `terminate` = 1 ends the consumer once the ring is drained.
 //
 // What differs from the reference's consumer (one block of 32 threads that
-// dequeues with a CAS and runs the reduce itself): here EVERY workgroup of a
-// full-width grid works on every trigger -- workgroup w takes tiles w, w+G, ...
-// of it -- and the last workgroup to finish marks it Complete.  Workgroup 0
-// alone reads the pinned host ring (over PCIe) and mirrors it into device
-// memory, where the other workgroups poll it.  Nothing waits on another
+// dequeues with a CAS and runs the reduce itself): here a full-width grid
+// shares every trigger -- one workgroup per 16 KiB tile, all of them for a large
+// trigger, taking tiles idx, idx + takers, ... -- and the last workgroup to
+// finish marks it Complete.  Workgroup 0 does no arithmetic: it alone reads the
+// pinned host ring (over PCIe) and mirrors it into device memory, where the
+// other workgroups poll it.  Nothing waits on another
 // workgroup, so the kernel cannot deadlock on residency; every polling loop is
 // bounded by maxIdlePolls.  Triggers that are in the ring at the same time must
 // be independent of each other, which is how the reference's scheduler uses it
@@ -68,41 +69,69 @@ __device__ __forceinline__ void storeSys(T *p, T v) {
   __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// Which part of a trigger a workgroup takes: tiles idx, idx + takers, ...;
+// idx >= takers means none.
+struct Share {
+  uint32_t idx, takers;
+};
+
 // This workgroup's share of one two-input trigger.
 template <int DT, int OP>
-__device__ __forceinline__ void runShare(const void *in1, const void *in2, void *out, uint64_t count) {
+__device__ __forceinline__ void runShare(const void *in1, const void *in2, void *out, uint64_t count, Share sh) {
   using R = Red<DT, OP>;
   const void *in[2] = {in1, in2};
   Seg<2> sg;
   const TilePlan tp = makeSeg<R::ES, kFifoU>(sg, in, out, count, 2);
   const uint64_t tiles = tp.tiles();
-  for (uint64_t t = blockIdx.x; t < tiles; t += gridDim.x) reduceTile<R, 2, kFifoU>(sg, tp, (uint32_t)t);
+  for (uint64_t t = sh.idx; t < tiles; t += sh.takers) reduceTile<R, 2, kFifoU>(sg, tp, (uint32_t)t);
 }
 
 template <int DT>
-__device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b, void *o, uint64_t n) {
+__device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b, void *o, uint64_t n, Share sh) {
   switch (op) {
-    case flagcxSum: runShare<DT, flagcxSum>(a, b, o, n); return true;
-    case flagcxProd: runShare<DT, flagcxProd>(a, b, o, n); return true;
-    case flagcxMax: runShare<DT, flagcxMax>(a, b, o, n); return true;
-    case flagcxMin: runShare<DT, flagcxMin>(a, b, o, n); return true;
+    case flagcxSum: runShare<DT, flagcxSum>(a, b, o, n, sh); return true;
+    case flagcxProd: runShare<DT, flagcxProd>(a, b, o, n, sh); return true;
+    case flagcxMax: runShare<DT, flagcxMax>(a, b, o, n, sh); return true;
+    case flagcxMin: runShare<DT, flagcxMin>(a, b, o, n, sh); return true;
     default: return false;
   }
 }
 
-// Workgroups that take part in one trigger: one per tile, at most the grid,
-// at least one (which completes empty and unsupported triggers).  Every
-// workgroup computes the same number from the trigger words alone, so the ones
-// left out neither work nor report in -- a small trigger costs a few counter
-// updates instead of one per workgroup.
-__device__ __forceinline__ uint32_t participants(const void *in1, const void *in2, void *out, uint64_t count, int dtype,
-                                                 int op) {
+// Who works on trigger number seq.  One workgroup per 16 KiB tile, at least one
+// (which completes empty and unsupported triggers), at most G-1: workgroup 0
+// never computes, so it is always free to talk to the host, and the workers of
+// a small trigger start at a position that rotates with seq, so consecutive
+// small triggers run side by side on different workgroups.  Every workgroup
+// computes the same answer from the trigger words alone, so the ones left out
+// neither work nor report in.
+__device__ __forceinline__ Share shareOf(uint64_t seq, const void *in1, const void *in2, void *out, uint64_t count,
+                                         int dtype, int op) {
+  const uint32_t grid = gridDim.x;
   const int es = (int)dtypeSize(dtype);
-  if (es == 0 || count == 0 || op < flagcxSum || op > flagcxMin) return 1;
-  const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
-  const bool co = (((uint64_t)(uintptr_t)in1 & 15u) == mis) && (((uint64_t)(uintptr_t)in2 & 15u) == mis);
-  const uint64_t tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, co).tiles();
-  return (uint32_t)(tiles < gridDim.x ? (tiles ? tiles : 1) : gridDim.x);
+  uint64_t tiles = 1;
+  if (es != 0 && count != 0 && op >= flagcxSum && op <= flagcxMin) {
+    const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
+    const bool co = (((uint64_t)(uintptr_t)in1 & 15u) == mis) && (((uint64_t)(uintptr_t)in2 & 15u) == mis);
+    tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, co).tiles();
+    if (tiles == 0) tiles = 1;
+  }
+  Share sh;
+  if (grid == 1) {  // a one-workgroup launch does everything itself
+    sh.takers = 1;
+    sh.idx = 0;
+    return sh;
+  }
+  const uint32_t pool = grid - 1, rot = (uint32_t)((seq * 61u) % pool);
+  sh.takers = (uint32_t)(tiles < pool ? tiles : pool);
+  sh.idx = (blockIdx.x == 0) ? sh.takers : (blockIdx.x - 1 + pool - rot) % pool;
+  return sh;
+}
+
+// Value of lane `src` of the wavefront as a wave-uniform 64-bit scalar.
+__device__ __forceinline__ uint64_t fromLane(uint64_t v, int src) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, src);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), src);
+  return ((uint64_t)hi << 32) | lo;
 }
 
 // Clears the mirror before a consumer launch.  A kernel rather than a memset
@@ -113,42 +142,68 @@ __global__ void __launch_bounds__(kBlock) clearMirror(uint64_t *words, uint32_t 
 
 __global__ void __launch_bounds__(kBlock)
 fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uint64_t maxIdlePolls) {
-  __shared__ uint64_t sh[6];  // [0] state, [1..4] trigger words, [5] scratch
+  __shared__ uint64_t sh[6];  // [0] state, [1..4] trigger words
   enum { kWork = 0, kExitTerminate = FX_FIFO_EXIT_TERMINATE, kExitIdle = FX_FIFO_EXIT_IDLE };
   uint64_t seq = startSeq;
   uint64_t *hostTrig = host + 4;
-  uint64_t mirrored = startSeq;      // workgroup 0: triggers copied to the mirror so far
-  uint64_t lastPublished = ~0ull;    // workgroup 0: last `completed` written to the host's `consumed`
+  // workgroup 0, wavefront 0 (all of these stay wave-uniform):
+  uint64_t mirrored = startSeq;      // triggers copied to the mirror so far
+  uint64_t lastPublished = ~0ull;    // last `completed` written to the host's `consumed`
   bool hostTermSeen = false;
+  const uint32_t lane = threadIdx.x;
   for (;;) {
-    if (threadIdx.x == 0) {
+    if (threadIdx.x < 64) {
+      // Wavefront 0 does the polling.  Reads over PCIe cost microseconds each, so
+      // they are issued by different lanes of one instruction and the results are
+      // broadcast; every branch below depends on broadcast values only.
       uint64_t idle = 0, state;
       bool termSeen = false;
       for (;;) {
+        uint64_t p, term;
         if (blockIdx.x == 0) {
-          const uint64_t hp = pollSys(host + 2), ht = pollSys(host + 3);
-          if (mirrored < hp) {
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // the triggers behind `produced`
-            for (; mirrored < hp; mirrored++) {
-              const uint32_t slot = (uint32_t)(mirrored % cap);
-              for (int w = 0; w < 4; w++) m->trig[slot][w] = pollSys(hostTrig + 4 * slot + w);
+          if (mirrored <= seq) {  // nothing mirrored is waiting for this workgroup: talk to the host
+            uint64_t v = 0;
+            if (lane < 2) v = pollSys(host + 2 + lane);
+            const uint64_t hp = fromLane(v, 0), ht = fromLane(v, 1);
+            if (mirrored < hp) {
+              __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // the triggers behind `produced`
+              const uint64_t words = 4 * (hp - mirrored);     // at most 4 * capacity
+              for (uint64_t w = lane; w < words; w += 64) {
+                const uint32_t slot = (uint32_t)((mirrored + w / 4) % cap);
+                m->trig[slot][w & 3] = pollSys(hostTrig + 4 * slot + (w & 3));
+              }
+              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // every lane's copies before the new count
+              mirrored = hp;
+              if (lane == 0) __hip_atomic_store(&m->produced, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            storeDev(&m->produced, hp);  // release: the mirrored triggers are visible first
+            // The host sets terminate after its last enqueue, but two relaxed
+            // polls may be served out of order: act on terminate only on the poll
+            // AFTER the one that first saw it, when `produced` has been re-read.
+            if (ht) {
+              if (hostTermSeen && lane == 0) storeDev(&m->terminate, ht);
+              hostTermSeen = true;
+            }
+            uint64_t c = 0;
+            if (lane == 0) c = pollDev(&m->completed);
+            c = fromLane(c, 0);
+            if (c != lastPublished) {
+              if (lane == 0) storeSys(host + 1, startSeq + c);  // consumed
+              lastPublished = c;
+            }
           }
-          // The host sets terminate after its last enqueue, but two relaxed
-          // polls may be served out of order: act on terminate only on the poll
-          // AFTER the one that first saw it, when `produced` has been re-read.
-          if (ht) {
-            if (hostTermSeen) storeDev(&m->terminate, ht);
-            hostTermSeen = true;
+          uint64_t t = 0;
+          if (lane == 0) t = pollDev(&m->terminate);
+          term = fromLane(t, 0);
+          p = mirrored;
+        } else {
+          uint64_t t = 0, q = 0;
+          if (lane == 0) {
+            t = pollDev(&m->terminate);
+            q = pollDev(&m->produced);
           }
-          const uint64_t c = pollDev(&m->completed);
-          if (c != lastPublished) {
-            storeSys(host + 1, startSeq + c);  // consumed
-            lastPublished = c;
-          }
+          term = fromLane(t, 0);
+          p = fromLane(q, 0);
         }
-        const uint64_t term = pollDev(&m->terminate), p = pollDev(&m->produced);
         if (p > seq) { state = kWork; break; }
         if (term) {
           if (termSeen) { state = kExitTerminate; break; }  // same two-step rule as above
@@ -158,11 +213,13 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
         if (++idle > maxIdlePolls) { state = kExitIdle; break; }
         __builtin_amdgcn_s_sleep(32);
       }
-      sh[0] = state;
-      if (state == kWork) {
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        const uint32_t slot = (uint32_t)(seq % cap);
-        for (int w = 0; w < 4; w++) sh[1 + w] = m->trig[slot][w];
+      if (lane == 0) {
+        sh[0] = state;
+        if (state == kWork) {
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+          const uint32_t slot = (uint32_t)(seq % cap);
+          for (int w = 0; w < 4; w++) sh[1 + w] = m->trig[slot][w];
+        }
       }
     }
     __syncthreads();
@@ -174,42 +231,43 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       }
       break;
     }
-    // The trigger's buffers may have been written by other agents since this
-    // kernel last looked: drop stale cache lines before reading them.
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
     const void *in1 = (const void *)(uintptr_t)sh[1], *in2 = (const void *)(uintptr_t)sh[2];
     void *out = (void *)(uintptr_t)sh[3];
     const uint64_t w3 = sh[4];
     const uint64_t count = w3 & 0xffffffffull;
     const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
-    bool ok = true;
-    const uint32_t takers = participants(in1, in2, out, count, dtype, op);
-    if (blockIdx.x >= takers) {  // not needed for this trigger
+    const Share share = shareOf(seq, in1, in2, out, count, dtype, op);
+    if (share.idx >= share.takers) {  // not needed for this trigger
       seq++;
       __syncthreads();
       continue;
     }
+    // The trigger's buffers may have been written by other agents since this
+    // kernel last looked: drop stale cache lines before reading them.
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    bool ok = true;
     if (count) {
       switch (dtype) {
-        case flagcxFloat32: ok = runShareOp<flagcxFloat32>(op, in1, in2, out, count); break;
-        case flagcxInt32: ok = runShareOp<flagcxInt32>(op, in1, in2, out, count); break;
-        case flagcxBfloat16: ok = runShareOp<flagcxBfloat16>(op, in1, in2, out, count); break;
-        case flagcxFloat16: ok = runShareOp<flagcxFloat16>(op, in1, in2, out, count); break;
-        case flagcxUint32: ok = runShareOp<flagcxUint32>(op, in1, in2, out, count); break;
-        case flagcxInt8: ok = runShareOp<flagcxInt8>(op, in1, in2, out, count); break;
-        case flagcxUint8: ok = runShareOp<flagcxUint8>(op, in1, in2, out, count); break;
-        case flagcxInt64: ok = runShareOp<flagcxInt64>(op, in1, in2, out, count); break;
-        case flagcxUint64: ok = runShareOp<flagcxUint64>(op, in1, in2, out, count); break;
-        case flagcxFloat64: ok = runShareOp<flagcxFloat64>(op, in1, in2, out, count); break;
+        case flagcxFloat32: ok = runShareOp<flagcxFloat32>(op, in1, in2, out, count, share); break;
+        case flagcxInt32: ok = runShareOp<flagcxInt32>(op, in1, in2, out, count, share); break;
+        case flagcxBfloat16: ok = runShareOp<flagcxBfloat16>(op, in1, in2, out, count, share); break;
+        case flagcxFloat16: ok = runShareOp<flagcxFloat16>(op, in1, in2, out, count, share); break;
+        case flagcxUint32: ok = runShareOp<flagcxUint32>(op, in1, in2, out, count, share); break;
+        case flagcxInt8: ok = runShareOp<flagcxInt8>(op, in1, in2, out, count, share); break;
+        case flagcxUint8: ok = runShareOp<flagcxUint8>(op, in1, in2, out, count, share); break;
+        case flagcxInt64: ok = runShareOp<flagcxInt64>(op, in1, in2, out, count, share); break;
+        case flagcxUint64: ok = runShareOp<flagcxUint64>(op, in1, in2, out, count, share); break;
+        case flagcxFloat64: ok = runShareOp<flagcxFloat64>(op, in1, in2, out, count, share); break;
         default: ok = false;
       }
     }
     __syncthreads();
     if (threadIdx.x == 0) {
       const uint32_t slot = (uint32_t)(seq % cap);
-      __threadfence();  // this workgroup's stores are out before it reports in
+      // Release: with the barrier above, this workgroup's stores are out before
+      // it reports in.  Acquire: the last one in has everybody's stores behind it.
       const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-      if (prev == takers - 1) {  // last one out completes the trigger
+      if (prev == share.takers - 1) {  // last one out completes the trigger
         __hip_atomic_store(&m->done[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (!ok) __hip_atomic_fetch_add(&m->badTriggers, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __threadfence_system();

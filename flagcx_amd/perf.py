@@ -186,6 +186,25 @@ def run_fifo(dev, a):
                 one(n)
             ms = (time.perf_counter() - t0) * 1e3 / 20
             row("fifo round trip, fp32 sum, 2 inputs", nbytes, ms, 3 * nbytes)
+            # the ring kept full: 256 independent triggers, collected as they complete
+            if 3 * nbytes * 64 <= emax * 3:
+                span = emax // (64 * 4) * 4                      # 64 disjoint windows of the buffers
+                n = min(n, span // 4)
+                pending, done, t0 = [], 0, time.perf_counter()
+                issued = 0
+                while done < 256:
+                    if issued < 256:
+                        off = (issued % 64) * span
+                        lib.fx_fifo_enqueue(host, bufs[0] + off, bufs[1] + off, bufs[2] + off, n, 32, N.DT_FP32,
+                                            N.OP_SUM, C.byref(idx))
+                        if idx.value >= 0:
+                            pending.append(idx.value)
+                            issued += 1
+                    if pending and lib.fx_fifo_poll_state(host, pending[0]) == 3:
+                        lib.fx_fifo_set_state(host, pending.pop(0), 0)
+                        done += 1
+                ms = (time.perf_counter() - t0) * 1e3 / 256
+                row("fifo ring kept full, per trigger", n * 4, ms, 3 * n * 4)
             nbytes *= a.factor
     finally:
         lib.fx_fifo_terminate(host)

@@ -133,7 +133,21 @@ def main():
         dev.event_destroy(e1)
         return wall * 1e3 / steps, ev_ms / steps
 
+    def per_launch(dst, steps):
+        """Durations of individual launches: one event between consecutive steps."""
+        ev = [dev.event_create() for _ in range(steps + 1)]
+        dev.event_record(ev[0], stream)
+        for i in range(steps):
+            step(dst)
+            dev.event_record(ev[i + 1], stream)
+        dev.sync()
+        ms = sorted(dev.event_ms(ev[i], ev[i + 1]) for i in range(steps))
+        for e in ev:
+            dev.event_destroy(e)
+        return ms
+
     wall_ms, kern_ms = timed(out, args.steps, args.warmup)
+    each = per_launch(out, 20)
     _, inplace_ms = timed(ins[0], max(args.steps // 2, 1), 2)      # out = in[0]; destroys input 0, run last
     gbs = algo_bytes / (wall_ms * 1e-3) / 1e9
     kern_gbs = algo_bytes / (kern_ms * 1e-3) / 1e9
@@ -151,7 +165,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(kern_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kern_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "reduceCopyDirect<Red<bf16,sum>,8,8>", "bytes_per_launch": algo_bytes,
-                     "avg_launch_ms": round(kern_ms, 4)},
+                     "avg_launch_ms": round(kern_ms, 4), "min_launch_ms": round(each[0], 4),
+                     "median_launch_ms": round(each[len(each) // 2], 4)},
     }
     for p in ins + [out]:
         dev.free(p)

@@ -20,7 +20,7 @@ flagcxResult_t screen(int dtype, int op) {
   if (dtype < 0 || dtype >= flagcxNumTypes) return flagcxInvalidArgument;
   if (op < 0 || op >= flagcxNumRedOps) return flagcxInvalidArgument;
   if (dtypeSize(dtype) == 0) return flagcxNotSupported;
-  if (!opSupported(op)) return flagcxNotSupported;  // flagcxAvg
+  if (!opSupported(op)) return flagcxNotSupported;
   return flagcxSuccess;
 }
 

@@ -31,7 +31,7 @@ __host__ __device__ inline size_t dtypeSize(int dt) {
   }
 }
 
-inline bool opSupported(int op) { return op >= flagcxSum && op <= flagcxMin; }
+inline bool opSupported(int op) { return op >= flagcxSum && op <= flagcxAvg; }
 
 #define FX_HIP(call)                                                           \
   do {                                                                         \

@@ -93,6 +93,7 @@ __device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b,
     case flagcxProd: runShare<DT, flagcxProd>(a, b, o, n, sh); return true;
     case flagcxMax: runShare<DT, flagcxMax>(a, b, o, n, sh); return true;
     case flagcxMin: runShare<DT, flagcxMin>(a, b, o, n, sh); return true;
+    case flagcxAvg: runShare<DT, flagcxAvg>(a, b, o, n, sh); return true;
     default: return false;
   }
 }
@@ -109,7 +110,7 @@ __device__ __forceinline__ Share shareOf(uint64_t seq, const void *in1, const vo
   const uint32_t grid = gridDim.x;
   const int es = (int)dtypeSize(dtype);
   uint64_t tiles = 1;
-  if (es != 0 && count != 0 && op >= flagcxSum && op <= flagcxMin) {
+  if (es != 0 && count != 0 && op >= flagcxSum && op <= flagcxAvg) {
     const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
     const bool co = (((uint64_t)(uintptr_t)in1 & 15u) == mis) && (((uint64_t)(uintptr_t)in2 & 15u) == mis);
     tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, co).tiles();

@@ -125,8 +125,9 @@ KernelSet makeCopySet() {
 
 template <int DT>
 const KernelSet *makeSets() {
-  static const KernelSet sets[4] = {makeSet<Red<DT, flagcxSum>>(), makeSet<Red<DT, flagcxProd>>(),
-                                    makeSet<Red<DT, flagcxMax>>(), makeSet<Red<DT, flagcxMin>>()};
+  static const KernelSet sets[5] = {makeSet<Red<DT, flagcxSum>>(), makeSet<Red<DT, flagcxProd>>(),
+                                    makeSet<Red<DT, flagcxMax>>(), makeSet<Red<DT, flagcxMin>>(),
+                                    makeSet<Red<DT, flagcxAvg>>()};  // indexed by flagcxRedOp_t
   return sets;
 }
 

@@ -12,6 +12,11 @@
 //   min = (x < acc) ? x : acc (the std::max / std::min of
 //   flagcx/service/include/utils.h:707-725: ties and NaN keep the earlier
 //   operand); for 16-bit types the chosen input's own bits are returned.
+//   avg = the sum above divided once by the number of inputs before the final
+//   rounding: IEEE division for the floating types (16-bit: in fp32), C division
+//   (truncating toward zero, on the wrapped sum) for signed integers, unsigned
+//   division for unsigned ones.  FlagCX itself only forwards avg to vendor
+//   libraries, so this definition is this path's own.
 //
 // Data movement: one 16-byte vector per lane per input, U vectors per lane in
 // flight per input, all K*U loads issued before the first use.  The index
@@ -29,9 +34,12 @@ namespace fx {
 
 // ------------------------------------------------------------------ reducers
 
+// avg accumulates like sum and divides in finish().
+constexpr bool isAdd(int op) { return op == flagcxSum || op == flagcxAvg; }
+
 template <int OP>
 __device__ __forceinline__ float opF32(float a, float b) {
-  if (OP == flagcxSum) return a + b;
+  if (isAdd(OP)) return a + b;
   if (OP == flagcxProd) return a * b;
   if (OP == flagcxMax) return (a < b) ? b : a;
   return (b < a) ? b : a;
@@ -39,7 +47,7 @@ __device__ __forceinline__ float opF32(float a, float b) {
 
 template <int OP>
 __device__ __forceinline__ uint32_t opI32(uint32_t a, uint32_t b) {
-  if (OP == flagcxSum) return a + b;
+  if (isAdd(OP)) return a + b;
   if (OP == flagcxProd) return a * b;
   if (OP == flagcxMax) return ((int32_t)a < (int32_t)b) ? b : a;
   return ((int32_t)b < (int32_t)a) ? b : a;
@@ -77,10 +85,10 @@ struct Red<flagcxFloat32, OP> {
 #pragma unroll
     for (int i = 0; i < 4; i++) c.a[i] = opF32<OP>(c.a[i], __uint_as_float(v[i]));
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
     u32x4 r;
 #pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = __float_as_uint(c.a[i]);
+    for (int i = 0; i < 4; i++) r[i] = __float_as_uint(OP == flagcxAvg ? c.a[i] / (float)k : c.a[i]);
     return r;
   }
 };
@@ -99,10 +107,10 @@ struct Red<flagcxInt32, OP> {
 #pragma unroll
     for (int i = 0; i < 4; i++) c.a[i] = opI32<OP>(c.a[i], v[i]);
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
     u32x4 r;
 #pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = c.a[i];
+    for (int i = 0; i < 4; i++) r[i] = (OP == flagcxAvg) ? (uint32_t)((int32_t)c.a[i] / (int32_t)k) : c.a[i];
     return r;
   }
 };
@@ -115,7 +123,7 @@ struct Red<flagcxUint32, OP> {
     uint32_t a[4];
   };
   static __device__ __forceinline__ uint32_t op(uint32_t a, uint32_t b) {
-    if (OP == flagcxSum) return a + b;
+    if (isAdd(OP)) return a + b;
     if (OP == flagcxProd) return a * b;
     if (OP == flagcxMax) return (a < b) ? b : a;
     return (b < a) ? b : a;
@@ -128,10 +136,10 @@ struct Red<flagcxUint32, OP> {
 #pragma unroll
     for (int i = 0; i < 4; i++) c.a[i] = op(c.a[i], v[i]);
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
     u32x4 r;
 #pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = c.a[i];
+    for (int i = 0; i < 4; i++) r[i] = (OP == flagcxAvg) ? c.a[i] / k : c.a[i];
     return r;
   }
 };
@@ -149,7 +157,7 @@ struct Red8 {
     return SIGNED ? ((int32_t)(w << (24 - 8 * b)) >> 24) : (int32_t)((w >> (8 * b)) & 0xffu);
   }
   static __device__ __forceinline__ int32_t op(int32_t a, int32_t b) {
-    if (OP == flagcxSum) return (int32_t)((uint32_t)a + (uint32_t)b);
+    if (isAdd(OP)) return (int32_t)((uint32_t)a + (uint32_t)b);
     if (OP == flagcxProd) return (int32_t)((uint32_t)a * (uint32_t)b);
     if (OP == flagcxMax) return (a < b) ? b : a;
     return (b < a) ? b : a;
@@ -162,12 +170,18 @@ struct Red8 {
 #pragma unroll
     for (int i = 0; i < 16; i++) c.a[i] = op(c.a[i], lane(v[i / 4], i & 3));
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+  // avg divides the sum as it would read in 8 bits (wrapped), not the wide accumulator
+  static __device__ __forceinline__ uint32_t byteOf(int32_t a, uint32_t k) {
+    if (OP != flagcxAvg) return (uint32_t)a & 0xffu;
+    if (SIGNED) return (uint32_t)(((int32_t)(a << 24) >> 24) / (int32_t)k) & 0xffu;
+    return ((uint32_t)a & 0xffu) / k;
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
     u32x4 r;
 #pragma unroll
     for (int i = 0; i < 4; i++)
-      r[i] = ((uint32_t)c.a[4 * i] & 0xffu) | (((uint32_t)c.a[4 * i + 1] & 0xffu) << 8) |
-             (((uint32_t)c.a[4 * i + 2] & 0xffu) << 16) | ((uint32_t)c.a[4 * i + 3] << 24);
+      r[i] = byteOf(c.a[4 * i], k) | (byteOf(c.a[4 * i + 1], k) << 8) | (byteOf(c.a[4 * i + 2], k) << 16) |
+             (byteOf(c.a[4 * i + 3], k) << 24);
     return r;
   }
 };
@@ -184,7 +198,7 @@ struct RedI64 {
     uint64_t a[2];
   };
   static __device__ __forceinline__ uint64_t op(uint64_t a, uint64_t b) {
-    if (OP == flagcxSum) return a + b;
+    if (isAdd(OP)) return a + b;
     if (OP == flagcxProd) return a * b;
     const bool lt = SIGNED ? ((int64_t)a < (int64_t)b) : (a < b);
     const bool gt = SIGNED ? ((int64_t)b < (int64_t)a) : (b < a);
@@ -202,8 +216,13 @@ struct RedI64 {
     c.a[0] = op(c.a[0], word(v, 0));
     c.a[1] = op(c.a[1], word(v, 1));
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
-    u32x4 r = {(uint32_t)c.a[0], (uint32_t)(c.a[0] >> 32), (uint32_t)c.a[1], (uint32_t)(c.a[1] >> 32)};
+  static __device__ __forceinline__ uint64_t mean(uint64_t a, uint32_t k) {
+    if (OP != flagcxAvg) return a;
+    return SIGNED ? (uint64_t)((int64_t)a / (int64_t)k) : a / (uint64_t)k;
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
+    const uint64_t x = mean(c.a[0], k), y = mean(c.a[1], k);
+    u32x4 r = {(uint32_t)x, (uint32_t)(x >> 32), (uint32_t)y, (uint32_t)(y >> 32)};
     return r;
   }
 };
@@ -219,7 +238,7 @@ struct Red<flagcxFloat64, OP> {
     double a[2];
   };
   static __device__ __forceinline__ double op(double a, double b) {
-    if (OP == flagcxSum) return a + b;
+    if (isAdd(OP)) return a + b;
     if (OP == flagcxProd) return a * b;
     if (OP == flagcxMax) return (a < b) ? b : a;
     return (b < a) ? b : a;
@@ -235,8 +254,9 @@ struct Red<flagcxFloat64, OP> {
     c.a[0] = op(c.a[0], word(v, 0));
     c.a[1] = op(c.a[1], word(v, 1));
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
-    const uint64_t x = (uint64_t)__double_as_longlong(c.a[0]), y = (uint64_t)__double_as_longlong(c.a[1]);
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
+    const double d0 = (OP == flagcxAvg) ? c.a[0] / (double)k : c.a[0], d1 = (OP == flagcxAvg) ? c.a[1] / (double)k : c.a[1];
+    const uint64_t x = (uint64_t)__double_as_longlong(d0), y = (uint64_t)__double_as_longlong(d1);
     u32x4 r = {(uint32_t)x, (uint32_t)(x >> 32), (uint32_t)y, (uint32_t)(y >> 32)};
     return r;
   }
@@ -264,12 +284,15 @@ struct Red<flagcxBfloat16, OP> {
       c.a[2 * i + 1] = opF32<OP>(c.a[2 * i + 1], __uint_as_float(v[i] & 0xffff0000u));
     }
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
     u32x4 r;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       uint32_t lo, hi;
-      if (OP == flagcxSum || OP == flagcxProd) {
+      if (OP == flagcxAvg) {
+        lo = roundBf16Top(c.a[2 * i] / (float)k);
+        hi = roundBf16Top(c.a[2 * i + 1] / (float)k);
+      } else if (OP == flagcxSum || OP == flagcxProd) {
         lo = roundBf16Top(c.a[2 * i]);
         hi = roundBf16Top(c.a[2 * i + 1]);
       } else {
@@ -321,7 +344,7 @@ struct Red<flagcxFloat16, OP> {
       fold1(c, 2 * i + 1, v[i] >> 16);
     }
   }
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) {
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t k) {
     u32x4 r;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -329,6 +352,9 @@ struct Red<flagcxFloat16, OP> {
       if (kSelect) {
         lo = c.b[2 * i];
         hi = c.b[2 * i + 1];
+      } else if (OP == flagcxAvg) {
+        lo = f32ToHalf(c.a[2 * i] / (float)k);
+        hi = f32ToHalf(c.a[2 * i + 1] / (float)k);
       } else {
         lo = f32ToHalf(c.a[2 * i]);
         hi = f32ToHalf(c.a[2 * i + 1]);
@@ -349,7 +375,7 @@ struct CopyRed {
   };
   static __device__ __forceinline__ void init(Acc &c, u32x4 v) { c.v = v; }
   static __device__ __forceinline__ void fold(Acc &, u32x4) {}
-  static __device__ __forceinline__ u32x4 finish(const Acc &c) { return c.v; }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t) { return c.v; }
 };
 
 // ------------------------------------------------------------- one segment
@@ -545,7 +571,7 @@ __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
   };
   R::init(acc, fetch(0));
   for (int p = 1; p < k; p++) R::fold(acc, fetch(p));
-  u32x4 r = R::finish(acc);
+  u32x4 r = R::finish(acc, (uint32_t)k);
   if (full)
     storeVector(sg, j * 16, r);
   else
@@ -568,7 +594,7 @@ __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, ui
       R::init(acc, v[u][0]);
 #pragma unroll
       for (int p = 1; p < K; p++) R::fold(acc, v[u][p]);
-      storeVector(sg, off + u * ustride, R::finish(acc));
+      storeVector(sg, off + u * ustride, R::finish(acc, (uint32_t)K));
     }
   } else {
     typename R::Acc acc[U];
@@ -583,7 +609,7 @@ __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, ui
       for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
     }
 #pragma unroll
-    for (int u = 0; u < U; u++) storeVector(sg, off + u * ustride, R::finish(acc[u]));
+    for (int u = 0; u < U; u++) storeVector(sg, off + u * ustride, R::finish(acc[u], (uint32_t)sg.inputs()));
   }
 }
 

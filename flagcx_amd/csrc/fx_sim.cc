@@ -190,7 +190,7 @@ flagcxResult_t runAllReduce(const Ctx &c) {
   }
   const size_t nred = fx_nredslices(count, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
   std::vector<fxSliceDesc> descs;
-  if (g->algo == FX_ALGO_RING) {
+  if (g->algo == FX_ALGO_RING && g->op != flagcxAvg) {  // a mean is not a chain of two-input means
     // reduce-scatter: step i, rank r reduces chunk (r-i-1)%n: partial from the
     // previous rank (its sendbuff at step 0, its recvbuff afterwards) + own data.
     for (int i = 0; i < n - 1; i++) {
@@ -297,7 +297,7 @@ flagcxResult_t runReduce(const Ctx &c) {
   const int n = c.n, root = g->root;
   const size_t count = g->count, ts = c.ts;
   if (count == 0) return flagcxSuccess;
-  if (g->order != FX_ORDER_TREE || n == 1) {
+  if (g->order != FX_ORDER_TREE || n == 1 || g->op == flagcxAvg) {
     std::vector<const void *> in(n);
     for (int j = 0; j < n; j++) in[j] = c.send(j);
     return R(fx_reduce_copy(c.recv(root), in.data(), n, count, g->dtype, g->op, 0, c.s));
@@ -344,7 +344,7 @@ flagcxResult_t runReduceScatter(const Ctx &c) {
   }
   const size_t nred = fx_nredslices(rcount, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
   std::vector<fxSliceDesc> descs;
-  if (g->algo == FX_ALGO_RING) {
+  if (g->algo == FX_ALGO_RING && g->op != flagcxAvg) {  // a mean is not a chain of two-input means
     // Per-rank scratch of n*recvcount elements holds the travelling partials.
     flagcxResult_t rc = ensureScratch(g, (size_t)n * n * rcount * ts);
     if (rc != flagcxSuccess) return rc;
@@ -700,7 +700,6 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
 // kernel layer (unsupported-but-known -> flagcxNotSupported).
 flagcxResult_t screenReduce(int dtype, int op) {
   if (dtype < 0 || dtype >= flagcxNumTypes || op < 0 || op >= flagcxNumRedOps) return flagcxInvalidArgument;
-  if (op > flagcxMin) return flagcxNotSupported;
   return flagcxSuccess;
 }
 

@@ -8,9 +8,13 @@
  * default stream); all launches are enqueue-only.  dtype / op are FlagCX enum
  * values (flagcx/include/flagcx.h:36-66): int8 = 0, uint8 = 1, int32 = 2,
  * uint32 = 3, int64 = 4, uint64 = 5, fp16 = 6, fp32 = 7, fp64 = 8, bf16 = 9;
- * sum = 0, prod = 1, max = 2, min = 3.  All ten types are carried; avg = 4 is
- * answered with 9.  Integer sum / prod wrap modulo 2^width, as the host loops
- * of flagcx/service/include/utils.h:664-725 do.
+ * sum = 0, prod = 1, max = 2, min = 3, avg = 4.  All ten types and five ops
+ * are carried.  Integer sum / prod wrap modulo 2^width, as the host loops of
+ * flagcx/service/include/utils.h:664-725 do.  avg is the sum divided once by
+ * the number of inputs (IEEE division before the final rounding; C division of
+ * the wrapped sum for integers): FlagCX only forwards avg to vendor libraries
+ * (flagcx/adaptor/ccl/rccl_adaptor.cc:124,200), so this definition is this
+ * library's own.
  */
 #ifndef FLAGCX_AMD_FX_KERNELS_H_
 #define FLAGCX_AMD_FX_KERNELS_H_

@@ -26,6 +26,11 @@
  *   prod (all dtypes) ......................... PARITY UNPINNED by the
  *       reference (it rejects prod, service/bootstrap.cc:872-874); defined as
  *       acc*=x left to right and checked against numpy only.
+ *   avg (all dtypes) .......................... PARITY UNPINNED by the
+ *       reference (it only forwards avg to vendor libraries and rejects it on
+ *       its own host path, service/bootstrap.cc:872-874); defined as the sum
+ *       divided once by k (IEEE division before the final rounding; C division
+ *       of the wrapped sum for integers) and checked against numpy only.
  *   oracle_split / plans ...................... tiling invariants + closed
  *       forms of the reference's divisible cases.
  *   oracle_tree_reduce ........................ hand-derived associations for
@@ -49,7 +54,7 @@ enum {
   DT_INT8 = 0, DT_UINT8 = 1, DT_INT32 = 2, DT_UINT32 = 3, DT_INT64 = 4, DT_UINT64 = 5,
   DT_FP16 = 6, DT_FP32 = 7, DT_FP64 = 8, DT_BF16 = 9
 };
-enum { OP_SUM = 0, OP_PROD = 1, OP_MAX = 2, OP_MIN = 3 };
+enum { OP_SUM = 0, OP_PROD = 1, OP_MAX = 2, OP_MIN = 3, OP_AVG = 4 };
 enum { RC_OK = 0, RC_INVALID = 4, RC_UNSUPPORTED = 9 };
 
 static int g_threads = 1;
@@ -148,6 +153,7 @@ uint16_t oracle_f32_to_f16(float f) {
  */
 static inline float op_f32(float a, float b, int op) {
   switch (op) {
+    case OP_AVG: /* accumulates like sum; the caller divides at the end */
     case OP_SUM: return a + b;
     case OP_PROD: return a * b;
     case OP_MAX: return (a < b) ? b : a;
@@ -156,6 +162,7 @@ static inline float op_f32(float a, float b, int op) {
 }
 static inline int32_t op_i32(int32_t a, int32_t b, int op) {
   switch (op) {
+    case OP_AVG:
     case OP_SUM: return (int32_t)((uint32_t)a + (uint32_t)b);
     case OP_PROD: return (int32_t)((uint32_t)a * (uint32_t)b);
     case OP_MAX: return (a < b) ? b : a;
@@ -180,18 +187,20 @@ static inline int32_t op_i32(int32_t a, int32_t b, int op) {
       for (int j = 1; j < k; j++) {                                            \
         T x = ((const T *)in[(first + j) % k])[i];                             \
         switch (op) {                                                          \
+          case OP_AVG:                                                         \
           case OP_SUM: acc = (T)(W)((W)acc + (W)x); break;                     \
           case OP_PROD: acc = (T)(W)((W)acc * (W)x); break;                    \
           case OP_MAX: acc = (acc < x) ? x : acc; break;                       \
           default: acc = (x < acc) ? x : acc; break;                           \
         }                                                                      \
       }                                                                        \
-      o[i] = acc;                                                              \
+      o[i] = (op == OP_AVG) ? (T)(acc / (T)k) : acc;                           \
     }                                                                          \
   } while (0)
 
 static inline double op_f64(double a, double b, int op) {
   switch (op) {
+    case OP_AVG:
     case OP_SUM: return a + b;
     case OP_PROD: return a * b;
     case OP_MAX: return (a < b) ? b : a;
@@ -201,7 +210,7 @@ static inline double op_f64(double a, double b, int op) {
 
 static int check_args(int dtype, int op) {
   if (oracle_dtype_size(dtype) == 0) return RC_INVALID; /* utils.h:690-694 */
-  if (op < OP_SUM || op > OP_MIN) return RC_INVALID;    /* bootstrap.cc:872-874 */
+  if (op < OP_SUM || op > OP_AVG) return RC_INVALID;    /* bootstrap.cc:872-874 rejects prod and avg; both are this path's own */
   return RC_OK;
 }
 
@@ -227,7 +236,7 @@ int oracle_reduce_copy(void *out, const void *const *in, int k, size_t count,
       float acc = ((const float *)in[first])[i];
       for (int j = 1; j < k; j++)
         acc = op_f32(acc, ((const float *)in[(first + j) % k])[i], op);
-      o[i] = acc;
+      o[i] = (op == OP_AVG) ? acc / (float)k : acc;
     }
   } else if (dtype == DT_INT32) {
     int32_t *o = (int32_t *)out;
@@ -236,7 +245,7 @@ int oracle_reduce_copy(void *out, const void *const *in, int k, size_t count,
       int32_t acc = ((const int32_t *)in[first])[i];
       for (int j = 1; j < k; j++)
         acc = op_i32(acc, ((const int32_t *)in[(first + j) % k])[i], op);
-      o[i] = acc;
+      o[i] = (op == OP_AVG) ? acc / k : acc;
     }
   } else if (dtype == DT_INT8) {
     ORACLE_INT_LOOP(int8_t, uint8_t);
@@ -255,7 +264,7 @@ int oracle_reduce_copy(void *out, const void *const *in, int k, size_t count,
       double acc = ((const double *)in[first])[i];
       for (int j = 1; j < k; j++)
         acc = op_f64(acc, ((const double *)in[(first + j) % k])[i], op);
-      o[i] = acc;
+      o[i] = (op == OP_AVG) ? acc / (double)k : acc;
     }
   } else {
     uint16_t *o = (uint16_t *)out;
@@ -264,12 +273,13 @@ int oracle_reduce_copy(void *out, const void *const *in, int k, size_t count,
     for (long long i = 0; i < n; i++) {
       uint16_t hb = ((const uint16_t *)in[first])[i];
       float acc = bf ? oracle_bf16_to_f32(hb) : oracle_f16_to_f32(hb);
-      if (op == OP_SUM || op == OP_PROD) {
+      if (op == OP_SUM || op == OP_PROD || op == OP_AVG) {
         for (int j = 1; j < k; j++) {
           uint16_t xb = ((const uint16_t *)in[(first + j) % k])[i];
           float x = bf ? oracle_bf16_to_f32(xb) : oracle_f16_to_f32(xb);
           acc = op_f32(acc, x, op);
         }
+        if (op == OP_AVG) acc = acc / (float)k;
         o[i] = bf ? oracle_f32_to_bf16(acc) : oracle_f32_to_f16(acc);
       } else {
         for (int j = 1; j < k; j++) {
@@ -311,6 +321,7 @@ int oracle_host_ring_passes(void *acc, const void *const *in, int k,
                             size_t count, int dtype, int op) {
   int rc = check_args(dtype, op);
   if (rc) return rc;
+  if (op == OP_AVG) return RC_INVALID; /* a mean is not a chain of two-input means */
   if (k < 1) return RC_INVALID;
   size_t bytes = count * oracle_dtype_size(dtype);
   if (k == 1) {
@@ -475,6 +486,7 @@ int oracle_ring_allreduce(void *const *recv, const void *const *send,
                           int nranks, size_t count, int dtype, int op) {
   int rc = check_args(dtype, op);
   if (rc) return rc;
+  if (op == OP_AVG) return RC_INVALID; /* a mean is not a chain of two-input means */
   size_t ts = oracle_dtype_size(dtype);
   if (nranks < 1) return RC_INVALID;
   if (nranks == 1) {
@@ -570,6 +582,7 @@ int oracle_tree_reduce(void *recv_root, const void *const *send, int nranks, int
                        int op) {
   int rc = check_args(dtype, op);
   if (rc) return rc;
+  if (op == OP_AVG) return RC_INVALID; /* a mean is not a chain of two-input means */
   if (nranks < 1 || root < 0 || root >= nranks) return RC_INVALID;
   if (nranks == 1) {
     if (count && recv_root != send[0]) memmove(recv_root, send[0], count * oracle_dtype_size(dtype));

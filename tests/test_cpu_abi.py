@@ -190,8 +190,8 @@ def test_argument_screening_needs_no_gpu():
     p = 0x1000
     rc = lambda **kw: K.reduce_copy(kw.get("out", p), kw.get("ins", [p, p]), kw.get("n", 4), kw.get("dtype", N.DT_FP32),
                                     kw.get("op", N.OP_SUM), kw.get("first", 0))
-    assert rc(op=N.OP_AVG) == N.NOT_SUPPORTED
-    assert rc(dtype=N.DT_FP64, op=N.OP_AVG) == N.NOT_SUPPORTED
+    assert rc(op=N.OP_AVG, out=None) == N.INVALID_ARGUMENT           # every FlagCX type and op is carried; what is left
+    assert rc(dtype=N.DT_FP64, op=5) == N.INVALID_ARGUMENT             # to reject lies outside the enums
     assert rc(dtype=N.DT_INT64, out=p + 4) == N.INVALID_ARGUMENT      # 8-byte elements need 8-byte alignment
     assert rc(dtype=10) == N.INVALID_ARGUMENT and rc(dtype=-1) == N.INVALID_ARGUMENT
     assert rc(op=5) == N.INVALID_ARGUMENT
@@ -211,7 +211,7 @@ def test_argument_screening_needs_no_gpu():
     assert N.lib.fxSimCommInitAll(None, 2) == N.INVALID_ARGUMENT
     comms = (C.c_void_p * 2)()
     assert N.lib.fxSimCommInitAll(comms, 0) == N.INVALID_ARGUMENT
-    assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP64, N.OP_AVG, None, None) == N.NOT_SUPPORTED
+    assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP64, 5, None, None) == N.INVALID_ARGUMENT
     assert N.lib.flagcxAllReduce(p, p, 4, N.DT_FP32, N.OP_SUM, None, None) == N.INVALID_ARGUMENT
 
 
@@ -273,7 +273,7 @@ int main(void) {
   fx_trigger_get(&t, NULL, NULL, NULL, &c, NULL, &dt, &op, &st);
   if (c != 77 || dt != flagcxBfloat16 || op != flagcxMax || st != fxTriggerEnqueued) return 2;
   if (fx_dtype_size(flagcxFloat64) != 8 || fx_dtype_size(99) != 0) return 3;
-  if (fx_reduce_copy(NULL, NULL, 2, 4, flagcxFloat32, flagcxAvg, 0, NULL) != flagcxNotSupported) return 4;
+  if (fx_reduce_copy(NULL, NULL, 2, 4, flagcxFloat32, flagcxNumRedOps, 0, NULL) != flagcxInvalidArgument) return 4;
   if (strcmp(flagcxGetErrorString(flagcxInvalidArgument), "invalid argument")) return 5;
   if (flagcxGetVersion(&version) != flagcxSuccess || version != FX_SIM_VERSION) return 6;
   if (flagcxGetUniqueId(&a) != flagcxSuccess || flagcxGetUniqueId(&b) != flagcxSuccess) return 7;

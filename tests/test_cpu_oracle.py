@@ -222,7 +222,7 @@ def test_host_ring_passes_equal_kway_for_exact_types():
 
 def test_unsupported_arguments_are_rejected():
     a = np.zeros(4, np.float32)
-    for dtype, op in ((10, SUM), (-1, SUM), (F32, 4), (F32, -1)):   # outside the enum / avg: bootstrap.cc:872-874
+    for dtype, op in ((10, SUM), (-1, SUM), (F32, 5), (F32, -1)):   # outside the enums
         with pytest.raises(ValueError):
             O.reduce2(a, a, dtype, op)
 
@@ -288,6 +288,57 @@ def test_fp64_left_fold_matches_numpy():
     # order: a triple whose left fold differs from the right fold in double precision
     a, b, c = np.array([1e16]), np.array([1.0]), np.array([-1e16])
     assert O.reduce_copy([a, b, c], 8, SUM)[0] == 0.0 and O.reduce_copy([a, c, b], 8, SUM)[0] == 1.0
+
+
+# ---- avg: this path's own definition (parity unpinned by the reference) -----------------------
+def test_avg_is_the_sum_divided_once():
+    """Sum as defined above, then one division by k before the final rounding:
+    IEEE division for floating types, C division (toward zero) of the wrapped sum
+    for signed integers, unsigned division otherwise.  Checked against numpy and
+    Python integers; chains of two-input passes refuse it."""
+    AVG = 4
+    rng = np.random.default_rng(44)
+    for k in (1, 2, 3, 7, 8):
+        f = [rng.uniform(-1, 1, 5000).astype(np.float32) for _ in range(k)]
+        acc = f[0].copy()
+        for x in f[1:]:
+            acc = acc + x
+        assert np.array_equal(O.reduce_copy(f, F32, AVG), acc / np.float32(k))
+        d = [rng.uniform(-1, 1, 5000) for _ in range(k)]
+        acc = d[0].copy()
+        for x in d[1:]:
+            acc = acc + x
+        assert np.array_equal(O.reduce_copy(d, 8, AVG), acc / float(k))
+        # 16-bit: fp32 sum / k rounded once
+        h = [rng.normal(0, 1, 5000).astype(np.float16) for _ in range(k)]
+        acc = h[0].astype(np.float32)
+        for x in h[1:]:
+            acc = acc + x.astype(np.float32)
+        assert np.array_equal(O.reduce_copy([x.view(np.uint16) for x in h], F16, AVG),
+                              (acc / np.float32(k)).astype(np.float16).view(np.uint16))
+        b = [(rng.normal(0, 1, 5000).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16) for _ in range(k)]
+        acc = (b[0].astype(np.uint32) << 16).view(np.float32)
+        for x in b[1:]:
+            acc = acc + (x.astype(np.uint32) << 16).view(np.float32)
+        want = np.array([O.lib.oracle_f32_to_bf16(float(v)) for v in (acc / np.float32(k))], np.uint16)
+        assert np.array_equal(O.reduce_copy(b, BF16, AVG), want)
+        for dtype, t in ((0, np.int8), (1, np.uint8), (I32, np.int32), (3, np.uint32), (4, np.int64), (5, np.uint64)):
+            t = np.dtype(t)
+            lo, hi, bits = int(np.iinfo(t).min), int(np.iinfo(t).max), 8 * t.itemsize
+            ins = [rng.integers(lo, hi, 300, dtype=t, endpoint=True) for _ in range(k)]
+            want = []
+            for col in zip(*[a.tolist() for a in ins]):
+                tot = sum(col) % (1 << bits)
+                if lo < 0 and tot >= 1 << (bits - 1):
+                    tot -= 1 << bits
+                want.append(int(tot / k) if abs(tot) < 2**52 else (abs(tot) // k) * (1 if tot >= 0 else -1))
+            assert O.reduce_copy(ins, dtype, AVG).tolist() == want, (dtype, k)
+    with pytest.raises(ValueError):
+        O.host_ring_passes([np.zeros(4, np.float32)] * 3, F32, AVG)
+    with pytest.raises(ValueError):
+        O.ring_allreduce([np.zeros(4, np.float32)] * 3, F32, AVG)
+    with pytest.raises(ValueError):
+        O.tree_reduce([np.zeros(4, np.float32)] * 3, 0, F32, AVG)
 
 
 # ---- partition arithmetic ------------------------------------------------------------------

@@ -117,7 +117,11 @@ def test_reducing_collectives_closed_forms(dev, ccl, stream):
         wantb = O.reduce_copy(bf, N.DT_BF16, N.OP_SUM)
         for r in (0, 7):
             assert np.array_equal(dev.to_host(dr[r], 300001, np.uint16), wantb)
-        assert ccl.allReduce(ds[0], dr[0], count, N.DT_FP32, N.OP_AVG, comms[0], stream) == N.NOT_SUPPORTED
+        assert ccl.allReduce(ds[0], dr[0], count, N.DT_FP32, 5, comms[0], stream) == N.INVALID_ARGUMENT
+        for r in range(n):      # avg, the op the torch backend maps ReduceOp.AVG to (backend_flagcx.cpp:21-25)
+            assert ccl.allReduce(ds[r], dr[r], count, N.DT_FP32, N.OP_AVG, comms[r], stream) == OK
+        dev.stream_sync(stream)
+        assert np.array_equal(dev.to_host(dr[n - 1], count, np.float32), O.reduce_copy(sends, N.DT_FP32, N.OP_AVG))
     destroy(ccl, comms)
 
 

@@ -223,8 +223,8 @@ def test_custom_allreduce_hook(dev, stream):
         wins = [b.alloc(8 << 20) for _ in range(n)]
         N.check(g.register_windows(wins, 8 << 20))
         assert g.custom_all_reduce(ds, dr, count + 1, dtype, N.OP_SUM, stream) == N.NOT_SUPPORTED   # > window
-        assert g.custom_all_reduce(ds, dr, count, dtype, N.OP_AVG, stream) == N.NOT_SUPPORTED
-        for op in (N.OP_SUM, N.OP_MIN):
+        assert g.custom_all_reduce(ds, dr, count, dtype, 5, stream) == N.NOT_SUPPORTED               # the hook only declines
+        for op in (N.OP_SUM, N.OP_MIN, N.OP_AVG):
             N.check(g.custom_all_reduce(ds, dr, count, dtype, op, stream))
             dev.stream_sync(stream)
             want = O.reduce_copy(sends, dtype, op)

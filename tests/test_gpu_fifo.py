@@ -103,8 +103,8 @@ def test_triggers_through_the_ring(dev):
                 total += 1
             assert_parity(dev.to_host(dins[0], n, np.float32), O.reduce_copy(ins, N.DT_FP32, N.OP_SUM), N.DT_FP32,
                           N.OP_SUM, "chain")
-            # an op the path does not carry is completed (so the producer is not left waiting) and counted
-            ring.wait(ring.enqueue(dins[0], dins[1], dins[0], 16, N.DT_FP32, N.OP_AVG))
+            # an op outside the enum is completed (so the producer is not left waiting) and counted
+            ring.wait(ring.enqueue(dins[0], dins[1], dins[0], 16, N.DT_FP32, 7))
             total += 1
             w = ring.words()
             assert w[0] == 4 and w[2] == total                      # capacity, produced

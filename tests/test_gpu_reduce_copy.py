@@ -186,8 +186,7 @@ def test_error_paths(dev):
     try:
         ok = lambda dtype, op, k=2, first=0, out=p, ins=None, n=4: K.reduce_copy(out, ins or [p] * k, n, dtype, op, first)
         assert ok(N.DT_FP32, N.OP_SUM) == N.SUCCESS
-        assert ok(N.DT_FP32, N.OP_AVG) == N.NOT_SUPPORTED       # known to FlagCX, not on this path
-        assert ok(N.DT_INT8, N.OP_AVG) == N.NOT_SUPPORTED
+        assert ok(N.DT_FP32, N.OP_AVG) == N.SUCCESS             # every FlagCX type and op is carried
         assert ok(10, N.OP_SUM) == N.INVALID_ARGUMENT           # outside the enums
         assert ok(N.DT_FP32, 5) == N.INVALID_ARGUMENT
         assert ok(N.DT_FP32, N.OP_SUM, first=2) == N.INVALID_ARGUMENT

@@ -95,8 +95,8 @@ def test_triggers_ring_step_semantics(dev):
         assert_parity(dev.to_host(di[0], n, np.int32), O.reduce2(i[0], i[1], N.DT_INT32, N.OP_PROD), N.DT_INT32,
                       N.OP_PROD)
         assert_parity(dev.to_host(dh[0], n, np.uint16), O.reduce2(h[0], h[1], N.DT_FP16, N.OP_MAX), N.DT_FP16, N.OP_MAX)
-        bad = [K.make_trigger(df[0], df[1], df[0], 4, 32, N.DT_FP32, N.OP_AVG)]
-        assert K.reduce_triggers(bad) == N.NOT_SUPPORTED
+        bad = [K.make_trigger(df[0], df[1], df[0], 4, 32, N.DT_FP32, 7)]
+        assert K.reduce_triggers(bad) == N.INVALID_ARGUMENT
 
 
 def test_reduce2_all_types(dev):

@@ -30,8 +30,9 @@ def test_life_cycle_and_errors(dev, fx):
     comms = _group(fx, 3)
     assert [fx.flagcxCommUserRank(c) for c in comms] == [0, 1, 2] and fx.flagcxCommCount(comms[1]) == 3
     stream = fx.adaptor_stream_create()
-    with pytest.raises(RuntimeError, match="not supported"):
-        fx.flagcxAllReduce(1 << 12, 1 << 12, 4, DT.flagcxFloat, OP.flagcxAvg, comms[0], stream)
+    assert fx.flagcxGetErrorString(N.NOT_SUPPORTED) == "not supported"
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        fx.flagcxAllReduce(1 << 12, 1 << 12, 4, DT.flagcxFloat, OP.flagcxNumOps, comms[0], stream)
     with pytest.raises(RuntimeError, match="invalid argument"):
         fx.flagcxAllReduce(None, None, 4, DT.flagcxFloat, OP.flagcxSum, comms[0], stream)
     with pytest.raises(ValueError):

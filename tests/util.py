@@ -7,7 +7,7 @@ from flagcx_amd import kernels as K
 DTYPES = {"fp32": N.DT_FP32, "int32": N.DT_INT32, "bf16": N.DT_BF16, "fp16": N.DT_FP16,
           "uint32": N.DT_UINT32, "int8": N.DT_INT8, "uint8": N.DT_UINT8, "int64": N.DT_INT64, "uint64": N.DT_UINT64,
           "fp64": N.DT_FP64}
-OPS = {"sum": N.OP_SUM, "prod": N.OP_PROD, "max": N.OP_MAX, "min": N.OP_MIN}
+OPS = {"sum": N.OP_SUM, "prod": N.OP_PROD, "max": N.OP_MAX, "min": N.OP_MIN, "avg": N.OP_AVG}
 
 
 def seeded_inputs(dtype, k, n, seed, dist=None):
@@ -48,10 +48,10 @@ def ordered16(bits):
 
 
 def assert_parity(got, want, dtype, op, what=""):
-    """Bit-exact for fp32 / int32 / every max-min; for 16-bit sum and prod the
-    stated tolerance is 1 ulp of the output type, NaN matching NaN."""
+    """Bit-exact for fp32 / fp64 / integers / every max-min; for 16-bit sum, prod
+    and avg the stated tolerance is 1 ulp of the output type, NaN matching NaN."""
     assert got.shape == want.shape
-    if dtype in (N.DT_BF16, N.DT_FP16) and op in (N.OP_SUM, N.OP_PROD):
+    if dtype in (N.DT_BF16, N.DT_FP16) and op in (N.OP_SUM, N.OP_PROD, N.OP_AVG):
         gn, wn = is_nan16(got, dtype), is_nan16(want, dtype)
         assert np.array_equal(gn, wn), f"{what}: NaN positions differ"
         d = np.abs(ordered16(got)[~gn] - ordered16(want)[~wn])

@@ -20,7 +20,7 @@ from .adaptor import Device
 
 DT = {"fp32": N.DT_FP32, "fp16": N.DT_FP16, "bf16": N.DT_BF16, "int32": N.DT_INT32, "uint32": N.DT_UINT32,
       "int8": N.DT_INT8, "uint8": N.DT_UINT8, "int64": N.DT_INT64, "uint64": N.DT_UINT64, "fp64": N.DT_FP64}
-OP = {"sum": N.OP_SUM, "prod": N.OP_PROD, "max": N.OP_MAX, "min": N.OP_MIN}
+OP = {"sum": N.OP_SUM, "prod": N.OP_PROD, "max": N.OP_MAX, "min": N.OP_MIN, "avg": N.OP_AVG}
 
 
 def size(s):

@@ -177,6 +177,86 @@ flagcxResult_t forPieces(const Group *g, size_t ccnt, size_t coff, size_t nred, 
   return flagcxSuccess;
 }
 
+// ---- the host path's schedule (FX_ORDER_HOST) ----
+// Element range of chunk i: ceil(size / n) bytes rounded up to whole elements,
+// the last non-empty chunk short, later ones empty (bootstrap.cc:900-922).
+void hostChunk(size_t count, int n, int i, size_t *cnt, size_t *off) {
+  const size_t chunk = (count + (size_t)n - 1) / (size_t)n;  // same as the byte formula divided by the element size
+  if (chunk * (size_t)i >= count) {
+    *off = count;
+    *cnt = 0;
+  } else {
+    *off = chunk * (size_t)i;
+    *cnt = (chunk * (size_t)(i + 1) >= count) ? count - *off : chunk;
+  }
+}
+
+// Rank order in which a left-to-right fold reproduces the host ring's result for
+// chunk c.  The ring computes x_c (op) (x_{c-1} (op) (.. (x_{c+2} (op) x_{c+1}))),
+// local operand first (bootstrap.cc:805-871).  For sum / prod / avg the operands
+// of one step commute bit for bit, so the fold runs c+1, c+2, .., c.  For max /
+// min ((a < b) ? b : a keeps the LOCAL value on a tie) the fold keeps its
+// accumulator on a tie instead, so it runs c, c-1, .., c+1: either way the last
+// rank of the ring wins ties.
+void hostOrder(int c, int n, int op, std::vector<int> &order) {
+  order.resize(n);
+  const bool select = (op == flagcxMax || op == flagcxMin);
+  for (int j = 0; j < n; j++) order[j] = select ? mod(c - j, n) : mod(c + 1 + j, n);
+}
+
+// Host-order reduce of `nchunks` element ranges (chunk i = [off[i], off[i]+cnt[i]) of
+// every send buffer, folded in hostOrder(chunkId[i])) into outs[i][0..nout-1].
+struct HostPiece {
+  int chunk;
+  size_t off, cnt;
+  std::vector<void *> outs;
+};
+
+flagcxResult_t reduceHostPieces(const Ctx &c, const std::vector<HostPiece> &pieces) {
+  std::vector<int> order;
+  std::vector<fxBcastDesc> bcast;
+  std::vector<fxSliceDesc> plain;
+  int nout = 0;
+  for (const HostPiece &p : pieces) {
+    if (p.cnt == 0) continue;
+    hostOrder(p.chunk, c.n, c.g->op, order);
+    nout = (int)p.outs.size();
+    if (c.n <= FX_MAX_SLICE_INPUTS && nout <= FX_MAX_SLICE_INPUTS) {
+      if (nout == 1) {
+        fxSliceDesc d;
+        memset(&d, 0, sizeof(d));
+        for (int j = 0; j < c.n; j++) d.in[j] = cadd(c.send(order[j]), p.off * c.ts);
+        d.out = p.outs[0];
+        d.count = p.cnt;
+        plain.push_back(d);
+      } else {
+        fxBcastDesc d;
+        memset(&d, 0, sizeof(d));
+        for (int j = 0; j < c.n; j++) d.in[j] = cadd(c.send(order[j]), p.off * c.ts);
+        for (int o = 0; o < nout; o++) d.out[o] = p.outs[o];
+        d.count = p.cnt;
+        bcast.push_back(d);
+      }
+      continue;
+    }
+    // more than eight ranks: one runtime-k launch per piece, then copies
+    std::vector<const void *> in(c.n);
+    for (int j = 0; j < c.n; j++) in[j] = cadd(c.send(order[j]), p.off * c.ts);
+    flagcxResult_t rc = R(fx_reduce_copy(p.outs[0], in.data(), c.n, p.cnt, c.g->dtype, c.g->op, 0, c.s));
+    if (rc != flagcxSuccess) return rc;
+    std::vector<fxSliceDesc> copies;
+    for (int o = 1; o < nout; o++) copies.push_back(copyDesc(p.outs[0], p.outs[o], p.cnt * c.ts));
+    rc = R(fx_copy_slices(copies.data(), copies.size(), c.s));
+    if (rc != flagcxSuccess) return rc;
+  }
+  if (!plain.empty()) {
+    flagcxResult_t rc = R(fx_reduce_slices(plain.data(), plain.size(), c.n, c.g->dtype, c.g->op, c.s));
+    if (rc != flagcxSuccess) return rc;
+  }
+  if (!bcast.empty()) return R(fx_reduce_bcast_slices(bcast.data(), bcast.size(), c.n, nout, c.g->dtype, c.g->op, c.s));
+  return flagcxSuccess;
+}
+
 flagcxResult_t runAllReduce(const Ctx &c) {
   Group *g = c.g;
   const int n = c.n;
@@ -187,6 +267,15 @@ flagcxResult_t runAllReduce(const Ctx &c) {
       return R(fx_copy_slices(&d, 1, c.s));
     }
     return flagcxSuccess;
+  }
+  if (g->order == FX_ORDER_HOST) {  // the host path's chunks and fold order; every rank receives every chunk
+    std::vector<HostPiece> pieces(n);
+    for (int ch = 0; ch < n; ch++) {
+      pieces[ch].chunk = ch;
+      hostChunk(count, n, ch, &pieces[ch].cnt, &pieces[ch].off);
+      for (int r = 0; r < n; r++) pieces[ch].outs.push_back(madd(c.recv(r), pieces[ch].off * ts));
+    }
+    return reduceHostPieces(c, pieces);
   }
   const size_t nred = fx_nredslices(count, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
   std::vector<fxSliceDesc> descs;
@@ -297,6 +386,15 @@ flagcxResult_t runReduce(const Ctx &c) {
   const int n = c.n, root = g->root;
   const size_t count = g->count, ts = c.ts;
   if (count == 0) return flagcxSuccess;
+  if (g->order == FX_ORDER_HOST && n > 1) {  // the host path reduce-scatters, then gathers the chunks on the root
+    std::vector<HostPiece> pieces(n);
+    for (int ch = 0; ch < n; ch++) {
+      pieces[ch].chunk = ch;
+      hostChunk(count, n, ch, &pieces[ch].cnt, &pieces[ch].off);
+      pieces[ch].outs.push_back(madd(c.recv(root), pieces[ch].off * ts));
+    }
+    return reduceHostPieces(c, pieces);
+  }
   if (g->order != FX_ORDER_TREE || n == 1 || g->op == flagcxAvg) {
     std::vector<const void *> in(n);
     for (int j = 0; j < n; j++) in[j] = c.send(j);
@@ -341,6 +439,16 @@ flagcxResult_t runReduceScatter(const Ctx &c) {
       return R(fx_copy_slices(&d, 1, c.s));
     }
     return flagcxSuccess;
+  }
+  if (g->order == FX_ORDER_HOST) {  // chunk r = [r * recvcount, (r+1) * recvcount) ends on rank r
+    std::vector<HostPiece> pieces(n);
+    for (int r = 0; r < n; r++) {
+      pieces[r].chunk = r;
+      pieces[r].off = (size_t)r * rcount;
+      pieces[r].cnt = rcount;
+      pieces[r].outs.push_back(c.recv(r));
+    }
+    return reduceHostPieces(c, pieces);
   }
   const size_t nred = fx_nredslices(rcount, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
   std::vector<fxSliceDesc> descs;
@@ -981,7 +1089,7 @@ flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
       g->algo = value;
       break;
     case FX_SIM_ORDER:
-      if (value != FX_ORDER_RANK && value != FX_ORDER_RING && value != FX_ORDER_TREE) return flagcxInvalidArgument;
+      if (value < FX_ORDER_RANK || value > FX_ORDER_HOST) return flagcxInvalidArgument;
       g->order = value;
       break;
     case FX_SIM_NSLICES:

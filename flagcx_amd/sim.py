@@ -8,7 +8,7 @@ lib = N.lib
 
 ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE, SYNC = 0, 1, 2, 3, 4, 5
 ALGO_DIRECT, ALGO_RING = 0, 1
-ORDER_RANK, ORDER_RING, ORDER_TREE = 0, 1, 2
+ORDER_RANK, ORDER_RING, ORDER_TREE, ORDER_HOST = 0, 1, 2, 3
 SYNC_GROUP, SYNC_RENDEZVOUS = 0, 1
 
 

@@ -97,9 +97,17 @@ enum {
 enum {
   FX_ORDER_RANK = 0, /* rank 0,1,..,n-1: the custom allreduce's peer loop    */
   FX_ORDER_RING = 1, /* the rotated order a ring yields for each chunk       */
-  FX_ORDER_TREE = 2  /* flagcxReduce only: the binomial tree of
+  FX_ORDER_TREE = 2, /* flagcxReduce only: the binomial tree of
                         initUniRunnerStateTreeRed (uni_runner_impl.cc:1266-1557),
                         ceil(log2 n) rounds of two-input reduces               */
+  FX_ORDER_HOST = 3  /* what the reference's host path computes
+                        (FLAGCX_USE_HOST_COMM=1, flagcx/service/bootstrap.cc:787-942,
+                        1039-1066): chunks of ceil(size/n) bytes rounded up to an
+                        element, chunk c folded along the ring c+1, c+2, .., c
+                        as local (op) received.  AllReduce, Reduce and
+                        ReduceScatter; bit-identical to that path for every type
+                        it carries, +-0 ties of max / min included (a NaN operand
+                        of max / min is the one case not reproduced)           */
 };
 flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value);
 

@@ -35,6 +35,10 @@
  *       forms of the reference's divisible cases.
  *   oracle_tree_reduce ........................ hand-derived associations for
  *       n = 3, 5, 6, 8 on non-associative values + the reference's closed forms.
+ *   oracle_bootstrap_* (the host ring) ........ chunk table against the quoted
+ *       formula's literal cases; association and operand order derived by hand
+ *       from the reference loop for n = 3 and 4 on values where every other
+ *       association / tie rule gives a different answer; closed forms.
  *   oracle_pack / oracle_unpack ............... round-trip identity and the
  *       displacement arithmetic of service/bootstrap.cc:1253-1258.
  *   trigger encode/decode ..................... bit constants of
@@ -589,6 +593,111 @@ int oracle_tree_reduce(void *recv_root, const void *const *send, int nranks, int
     return RC_OK;
   }
   return tree_value(recv_root, send, nranks, root, 0, count, dtype, op);
+}
+
+/* ------------------------------------------------ host (bootstrap) ring */
+/*
+ * Chunking of the reference's host collectives (service/bootstrap.cc:900-922,
+ * 950-972): ChunkBytes = ceil(size / n) rounded up to a whole element; chunk i
+ * starts at min(i * ChunkBytes, size); the last non-empty chunk is short and
+ * the ones after it are empty.  Offsets and lengths in bytes.
+ */
+void oracle_bootstrap_chunks(size_t size, int nranks, size_t ts, size_t *offset,
+                             size_t *length) {
+  size_t chunk = (size + (size_t)nranks - 1) / (size_t)nranks;
+  chunk = (chunk + ts - 1) / ts * ts;
+  for (size_t i = 0; i < (size_t)nranks; i++) {
+    if (chunk * i >= size) {
+      offset[i] = size;
+      length[i] = 0;
+    } else {
+      offset[i] = chunk * i;
+      length[i] = (chunk * (i + 1) >= size) ? size - chunk * i : chunk;
+    }
+  }
+}
+
+/*
+ * bootstrapRingReduceScatter (service/bootstrap.cc:787-897), every rank played
+ * hop by hop.  Iteration i: rank r forwards chunk (r-i-1)%n -- its own data in
+ * iteration 0, what it reduced in the previous iteration afterwards -- and
+ * reduces the chunk (r-i-2)%n it receives as res = local (op) received
+ * (operand order of the sum/max/min calls at :853-871).  After n-1 iterations
+ * rank r holds chunk r; out[r] receives those length[r] bytes.
+ */
+int oracle_bootstrap_reduce_scatter(void *const *out, const void *const *send,
+                                    int nranks, const size_t *offset,
+                                    const size_t *length, int dtype, int op) {
+  int rc = check_args(dtype, op);
+  if (rc) return rc;
+  if (op == OP_AVG || nranks < 2) return RC_INVALID;
+  const size_t ts = oracle_dtype_size(dtype);
+  size_t sub = 0;
+  for (int i = 0; i < nranks; i++)
+    if (length[i] > sub) sub = length[i];
+  /* partial[r] = what rank r reduced last (data_for_recv); flight[r] = what it sends */
+  char **partial = (char **)calloc((size_t)nranks, sizeof(char *));
+  char **flight = (char **)calloc((size_t)nranks, sizeof(char *));
+  if (!partial || !flight) return RC_INVALID;
+  for (int r = 0; r < nranks; r++) {
+    partial[r] = (char *)calloc(sub ? sub : 1, 1);
+    flight[r] = (char *)calloc(sub ? sub : 1, 1);
+  }
+  for (int iter = 0; iter < nranks - 1 && !rc; iter++) {
+    for (int r = 0; r < nranks; r++) { /* everybody prepares what it sends */
+      int sc = (r + 2 * nranks - iter - 1) % nranks;
+      if (!length[sc]) continue;
+      if (iter == 0)
+        memcpy(flight[r], (const char *)send[r] + offset[sc], length[sc]);
+      else
+        memcpy(flight[r], partial[r], length[sc]);
+    }
+    for (int r = 0; r < nranks && !rc; r++) { /* receive from the previous rank and reduce */
+      int rcv = (r + 2 * nranks - iter - 2) % nranks;
+      if (!length[rcv]) continue;
+      int prev = (r + nranks - 1) % nranks;
+      memcpy(partial[r], flight[prev], length[rcv]);
+      rc = oracle_reduce2(partial[r], (const char *)send[r] + offset[rcv], partial[r], length[rcv] / ts, dtype, op);
+    }
+  }
+  for (int r = 0; r < nranks; r++) {
+    if (!rc && length[r]) memcpy(out[r], partial[r], length[r]);
+    free(partial[r]);
+    free(flight[r]);
+  }
+  free(partial);
+  free(flight);
+  return rc;
+}
+
+/*
+ * AllReduceBootstrap (service/bootstrap.cc:993-1011, 899-942): chunks as above,
+ * the ring reduce-scatter, then an all-gather that moves bytes only.  recv[r]
+ * may alias send[r].
+ */
+int oracle_bootstrap_allreduce(void *const *recv, const void *const *send,
+                               int nranks, size_t count, int dtype, int op) {
+  int rc = check_args(dtype, op);
+  if (rc) return rc;
+  const size_t ts = oracle_dtype_size(dtype), size = count * ts;
+  if (nranks < 1) return RC_INVALID;
+  if (nranks == 1) {
+    if (size && recv[0] != send[0]) memmove(recv[0], send[0], size);
+    return RC_OK;
+  }
+  size_t *offset = (size_t *)calloc(2 * (size_t)nranks, sizeof(size_t)), *length = offset + nranks;
+  char *full = (char *)malloc(size ? size : 1);
+  void **piece = (void **)calloc((size_t)nranks, sizeof(void *));
+  if (!offset || !full || !piece) return RC_INVALID;
+  oracle_bootstrap_chunks(size, nranks, ts, offset, length);
+  for (int r = 0; r < nranks; r++) piece[r] = full + offset[r];
+  rc = oracle_bootstrap_reduce_scatter(piece, send, nranks, offset, length, dtype, op);
+  for (int r = 0; r < nranks && !rc; r++)
+    if (size) memcpy(recv[r], full, size);
+  free(piece);
+  free(full);
+  free(offset);
+  return rc;
 }
 
 /* ------------------------------------------------------------- alltoallv */

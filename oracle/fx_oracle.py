@@ -66,6 +66,13 @@ lib.oracle_f16_to_f32.restype = C.c_float
 lib.oracle_f16_to_f32.argtypes = [C.c_uint16]
 lib.oracle_f32_to_f16.restype = C.c_uint16
 lib.oracle_f32_to_f16.argtypes = [C.c_float]
+lib.oracle_bootstrap_chunks.restype = None
+lib.oracle_bootstrap_chunks.argtypes = [_sz, _i, _sz, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+lib.oracle_bootstrap_reduce_scatter.restype = _i
+lib.oracle_bootstrap_reduce_scatter.argtypes = [C.POINTER(_vp), C.POINTER(_vp), _i, C.POINTER(C.c_size_t),
+                                                C.POINTER(C.c_size_t), _i, _i]
+lib.oracle_bootstrap_allreduce.restype = _i
+lib.oracle_bootstrap_allreduce.argtypes = [C.POINTER(_vp), C.POINTER(_vp), _i, _sz, _i, _i]
 lib.oracle_set_threads.argtypes = [_i]
 lib.oracle_dtype_size.restype = _sz
 lib.oracle_dtype_size.argtypes = [_i]
@@ -136,6 +143,22 @@ def ring_allreduce(sends, dtype, op):
     rc = lib.oracle_ring_allreduce(_ptrs(recvs), _ptrs(sends), len(sends), sends[0].size, dtype, op)
     if rc:
         raise ValueError(f"oracle_ring_allreduce rc={rc}")
+    return recvs
+
+
+def bootstrap_chunks(size, nranks, ts):
+    off = (C.c_size_t * nranks)()
+    ln = (C.c_size_t * nranks)()
+    lib.oracle_bootstrap_chunks(size, nranks, ts, off, ln)
+    return list(off), list(ln)
+
+
+def bootstrap_allreduce(sends, dtype, op):
+    """The reference's host ring all-reduce played hop by hop; returns every rank's result."""
+    recvs = [np.empty_like(s) for s in sends]
+    rc = lib.oracle_bootstrap_allreduce(_ptrs(recvs), _ptrs(sends), len(sends), sends[0].size, dtype, op)
+    if rc:
+        raise ValueError(f"oracle_bootstrap_allreduce rc={rc}")
     return recvs
 
 

@@ -290,6 +290,59 @@ def test_fp64_left_fold_matches_numpy():
     assert O.reduce_copy([a, b, c], 8, SUM)[0] == 0.0 and O.reduce_copy([a, c, b], 8, SUM)[0] == 1.0
 
 
+# ---- the host ring (service/bootstrap.cc:787-942) --------------------------------------------
+def test_bootstrap_chunk_table():
+    # literal evaluations of ceil(size / n) rounded up to the element size, offsets clamped to size
+    assert O.bootstrap_chunks(40, 3, 4) == ([0, 16, 32], [16, 16, 8])          # 10 floats over 3 ranks: 4, 4, 2
+    assert O.bootstrap_chunks(8, 4, 4) == ([0, 4, 8, 8], [4, 4, 0, 0])          # fewer elements than ranks
+    assert O.bootstrap_chunks(7, 3, 1) == ([0, 3, 6], [3, 3, 1])
+    assert O.bootstrap_chunks(0, 2, 4) == ([0, 0], [0, 0])
+    assert O.bootstrap_chunks(64, 8, 8) == ([8 * i for i in range(8)], [8] * 8)
+    for size_el, n, ts in itertools.product((1, 5, 17, 1000, 1001), (1, 2, 3, 8), (1, 2, 4, 8)):
+        off, ln = O.bootstrap_chunks(size_el * ts, n, ts)
+        assert sum(ln) == size_el * ts and all(x % ts == 0 for x in off + ln)
+        assert all(off[i] + ln[i] == off[i + 1] for i in range(n - 1) if ln[i + 1]) and off[0] == 0
+
+
+def test_bootstrap_ring_association_derived_by_hand():
+    """Reading the loop at bootstrap.cc:805-871: chunk c starts on rank c+1 and
+    every later rank computes local + received, so rank c ends with
+    x_c + (x_{c-1} + (.. (x_{c+2} + x_{c+1}))).  The values make every other
+    association (rank order, the uniRunner ring's rotation, pairwise) differ."""
+    f = np.float32
+    for n in (3, 4):
+        per = 50
+        count = per * n                                      # chunk c = elements [50 c, 50 c + 50)
+        rng = np.random.default_rng(n)
+        sends = [(rng.uniform(-1, 1, count) * 10.0 ** rng.integers(-3, 9, count)).astype(f) for _ in range(n)]
+        want = np.empty(count, f)
+        for c in range(n):
+            sl = slice(per * c, per * (c + 1))
+            acc = sends[(c + 1) % n][sl]
+            for j in range(2, n + 1):
+                acc = sends[(c + j) % n][sl] + acc           # local + received
+            want[sl] = acc
+        got = O.bootstrap_allreduce(sends, F32, SUM)
+        for r in range(n):
+            assert np.array_equal(got[r].view(np.uint32), want.view(np.uint32)), (n, r)
+        assert not np.array_equal(O.reduce_copy(sends, F32, SUM).view(np.uint32), want.view(np.uint32))
+        ring = O.ring_allreduce(sends, F32, SUM)[0]
+        assert not np.array_equal(ring.view(np.uint32), want.view(np.uint32))
+    # max / min return the LOCAL operand unless strictly beaten ((a < b) ? b : a, utils.h:707-725), so among
+    # zeros of either sign the last rank of the chain -- rank c for chunk c -- decides
+    n, count = 3, 6
+    pz, nz = f(0.0), f(-0.0)
+    sends = [np.array([pz, nz, nz, pz, nz, pz], f), np.array([nz, nz, pz, pz, pz, nz], f), np.array([nz, pz, pz, nz, nz, nz], f)]
+    for op in (MAX, MIN):
+        got = O.bootstrap_allreduce(sends, F32, op)[0]
+        want = np.concatenate([sends[c][2 * c:2 * c + 2] for c in range(n)])          # chunk c = elements 2c, 2c+1
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), op
+    # closed form of the reference's collective tests holds on this path too
+    i = np.arange(1001)
+    sends = [(r * 1000 + i % 10).astype(f) for r in range(8)]
+    assert np.array_equal(O.bootstrap_allreduce(sends, F32, SUM)[5], (28 * 1000 + 8 * (i % 10)).astype(f))
+
+
 # ---- avg: this path's own definition (parity unpinned by the reference) -----------------------
 def test_avg_is_the_sum_divided_once():
     """Sum as defined above, then one division by k before the final rounding:

@@ -408,3 +408,48 @@ def test_rendezvous_times_out_when_a_rank_never_arrives(dev, stream, monkeypatch
         g.configure(sync=S.SYNC_GROUP)
         N.check(g.all_reduce([p] * n, [p] * n, 0, N.DT_FP32, N.OP_SUM, stream))
         dev.stream_sync(stream)
+
+
+@pytest.mark.parametrize("dname", ["fp32", "fp64", "int32", "uint8"])
+@pytest.mark.parametrize("n,count", [(8, 100003), (3, 10), (4, 2), (5, 77777), (12, 40001)])
+def test_host_order_matches_the_reference_host_ring(dev, stream, dname, n, count):
+    """FX_ORDER_HOST: the chunks and the fold of the reference's host path
+    (bootstrap.cc:787-942), bit for bit, for all-reduce, reduce and
+    reduce-scatter, in place and out of place; +-0 ties of max / min included."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    npdt = N.NP_DTYPE[dtype]
+    sends = seeded_inputs(dtype, n, count, seed=n + count)
+    if dname in ("fp32", "fp64"):                     # widen the exponent range so that association shows
+        rng = np.random.default_rng(count)
+        sends = [(a * 10.0 ** rng.integers(-3, 9, count)).astype(npdt) for a in sends]
+        for r, a in enumerate(sends):                 # and plant zeros of both signs for the tie rule
+            a[:min(count, 8)] = [(0.0, -0.0)[(r + i) % 2] for i in range(min(count, 8))]
+    for op in (N.OP_SUM, N.OP_MAX, N.OP_MIN):
+        want = O.bootstrap_allreduce(sends, dtype, op)[0]
+        for inplace in (False, True):
+            got = _allreduce(dev, stream, sends, dtype, op, inplace=inplace, order=3)
+            for r in range(n):
+                assert_parity(got[r], want, dtype, op, f"host order allreduce n={n} rank {r} op={op}")
+        with DevBufs(dev) as b, S.SimGroup(n, order=3) as g:
+            ds = [b.put(a) for a in sends]
+            root = n - 1
+            dout = b.alloc(count * es)
+            N.check(g.reduce(ds, [dout if r == root else None for r in range(n)], count, dtype, op, root, stream))
+            dev.stream_sync(stream)
+            assert_parity(dev.to_host(dout, count, npdt), want, dtype, op, f"host order reduce n={n}")
+    # reduce-scatter: chunk r = elements [r * rc, (r + 1) * rc) ends on rank r, same chain
+    rc = max(count // n, 1)
+    part = [a[:n * rc] if a.size >= n * rc else np.resize(a, n * rc) for a in sends]
+    off = (C.c_size_t * n)(*[r * rc * es for r in range(n)])
+    ln = (C.c_size_t * n)(*[rc * es] * n)
+    outs = [np.empty(rc, npdt) for _ in range(n)]
+    vp = lambda arrs: (C.c_void_p * n)(*[a.ctypes.data for a in arrs])
+    assert O.lib.oracle_bootstrap_reduce_scatter(vp(outs), vp(part), n, off, ln, dtype, N.OP_SUM) == 0
+    with DevBufs(dev) as b, S.SimGroup(n, order=3) as g:
+        ds = [b.put(a) for a in part]
+        dr = [b.alloc(rc * es) for _ in range(n)]
+        N.check(g.reduce_scatter(ds, dr, rc, dtype, N.OP_SUM, stream))
+        dev.stream_sync(stream)
+        for r in range(n):
+            assert_parity(dev.to_host(dr[r], rc, npdt), outs[r], dtype, N.OP_SUM, f"host order reduce-scatter rank {r}")

@@ -139,12 +139,30 @@ def test_special_values_fp32(dev):
     for op in OPS.values():
         want = O.reduce_copy(ins, N.DT_FP32, op)
         got = run_reduce(dev, ins, N.DT_FP32, op)
-        if op in (N.OP_SUM, N.OP_PROD):  # NaN payloads of arithmetic are not part of the contract
+        if op in (N.OP_SUM, N.OP_PROD, N.OP_AVG):  # NaN payloads of arithmetic are not part of the contract
             gn, wn = np.isnan(got), np.isnan(want)
             assert np.array_equal(gn, wn)
             assert np.array_equal(got[~gn].view(np.uint32), want[~wn].view(np.uint32))
         else:
             assert_parity(got, want, N.DT_FP32, op, f"special fp32 op={op}")
+
+
+def test_special_values_fp64(dev):
+    v = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 5e-324, -5e-324, 2.2250738585072014e-308,
+                  1.7976931348623157e308, -1.7976931348623157e308, 1e16, 1.0, -1e16, 9007199254740992.0, 0.5, 1.5,
+                  2.5, 1e-310], np.float64)
+    grid = np.array(list(itertools.product(v, v, v)), np.float64)
+    ins = [np.ascontiguousarray(grid[:, j]) for j in range(3)]
+    for op in OPS.values():
+        with np.errstate(all="ignore"):
+            want = O.reduce_copy(ins, N.DT_FP64, op)
+        got = run_reduce(dev, ins, N.DT_FP64, op)
+        if op in (N.OP_SUM, N.OP_PROD, N.OP_AVG):
+            gn, wn = np.isnan(got), np.isnan(want)
+            assert np.array_equal(gn, wn)
+            assert np.array_equal(got[~gn].view(np.uint64), want[~wn].view(np.uint64)), op
+        else:
+            assert_parity(got, want, N.DT_FP64, op, f"special fp64 op={op}")
 
 
 @pytest.mark.parametrize("dname", ["bf16", "fp16"])

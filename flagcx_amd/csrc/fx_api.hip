@@ -80,7 +80,7 @@ std::vector<fxSliceDesc> mergeAdjacent(const fxSliceDesc *slices, size_t n, int 
   return out;
 }
 
-// Launch n slices through kernel-argument tables of up to kInlineSlices each.
+// Launch n slices through kernel-argument tables (as many launches as the tables need).
 flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slicesIn, size_t nIn, int k, hipStream_t s) {
   for (size_t i = 0; i < nIn; i++)   // validate before merging so a bad slice is still reported
     if (slicesIn[i].count) {
@@ -88,37 +88,22 @@ flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slices
       for (int p = 0; p < k; p++)
         if (!slicesIn[i].in[p]) return flagcxInvalidArgument;
     }
-  const std::vector<fxSliceDesc> merged = mergeAdjacent(slicesIn, nIn, k, (size_t)ks->elemSize);
-  const fxSliceDesc *slices = merged.data();
-  const size_t n = merged.size();
+  std::vector<fxSliceDesc> merged = mergeAdjacent(slicesIn, nIn, k, (size_t)ks->elemSize);
   const int U = unrollFor(k);
-  InlineSliceTable t;
-  t.n = 0;
-  t.tileStart[0] = 0;
-  for (size_t i = 0; i <= n; i++) {
-    uint64_t tiles = 0;
-    if (i < n) {
-      flagcxResult_t rc = sliceTiles(slices[i], k, ks->elemSize, U, &tiles);
-      if (rc != flagcxSuccess) return rc;
-      if (tiles == 0) continue;
-      if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
-    }
-    const bool flush = (i == n) || t.n == (uint32_t)kInlineSlices ||
-                       (uint64_t)t.tileStart[t.n] + tiles > 0x7ffffff0ull;
-    if (flush && t.n > 0) {
-      flagcxResult_t rc = ks->slicesInline[k](t, s);
-      if (rc != flagcxSuccess) return rc;
-      t.n = 0;
-    }
-    if (i == n) break;
-    SliceDescDev &d = t.d[t.n];
-    for (int p = 0; p < kMaxFixedK; p++) d.in[p] = (p < k) ? slices[i].in[p] : nullptr;
-    d.out = slices[i].out;
-    d.count = slices[i].count;
-    t.tileStart[t.n + 1] = t.tileStart[t.n] + (uint32_t)tiles;
-    t.n++;
+  std::vector<uint32_t> tiles;
+  tiles.reserve(merged.size());
+  size_t kept = 0;
+  for (size_t i = 0; i < merged.size(); i++) {
+    uint64_t t = 0;
+    flagcxResult_t rc = sliceTiles(merged[i], k, ks->elemSize, U, &t);
+    if (rc != flagcxSuccess) return rc;
+    if (t == 0) continue;
+    if (t > 0x7ffffff0ull) return flagcxInvalidArgument;
+    merged[kept++] = merged[i];
+    tiles.push_back((uint32_t)t);
   }
-  return flagcxSuccess;
+  if (kept == 0) return flagcxSuccess;
+  return ks->slicesInline[k](merged.data(), tiles.data(), kept, s);
 }
 
 // Largest power-of-two granularity (4, 2 or 1 bytes) shared by all copy slices.

@@ -2,6 +2,7 @@
 // translation unit per element type instantiates a KernelSet per reduction
 // op; the C-ABI layer picks the entry for (dtype, op, k) at run time.
 #pragma once
+#include "flagcx_amd/fx_kernels.h"
 #include "fx_reduce_body.hpp"
 
 namespace fx {
@@ -16,7 +17,9 @@ constexpr uint64_t kBigLaunchTiles = 1024;  // use bigUnrollFor only above this 
 struct KernelSet {
   // index = compile-time input count, 0 = runtime-k kernel
   flagcxResult_t (*direct[kMaxFixedK + 1])(void *out, const void *const *in, int k, uint64_t count, hipStream_t s);
-  flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const InlineSliceTable &t, hipStream_t s);
+  // n slices with their tile counts (all non-zero), as many launches as their kernel-argument tables need
+  flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const fxSliceDesc *slices, const uint32_t *tiles, size_t n,
+                                                 hipStream_t s);
   flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
                                                 uint32_t grid, hipStream_t s);
   flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const InlineBcastTable &t, hipStream_t s);
@@ -54,12 +57,27 @@ flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t co
 }
 
 template <class R, int K>
-flagcxResult_t launchSlicesInline(const InlineSliceTable &t, hipStream_t s) {
+flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, const uint32_t *tiles, size_t n, hipStream_t s) {
   constexpr int U = unrollFor(K);
-  uint32_t grid = t.tileStart[t.n];
-  if (grid == 0) return flagcxSuccess;
-  hipLaunchKernelGGL((reduceSlicesInline<R, K, U>), dim3(grid), dim3(kBlock), 0, s, t);
-  FX_HIP(hipGetLastError());
+  InlineSliceTable<K> t;
+  t.n = 0;
+  t.tileStart[0] = 0;
+  for (size_t i = 0; i <= n; i++) {
+    const bool full = t.n == (uint32_t)InlineSliceTable<K>::kSlots ||
+                      (i < n && (uint64_t)t.tileStart[t.n] + tiles[i] > 0x7ffffff0ull);
+    if ((i == n || full) && t.n > 0) {
+      hipLaunchKernelGGL((reduceSlicesInline<R, K, U>), dim3(t.tileStart[t.n]), dim3(kBlock), 0, s, t);
+      FX_HIP(hipGetLastError());
+      t.n = 0;
+    }
+    if (i == n) break;
+    SliceDescK<K> &d = t.d[t.n];
+    for (int p = 0; p < K; p++) d.in[p] = slices[i].in[p];
+    d.out = slices[i].out;
+    d.count = slices[i].count;
+    t.tileStart[t.n + 1] = t.tileStart[t.n] + tiles[i];
+    t.n++;
+  }
   return flagcxSuccess;
 }
 

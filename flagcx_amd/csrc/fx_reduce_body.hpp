@@ -712,11 +712,27 @@ struct SliceDescDev {
   uint64_t count;
 };
 
-constexpr int kInlineSlices = 32;  // slices carried in the kernel argument block
+// Slices carried in the kernel argument block itself (no device table to fill
+// first).  The block is kept under 4 KiB, so a table for K inputs holds as many
+// descriptors of K+2 words as fit: 142 for copies (K = 1), 110 for two-input
+// reduces, 47 for K = 8.
+template <int K>
+struct SliceDescK {
+  const void *in[K];
+  void *out;
+  uint64_t count;
+};
 
+template <int K>
+constexpr int inlineSlicesFor() {
+  return (4000 - 8) / (int)(sizeof(SliceDescK<K>) + sizeof(uint32_t));
+}
+
+template <int K>
 struct InlineSliceTable {
-  SliceDescDev d[kInlineSlices];
-  uint32_t tileStart[kInlineSlices + 1];
+  static constexpr int kSlots = inlineSlicesFor<K>();
+  SliceDescK<K> d[kSlots];
+  uint32_t tileStart[kSlots + 1];
   uint32_t n;
 };
 
@@ -729,8 +745,8 @@ __device__ __forceinline__ uint32_t findSlice(const uint32_t *tileStart, uint32_
   return lo;
 }
 
-template <class R, int K, int U>
-__device__ __forceinline__ void reduceSlicesBody(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n) {
+template <class R, int K, int U, class D>
+__device__ __forceinline__ void reduceSlicesBody(const D *d, const uint32_t *tileStart, uint32_t n) {
   const uint32_t b = blockIdx.x;
   const uint32_t i = findSlice(tileStart, n, b);
   Seg<K> sg;
@@ -739,7 +755,7 @@ __device__ __forceinline__ void reduceSlicesBody(const SliceDescDev *d, const ui
 }
 
 template <class R, int K, int U>
-__global__ void __launch_bounds__(kBlock) reduceSlicesInline(InlineSliceTable t) {
+__global__ void __launch_bounds__(kBlock) reduceSlicesInline(InlineSliceTable<K> t) {
   reduceSlicesBody<R, K, U>(t.d, t.tileStart, t.n);
 }
 

@@ -232,3 +232,34 @@ def test_reduce_to_several_outputs_at_once(dev, dname):
         dev.sync()
         for d in dd:
             assert np.array_equal(dev.to_host(d, src.size, np.uint8), src)
+
+
+def test_more_slices_than_one_kernel_argument_table_holds(dev):
+    """500 disjoint, non-adjacent copies (the table for copies holds 142) and 300
+    two-input reduces (110 per table) in one call each: several launches, every
+    slice executed exactly once, gaps untouched."""
+    rng = np.random.default_rng(9)
+    nsl, seg, gap = 500, 777, 13
+    src = rng.integers(0, 256, nsl * (seg + gap), dtype=np.uint8)
+    with DevBufs(dev) as b:
+        dsrc, ddst = b.put(src), b.alloc(src.size)
+        dev.memset(ddst, 0xEE, src.size)
+        N.check(K.copy_slices([(dsrc + i * (seg + gap), ddst + i * (seg + gap), seg) for i in range(nsl)]))
+        dev.sync()
+        got = dev.to_host(ddst, src.size, np.uint8).reshape(nsl, seg + gap)
+    want = src.reshape(nsl, seg + gap).copy()
+    want[:, seg:] = 0xEE
+    assert np.array_equal(got, want)
+    nsl, seg, gap = 300, 1001, 3
+    a, c = seeded_inputs(N.DT_FP32, 2, nsl * (seg + gap), seed=17)
+    full = O.reduce2(a, c, N.DT_FP32, N.OP_SUM)
+    with DevBufs(dev) as b:
+        da, dc, do = b.put(a), b.put(c), b.alloc(a.nbytes)
+        dev.memset(do, 0, a.nbytes)
+        descs = [([da + 4 * i * (seg + gap), dc + 4 * i * (seg + gap)], do + 4 * i * (seg + gap), seg) for i in range(nsl)]
+        N.check(K.reduce_slices(descs, 2, N.DT_FP32, N.OP_SUM))
+        dev.sync()
+        got = dev.to_host(do, a.size, np.float32).reshape(nsl, seg + gap)
+    want = full.reshape(nsl, seg + gap).copy()
+    want[:, seg:] = 0
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

@@ -266,9 +266,11 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
     if (threadIdx.x == 0) {
       const uint32_t slot = (uint32_t)(seq % cap);
       // Release: with the barrier above, this workgroup's stores are out before
-      // it reports in.  Acquire: the last one in has everybody's stores behind it.
-      const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      // it reports in.  Only the last one in pays for the acquire that puts
+      // everybody's stores behind it (an L2 invalidate per workgroup otherwise).
+      const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
       if (prev == share.takers - 1) {  // last one out completes the trigger
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         __hip_atomic_store(&m->done[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (!ok) __hip_atomic_fetch_add(&m->badTriggers, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __threadfence_system();

@@ -613,36 +613,58 @@ __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, ui
   }
 }
 
-// Tile `tile` of the segment: striped zone first, then head, then tail.
-template <class R, int K, int U, class SG>
-__device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uint32_t tile) {
-  constexpr uint64_t V = (uint64_t)U * kBlock;
+// Which vectors lane `tid` of the workgroup that owns tile `tile` handles:
+// j, j + stride, .., U of them.  `fast` (the same for the whole workgroup) says
+// that all U * kBlock vectors of the tile are whole, inside the segment and
+// loadable with aligned vector loads; otherwise every vector below `limit` goes
+// through the checked path.  Shared by the kernels and by the host-side check of
+// this index arithmetic.
+struct TileLane {
+  uint64_t j, stride, limit;
+  bool fast;
+};
+
+__host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile, uint32_t tid, int U, bool coAligned) {
+  const uint64_t V = (uint64_t)U * kBlock;
+  TileLane tl;
   if (tile < tp.zoneTiles) {
     // tile i of region r owns vectors zs + r*RV + row*kRowVecs + i*kPieceVecs + [0, kPieceVecs)
     // for row = 0 .. V/kPieceVecs-1; lane (u, tid) takes row u*(kBlock/kPieceVecs) + tid/kPieceVecs.
     const uint32_t r = tile / kStripeTiles, i = tile % kStripeTiles;
-    const uint64_t j = tp.zs + (uint64_t)r * (V * kStripeTiles) + (uint64_t)(threadIdx.x / kPieceVecs) * kRowVecs +
-                       i * kPieceVecs + (threadIdx.x % kPieceVecs);
-    reduceVectorsFast<R, K, U>(sg, j * 16, (uint64_t)(kBlock / kPieceVecs) * kRowVecs * 16);
-    return;
+    tl.j = tp.zs + (uint64_t)r * (V * kStripeTiles) + (uint64_t)(tid / kPieceVecs) * kRowVecs + i * kPieceVecs +
+           (tid % kPieceVecs);
+    tl.stride = (uint64_t)(kBlock / kPieceVecs) * kRowVecs;
+    tl.limit = tp.ze;
+    tl.fast = true;
+    return tl;
   }
-  uint32_t t = tile - tp.zoneTiles;
-  uint64_t j0, limit;
+  const uint32_t t = tile - tp.zoneTiles;
+  uint64_t j0;
   if (t < tp.headTiles) {
     j0 = (uint64_t)t * V;
-    limit = (tp.ze > tp.zs) ? tp.zs : tp.nv;   // the head stops where the zone begins
+    tl.limit = (tp.ze > tp.zs) ? tp.zs : tp.nv;   // the head stops where the zone begins
   } else {
     j0 = tp.ze + (uint64_t)(t - tp.headTiles) * V;
-    limit = tp.nv;
+    tl.limit = tp.nv;
   }
-  const uint64_t fastEnd = (limit < tp.endFull) ? limit : tp.endFull;
-  if (sg.coAligned && j0 >= tp.firstFull && j0 + V <= fastEnd) {
-    reduceVectorsFast<R, K, U>(sg, (j0 + threadIdx.x) * 16, (uint64_t)kBlock * 16);
+  const uint64_t fastEnd = (tl.limit < tp.endFull) ? tl.limit : tp.endFull;
+  tl.j = j0 + tid;
+  tl.stride = kBlock;
+  tl.fast = coAligned && j0 >= tp.firstFull && j0 + V <= fastEnd;
+  return tl;
+}
+
+// Tile `tile` of the segment: striped zone first, then head, then tail.
+template <class R, int K, int U, class SG>
+__device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uint32_t tile) {
+  const TileLane tl = laneOfTile(tp, tile, threadIdx.x, U, sg.coAligned);
+  if (tl.fast) {
+    reduceVectorsFast<R, K, U>(sg, tl.j * 16, tl.stride * 16);
   } else {
 #pragma unroll 1
     for (int u = 0; u < U; u++) {
-      const uint64_t j = j0 + (uint64_t)u * kBlock + threadIdx.x;
-      if (j < limit) reduceVectorChecked<R, K>(sg, j);
+      const uint64_t j = tl.j + (uint64_t)u * tl.stride;
+      if (j < tl.limit) reduceVectorChecked<R, K>(sg, j);
     }
   }
 }

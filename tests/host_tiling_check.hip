@@ -1,0 +1,80 @@
+// Host-side check of the kernels' index arithmetic (no GPU needed): for a grid
+// of output addresses, lengths, element sizes, unrolls and alignment classes,
+// every 16-byte vector that overlaps the segment must be handled by exactly one
+// (tile, lane, u), the fast path must only ever see whole in-segment vectors,
+// and nothing outside [0, nv) may be touched.  Uses the very functions the
+// kernels call (fx::planTiles, fx::laneOfTile).
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "fx_reduce_body.hpp"
+
+using namespace fx;
+
+static long checkOne(uint64_t outAddr, uint64_t count, int es, int U, bool co) {
+  const TilePlan tp = planTiles(outAddr, count, es, U, co);
+  const uint64_t ve = 16u / (uint32_t)es, lead = (outAddr & 15u) / (uint32_t)es, end = lead + count;
+  if (count == 0) return 0;  // empty segments never reach a kernel (the launchers return first)
+  std::vector<unsigned char> seen(tp.nv, 0);
+  const uint64_t tiles = tp.tiles();
+  for (uint64_t tile = 0; tile < tiles; tile++) {
+    bool fast0 = false;
+    for (uint32_t tid = 0; tid < (uint32_t)kBlock; tid++) {
+      const TileLane tl = laneOfTile(tp, (uint32_t)tile, tid, U, co);
+      if (tid == 0) fast0 = tl.fast;
+      if (tl.fast != fast0) return 2;                       // the path must be uniform in a workgroup
+      for (int u = 0; u < U; u++) {
+        const uint64_t j = tl.j + (uint64_t)u * tl.stride;
+        if (tl.fast) {
+          if (!co) return 3;                                  // vector loads need co-aligned inputs
+          if (j < tp.firstFull || j >= tp.endFull) return 4;  // whole vectors inside the segment only
+          if (seen[j]++) return 5;
+        } else {
+          if (j >= tl.limit) continue;                        // the checked path's own guard
+          if (j >= tp.nv) return 6;
+          const uint64_t e0 = j * ve;
+          if (e0 >= end || e0 + ve <= lead) continue;         // reduceVectorChecked returns at once
+          if (seen[j]++) return 7;
+        }
+      }
+    }
+  }
+  for (uint64_t j = 0; j < tp.nv; j++) {
+    const uint64_t e0 = j * ve;
+    const bool overlaps = !(e0 >= end || e0 + ve <= lead);
+    if (overlaps != (seen[j] == 1)) return 8;
+  }
+  return 0;
+}
+
+int main() {
+  long cases = 0;
+  const uint64_t MiB = 1ull << 20;
+  const uint64_t bases[] = {0x7f0000000000ull, 0x7f0000000000ull + 512, 0x7f0000000000ull + 96 * 1024 + 16,
+                            0x7f0000000000ull + MiB - 16, 0x7f0000000000ull + 3 * MiB + 4096};
+  for (int es : {1, 2, 4, 8})
+    for (int U : {2, 4, 8})
+      for (bool co : {true, false})
+        for (uint64_t base : bases)
+          for (uint64_t mis = 0; mis < 16; mis += (uint64_t)es * (es == 1 ? 5 : 1)) {
+            const uint64_t V = (uint64_t)U * kBlock * 16 / es;   // elements per tile
+            const uint64_t small[] = {0, 1, 2, 16 / (uint64_t)es - 1, 16 / (uint64_t)es, 16 / (uint64_t)es + 1, V - 1, V,
+                                      V + 1, 3 * V + 7};
+            const uint64_t zone = 4 * MiB / es;
+            const uint64_t big[] = {zone - 1, zone, zone + 1, zone + V * 64 - 3, 2 * zone + 12345, 9 * MiB / es + 1};
+            for (uint64_t c : small) {
+              long rc = checkOne(base + mis, c, es, U, co);
+              cases++;
+              if (rc) { printf("FAIL rc=%ld es=%d U=%d co=%d addr=%llx count=%llu\n", rc, es, U, (int)co, (unsigned long long)(base + mis), (unsigned long long)c); return 1; }
+            }
+            if (mis == 0 || mis == 8 || (es == 2 && mis == 2))
+              for (uint64_t c : big) {
+                long rc = checkOne(base + mis, c, es, U, co);
+                cases++;
+                if (rc) { printf("FAIL rc=%ld es=%d U=%d co=%d addr=%llx count=%llu\n", rc, es, U, (int)co, (unsigned long long)(base + mis), (unsigned long long)c); return 1; }
+              }
+          }
+  printf("ok %ld cases\n", cases);
+  return 0;
+}

@@ -289,3 +289,23 @@ int main(void) {
                    check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
     assert "flagcx_amd" in out
+
+
+def test_kernel_index_arithmetic_on_the_host(tmp_path):
+    """tests/host_tiling_check.hip drives fx::planTiles and fx::laneOfTile -- the
+    functions the kernels themselves call -- over 6,840 (address, length, element
+    size, unroll, alignment class) cases and checks that every vector of a segment
+    is handled exactly once, the unchecked path only ever sees whole in-segment
+    vectors, and nothing outside the segment is touched."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = tmp_path / "host_tiling_check"
+    subprocess.run([hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", f"-I{root}/include",
+                    f"-I{root}/flagcx_amd/csrc", f"{root}/tests/host_tiling_check.hip", "-o", str(exe)], check=True,
+                   capture_output=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.startswith("ok"), out.stdout

@@ -304,7 +304,8 @@ def test_kernel_index_arithmetic_on_the_host(tmp_path):
         pytest.skip("no hipcc")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     exe = tmp_path / "host_tiling_check"
-    subprocess.run([hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", f"-I{root}/include",
+    subprocess.run([hipcc, "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-O2",
+                    "-std=c++17", f"-I{root}/include",
                     f"-I{root}/flagcx_amd/csrc", f"{root}/tests/host_tiling_check.hip", "-o", str(exe)], check=True,
                    capture_output=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True)

@@ -1,0 +1,69 @@
+"""The enqueue-only entry points inside a captured HIP graph: what a caller that
+replays its step as a graph gets.  The graph is replayed several times with the
+program's own eager work and synchronisations between the replays, and every
+replay is compared with the oracle on the inputs it ran on."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from flagcx_amd import _native as N
+from flagcx_amd import kernels as K
+from oracle import fx_oracle as O
+from tests.util import DevBufs, assert_parity, seeded_inputs
+
+pytestmark = pytest.mark.gpu
+
+hip = C.CDLL("libamdhip64.so.7")          # the runtime the library itself is linked against (same mapping)
+hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+hip.hipGraphDestroy.argtypes = [C.c_void_p]
+
+
+def test_reduce_entry_points_replay_correctly_in_a_graph(dev):
+    k, n = 8, 300007
+    dtype, op = N.DT_BF16, N.OP_SUM
+    stream = dev.stream_create()
+    raw = dev.raw_stream(stream)
+    with DevBufs(dev) as b:
+        ins = seeded_inputs(dtype, k, n, seed=1)
+        dins = [b.put(a) for a in ins]
+        dsum, dmax, dcopy = b.alloc(n * 2), b.alloc(n * 2), b.alloc(n * 2)
+        douts = [b.alloc(n * 2) for _ in range(3)]
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(raw, 0) == 0                                  # hipStreamCaptureModeGlobal
+        try:
+            N.check(K.reduce_copy(dsum, dins, n, dtype, op, 0, raw))                    # direct kernel
+            half = n // 2                                                               # two slices with a gap in the table
+            N.check(K.reduce_slices([(dins[:2], dmax, half - 1), ([p + 2 * half for p in dins[:2]], dmax + 2 * half, n - half)],
+                                    2, dtype, N.OP_MAX, raw))                            # kernel-argument table
+            N.check(K.copy_slices([(dsum, dcopy, n * 2)], raw))                         # depends on the first node
+            N.check(K.reduce_bcast_slices([(dins, douts, n)], k, 3, dtype, N.OP_AVG, raw))
+        finally:
+            assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for rep in range(4):
+            if rep:                                   # eager work between replays: new inputs, scrubbed outputs
+                ins = seeded_inputs(dtype, k, n, seed=1 + rep)
+                for d, a in zip(dins, ins):
+                    dev.upload(d, a)
+                for d in [dsum, dmax, dcopy] + douts:
+                    dev.memset(d, 0xEE, n * 2)
+                dev.sync()
+            assert hip.hipGraphLaunch(gexec, raw) == 0
+            dev.stream_sync(stream)
+            want = O.reduce_copy(ins, dtype, op)
+            assert_parity(dev.to_host(dsum, n, np.uint16), want, dtype, op, f"replay {rep} sum")
+            assert np.array_equal(dev.to_host(dcopy, n, np.uint16), dev.to_host(dsum, n, np.uint16))
+            wmax = O.reduce_copy(ins[:2], dtype, N.OP_MAX)
+            wmax[half - 1] = 0xEEEE if rep else dev.to_host(dmax + 2 * (half - 1), 1, np.uint16)[0]   # the gap is not written
+            assert_parity(dev.to_host(dmax, n, np.uint16), wmax, dtype, N.OP_MAX, f"replay {rep} max")
+            avg = O.reduce_copy(ins, dtype, N.OP_AVG)
+            for d in douts:
+                assert_parity(dev.to_host(d, n, np.uint16), avg, dtype, N.OP_AVG, f"replay {rep} avg")
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+    dev.stream_destroy(stream)

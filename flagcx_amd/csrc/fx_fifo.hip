@@ -48,7 +48,13 @@ struct FifoMirror {              // device memory, zeroed at creation
   uint64_t pad[3];
   uint32_t done[kMaxCapacity];   // per slot: workgroups that finished their share
   uint64_t trig[kMaxCapacity][4];
+  // Which trigger number trig[slot] holds (kNoTrigger while it is being
+  // rewritten).  A workgroup that is not needed for a trigger does not hold up
+  // its completion, so it may still be looking at a slot when the ring has come
+  // round and workgroup 0 refills it; the number tells it so.
+  uint64_t trigSeq[kMaxCapacity];
 };
+constexpr uint64_t kNoTrigger = ~0ull;
 
 // Polling uses relaxed atomics (they bypass the non-coherent cache levels on
 // their own); the acquire / release fences are paid only when something changed.
@@ -143,7 +149,7 @@ __global__ void __launch_bounds__(kBlock) clearMirror(uint64_t *words, uint32_t 
 
 __global__ void __launch_bounds__(kBlock)
 fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uint64_t maxIdlePolls) {
-  __shared__ uint64_t sh[6];  // [0] state, [1..4] trigger words
+  __shared__ uint64_t sh[6];  // [0] state, [1..4] trigger words, [5] words valid
   enum { kWork = 0, kExitTerminate = FX_FIFO_EXIT_TERMINATE, kExitIdle = FX_FIFO_EXIT_IDLE };
   uint64_t seq = startSeq;
   uint64_t *hostTrig = host + 4;
@@ -169,10 +175,26 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
             if (mirrored < hp) {
               __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // the triggers behind `produced`
               const uint64_t words = 4 * (hp - mirrored);     // at most 4 * capacity
+              // Refill the slots like a sequence lock: number invalid, words, number
+              // valid.  All of these are agent-scope atomic stores (they go to the
+              // coherent cache level themselves); the workgroup-scope fences between
+              // the phases only make the wavefront wait for one phase's stores to be
+              // acknowledged before it issues the next -- no cache write-back each.
+              for (uint64_t w = lane; w < words; w += 64)
+                if ((w & 3) == 0)
+                  __hip_atomic_store(&m->trigSeq[(mirrored + w / 4) % cap], kNoTrigger, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
               for (uint64_t w = lane; w < words; w += 64) {
                 const uint32_t slot = (uint32_t)((mirrored + w / 4) % cap);
-                m->trig[slot][w & 3] = pollSys(hostTrig + 4 * slot + (w & 3));
+                __hip_atomic_store(&m->trig[slot][w & 3], pollSys(hostTrig + 4 * slot + (w & 3)), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
               }
+              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+              for (uint64_t w = lane; w < words; w += 64)
+                if ((w & 3) == 0)
+                  __hip_atomic_store(&m->trigSeq[(mirrored + w / 4) % cap], mirrored + w / 4, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
               __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // every lane's copies before the new count
               mirrored = hp;
               if (lane == 0) __hip_atomic_store(&m->produced, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -217,9 +239,21 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       if (lane == 0) {
         sh[0] = state;
         if (state == kWork) {
+          // Reader side of the sequence lock.  If the slot still carries number
+          // seq after the words were read, they are trigger seq's.  If not, the
+          // ring has come round: trigger seq is complete, which it could not be
+          // had this workgroup been one of its workers -- so there is nothing to do.
+          // (agent-scope atomic loads read the coherent cache level; the
+          // workgroup-scope fences make each step's loads return before the next
+          // step's are issued, without invalidating anything.)
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
           const uint32_t slot = (uint32_t)(seq % cap);
-          for (int w = 0; w < 4; w++) sh[1 + w] = m->trig[slot][w];
+          const uint64_t before = pollDev(&m->trigSeq[slot]);
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+          for (int w = 0; w < 4; w++) sh[1 + w] = pollDev(&m->trig[slot][w]);
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+          const uint64_t after = pollDev(&m->trigSeq[slot]);
+          sh[5] = (before == seq && after == seq) ? 1 : 0;
         }
       }
     }
@@ -238,7 +272,7 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
     const uint64_t count = w3 & 0xffffffffull;
     const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
     const Share share = shareOf(seq, in1, in2, out, count, dtype, op);
-    if (share.idx >= share.takers) {  // not needed for this trigger
+    if (sh[5] == 0 || share.idx >= share.takers) {  // overtaken by the ring, or not needed for this trigger
       seq++;
       __syncthreads();
       continue;

@@ -158,6 +158,7 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
   uint64_t lastPublished = ~0ull;    // last `completed` written to the host's `consumed`
   bool hostTermSeen = false;
   const uint32_t lane = threadIdx.x;
+  const uint64_t idleLimit = (blockIdx.x == 0 || maxIdlePolls > (~0ull >> 5)) ? maxIdlePolls : maxIdlePolls * 32;
   for (;;) {
     if (threadIdx.x < 64) {
       // Wavefront 0 does the polling.  Reads over PCIe cost microseconds each, so
@@ -233,7 +234,15 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
           termSeen = true;
           continue;
         }
-        if (++idle > maxIdlePolls) { state = kExitIdle; break; }
+        // Workgroup 0 decides when the kernel has idled long enough and tells the
+        // others through the mirror's terminate word, so that all leave together;
+        // their own limit (their polls are several times faster) is only the
+        // backstop that makes every loop finite.
+        if (++idle > idleLimit) {
+          if (blockIdx.x == 0 && lane == 0) storeDev(&m->terminate, (uint64_t)kExitIdle);
+          state = kExitIdle;
+          break;
+        }
         __builtin_amdgcn_s_sleep(32);
       }
       if (lane == 0) {

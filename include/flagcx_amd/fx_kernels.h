@@ -108,7 +108,7 @@ int fx_fifo_terminate(uint64_t *fifo);
  * persistent full-width kernel executes every trigger the host enqueues, for
  * all four ops and types, and marks it Complete; it returns when `terminate`
  * is set and the ring is drained, or after maxIdlePolls consecutive empty
- * polls (so it always ends).  fifoDevicePointer is hostGetDevicePointer() of
+ * polls of the host ring (a few microseconds each; so it always ends).  fifoDevicePointer is hostGetDevicePointer() of
  * the pinned ring, fifoHost the ring itself.  Triggers that sit in the ring at
  * the same time must not depend on each other.  Capacity <= 1024.
  */

@@ -7,8 +7,6 @@
 // unique id is what ties their commInitRank calls together.
 #include <hip/hip_runtime.h>
 
-#include <atomic>
-#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <new>
@@ -31,19 +29,20 @@ flagcxResult_t cclGetVersion(int *version) {
   return flagcxSuccess;
 }
 
-// 4120 bytes of id space; 16 of them are enough to be unique within a process
-// tree: wall clock, pid-independent counter, and the address of a static.
+// 4120 bytes of id space; the simulated-rank layer's 256-byte id (unique within
+// the process) goes into the front of it.
 flagcxResult_t cclGetUniqueId(flagcxInnerUniqueId_t *uniqueId) {
   if (!uniqueId) return flagcxInvalidArgument;
   if (*uniqueId == nullptr) {
     *uniqueId = static_cast<flagcxInnerUniqueId *>(calloc(1, sizeof(flagcxInnerUniqueId)));
     if (*uniqueId == nullptr) return flagcxSystemError;
   }
-  static std::atomic<uint64_t> counter{0};
-  uint64_t words[3] = {(uint64_t)std::chrono::steady_clock::now().time_since_epoch().count(), ++counter,
-                       (uint64_t)(uintptr_t)&counter};
+  flagcxUniqueId id;
+  flagcxResult_t rc = flagcxGetUniqueId(&id);
+  if (rc != flagcxSuccess) return rc;
+  static_assert(sizeof((*uniqueId)->internal) >= sizeof(id.internal), "inner id holds the group id");
   memset((*uniqueId)->internal, 0, sizeof((*uniqueId)->internal));
-  memcpy((*uniqueId)->internal, words, sizeof(words));
+  memcpy((*uniqueId)->internal, id.internal, sizeof(id.internal));
   return flagcxSuccess;
 }
 
@@ -71,7 +70,7 @@ flagcxResult_t cclCommInitRank(flagcxInnerComm_t *comm, int nranks, flagcxInnerU
   if (!comm || !commId) return flagcxInvalidArgument;
   flagcxInnerComm *c = *comm ? *comm : static_cast<flagcxInnerComm *>(calloc(1, sizeof(flagcxInnerComm)));
   if (!c) return flagcxSystemError;
-  flagcxResult_t rc = fxSimCommInitRank(&c->base, nranks, commId->internal, 64, rank);
+  flagcxResult_t rc = fxSimCommInitRank(&c->base, nranks, commId->internal, FLAGCX_UNIQUE_ID_BYTES, rank);
   if (rc != flagcxSuccess) {
     if (!*comm) free(c);
     return rc;

@@ -453,3 +453,48 @@ def test_host_order_matches_the_reference_host_ring(dev, stream, dname, n, count
         dev.stream_sync(stream)
         for r in range(n):
             assert_parity(dev.to_host(dr[r], rc, npdt), outs[r], dtype, N.OP_SUM, f"host order reduce-scatter rank {r}")
+
+
+def test_single_rank_and_empty_collectives(dev, stream):
+    """nranks == 1 is a copy when out of place and nothing when in place
+    (uni_runner_impl.cc:359-379, bootstrap.cc:1001-1006); count == 0 is accepted
+    everywhere and touches nothing."""
+    count = 1000
+    x = np.arange(count, dtype=np.float32)
+    with DevBufs(dev) as b, S.SimGroup(1) as g:
+        dx, dy = b.put(x), b.alloc(count * 4)
+        for order in (S.ORDER_RANK, S.ORDER_RING, S.ORDER_TREE, S.ORDER_HOST):
+            for algo in (S.ALGO_DIRECT, S.ALGO_RING):
+                g.configure(order=order, algo=algo)
+                dev.memset(dy, 0, count * 4)
+                N.check(g.all_reduce([dx], [dy], count, N.DT_FP32, N.OP_SUM, stream))
+                N.check(g.all_reduce([dx], [dx], count, N.DT_FP32, N.OP_MAX, stream))       # in place
+                dev.stream_sync(stream)
+                assert np.array_equal(dev.to_host(dy, count, np.float32), x)
+                assert np.array_equal(dev.to_host(dx, count, np.float32), x)
+        for call in (lambda: g.reduce([dx], [dy], count, N.DT_FP32, N.OP_AVG, 0, stream),
+                     lambda: g.reduce_scatter([dx], [dy], count, N.DT_FP32, N.OP_SUM, stream),
+                     lambda: g.all_gather([dx], [dy], count, N.DT_FP32, stream)):
+            dev.memset(dy, 0, count * 4)
+            N.check(call())
+            dev.stream_sync(stream)
+            assert np.array_equal(dev.to_host(dy, count, np.float32), x)
+    with DevBufs(dev) as b, S.SimGroup(4) as g:
+        p = [b.alloc(64) for _ in range(4)]
+        for q in p:
+            dev.memset(q, 0x77, 64)
+        zeros = np.zeros((4, 4), np.int64)
+        for order in (S.ORDER_RANK, S.ORDER_HOST):
+            g.configure(order=order)
+            N.check(g.all_reduce(p, p, 0, N.DT_FP32, N.OP_SUM, stream))
+            N.check(g.reduce(p, p, 0, N.DT_BF16, N.OP_MAX, 2, stream))
+            N.check(g.reduce_scatter(p, p, 0, N.DT_INT8, N.OP_PROD, stream))
+        N.check(g.all_gather(p, p, 0, N.DT_FP64, stream))
+        N.check(g.all_to_allv(p, zeros, zeros, p, zeros, zeros, N.DT_FP32, stream))
+        dev.stream_sync(stream)
+        for q in p:
+            assert (dev.to_host(q, 64, np.uint8) == 0x77).all()
+        # arguments the API must refuse without touching the device
+        assert g.reduce(p, p, 4, N.DT_FP32, N.OP_SUM, 4, stream) == N.INVALID_ARGUMENT          # root out of range
+        assert N.lib.flagcxAllReduce(p[0], p[0], 4, N.DT_FP32, N.OP_SUM, g.comms[0], None) == N.INVALID_ARGUMENT
+        assert N.lib.flagcxAllReduce(None, p[0], 4, N.DT_FP32, N.OP_SUM, g.comms[0], stream) == N.INVALID_ARGUMENT

@@ -106,10 +106,11 @@ int fx_fifo_terminate(uint64_t *fifo);
  * FIFO-compatible consumer: the drop-in for flagcxLaunchCollectiveKernel
  * (flagcx/adaptor/kernel/nvidia/flagcx_reduce_kernel_device.cu:88-192).  A
  * persistent full-width kernel executes every trigger the host enqueues, for
- * all four ops and types, and marks it Complete; it returns when `terminate`
+ * every op and type, and marks it Complete; it returns when `terminate`
  * is set and the ring is drained, or after maxIdlePolls consecutive empty
- * polls of the host ring (a few microseconds each; so it always ends).  fifoDevicePointer is hostGetDevicePointer() of
- * the pinned ring, fifoHost the ring itself.  Triggers that sit in the ring at
+ * polls of the host ring (a few microseconds each; so it always ends).
+ * fifoDevicePointer is hostGetDevicePointer() of the pinned ring, fifoHost
+ * the ring itself.  Triggers that sit in the ring at
  * the same time must not depend on each other.  Capacity <= 1024.
  */
 typedef struct fxFifoConsumer *fxFifoConsumer_t;

@@ -68,6 +68,21 @@ def main():
                                        "recv_len": rlen, "send_sha256": W.digest(send),
                                        "packed_sha256": W.digest(packed), "unpacked_sha256": W.digest(recv)}
 
+    # every element type x every op at a small size, plus the three reference schedules on one fp32 case
+    g["matrix"] = {}
+    for dname, dtype in W.ALL_DTYPES.items():
+        ins = W.matrix_inputs(dtype)
+        for oname, op in W.ALL_OPS.items():
+            g["matrix"][f"{dname}_{oname}"] = entry(ins, O.reduce_copy(ins, dtype, op))
+    sends = W.inputs(N.DT_FP32, 5, 1003, (0, -1000.0, 1000.0), 6, 1)
+    g["schedules_fp32_sum_5x1003"] = {
+        "inputs_sha256": [W.digest(a) for a in sends],
+        "ring": W.digest(O.ring_allreduce(sends, N.DT_FP32, N.OP_SUM)[0]),
+        "tree_root2": W.digest(O.tree_reduce(sends, 2, N.DT_FP32, N.OP_SUM)),
+        "host": W.digest(O.bootstrap_allreduce(sends, N.DT_FP32, N.OP_SUM)[0]),
+        "rank": W.digest(O.reduce_copy(sends, N.DT_FP32, N.OP_SUM)),
+    }
+
     c = W.CFG5
     for label, n in (("cfg5_bf16_sum_8x4194304", 4_194_304),) + ((("cfg5_bf16_sum_8x268435456", c["n"]),) if full else ()):
         ins = W.inputs(c["dtype"], c["k"], n, c["dist"], c["seed"])

@@ -32,6 +32,25 @@ def cfg3_inputs(dtype, n, threads=8):
     return inputs(dtype, CFG3["k"], n, CFG3["dists"][dtype], CFG3["seed"], threads, first_stream=16 * dtype)
 
 
+ALL_OPS = dict(OPS, avg=N.OP_AVG)
+ALL_DTYPES = {"int8": N.DT_INT8, "uint8": N.DT_UINT8, "int32": N.DT_INT32, "uint32": N.DT_UINT32, "int64": N.DT_INT64,
+              "uint64": N.DT_UINT64, "fp16": N.DT_FP16, "fp32": N.DT_FP32, "fp64": N.DT_FP64, "bf16": N.DT_BF16}
+
+
+def matrix_inputs(dtype, k=3, n=4099, seed=5):
+    """Small seeded inputs for every element type: the synthetic generator for
+    the types it knows, numpy's PCG64 over the whole integer range otherwise."""
+    if dtype in (N.DT_FP32, N.DT_FP64):
+        return inputs(dtype, k, n, (K.SYNTH_UNIFORM, -1.0, 1.0), seed, 1)
+    if dtype in (N.DT_FP16, N.DT_BF16):
+        return inputs(dtype, k, n, (K.SYNTH_NORMAL, 0.0, 1.0), seed, 1)
+    if dtype == N.DT_INT32:
+        return inputs(dtype, k, n, (K.SYNTH_UNIFORM_INT, -(1 << 20), 1 << 20), seed, 1)
+    t = np.dtype(N.NP_DTYPE[dtype])
+    return [np.random.Generator(np.random.PCG64([seed, p, dtype])).integers(np.iinfo(t).min, np.iinfo(t).max, n, dtype=t,
+                                                                            endpoint=True) for p in range(k)]
+
+
 def cfg4_layout():
     """Per-peer counts log-uniform in [1, 4194304] from seed 3 and random
     non-overlapping displacements (shuffled segment order, gaps of 0..63
@@ -66,5 +85,5 @@ def probe(arr, m=8):
     """A few raw words from fixed positions, for a readable diff when a digest fails."""
     a = np.ascontiguousarray(arr)
     idx = [0, 1, a.size // 3, a.size // 2, a.size - 1][:m]
-    w = a.view({2: np.uint16, 4: np.uint32}[a.itemsize])
+    w = a.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.itemsize])
     return [int(w[i]) for i in idx if a.size]

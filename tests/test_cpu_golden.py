@@ -70,3 +70,20 @@ def test_cfg4_layout_and_digests():
     packed = O.pack(send, counts, sd)
     assert W.digest(packed) == e["packed_sha256"]
     assert W.digest(O.unpack(np.zeros(rlen, np.float32), packed, counts, rd)) == e["unpacked_sha256"]
+
+
+def test_every_type_and_op_small_matrix():
+    for dname, dtype in W.ALL_DTYPES.items():
+        ins = W.matrix_inputs(dtype)
+        for oname, op in W.ALL_OPS.items():
+            _check(GOLDEN["matrix"][f"{dname}_{oname}"], ins, O.reduce_copy(ins, dtype, op))
+
+
+def test_reference_schedules_on_one_case():
+    e = GOLDEN["schedules_fp32_sum_5x1003"]
+    sends = W.inputs(N.DT_FP32, 5, 1003, (0, -1000.0, 1000.0), 6, 1)
+    assert [W.digest(a) for a in sends] == e["inputs_sha256"]
+    got = {"ring": O.ring_allreduce(sends, N.DT_FP32, N.OP_SUM)[0], "tree_root2": O.tree_reduce(sends, 2, N.DT_FP32, N.OP_SUM),
+           "host": O.bootstrap_allreduce(sends, N.DT_FP32, N.OP_SUM)[0], "rank": O.reduce_copy(sends, N.DT_FP32, N.OP_SUM)}
+    assert {k: W.digest(v) for k, v in got.items()} == {k: e[k] for k in got}
+    assert len({e[k] for k in got}) == 4, "the four schedules are expected to round differently on this case"

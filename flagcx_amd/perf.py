@@ -224,8 +224,11 @@ def run_allreduce(dev, a):
             nbytes = size(a.min)
             while nbytes <= emax:
                 cnt = nbytes // es
-                row(f"allreduce n={n} {a.dtype} {'ring' if algo else 'direct'}", nbytes,
-                    t.ms(lambda: N.check(g.all_reduce(ds, dr, cnt, dtype, OP[a.op], t.stream))), nbytes)
+                ms = t.ms(lambda: N.check(g.all_reduce(ds, dr, cnt, dtype, OP[a.op], t.stream)))
+                alg = nbytes / ms / 1e6
+                # algBw = size / time, busBw = algBw * 2 (n - 1) / n, as test/perf/host_api/test_allreduce.cpp:11
+                print(f"{'allreduce n=%d %s %s' % (n, a.dtype, 'ring' if algo else 'direct'):<44s} size {nbytes:>12d} B   "
+                      f"{ms * 1e3:10.2f} us   algBw {alg:9.1f} GB/s   busBw {alg * 2 * (n - 1) / n:9.1f} GB/s", flush=True)
                 nbytes *= a.factor
 
 

@@ -429,7 +429,9 @@ int fx_fifo_consumer_launch(fxFifoConsumer_t c, void *fifoDevicePointer, const u
   const uint32_t words = (uint32_t)(sizeof(FifoMirror) / sizeof(uint64_t));
   hipLaunchKernelGGL(clearMirror, dim3((words + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (uint64_t *)c->mirror, words);
   FX_HIP(hipGetLastError());
-  const uint64_t startSeq = fifoHost[2];  // triggers produced before this launch are not ours
+  // Start where the last consumer stopped: triggers enqueued before this launch
+  // are waiting between `consumed` and `produced` and are served first.
+  const uint64_t startSeq = __atomic_load_n(&fifoHost[1], __ATOMIC_ACQUIRE);
   hipLaunchKernelGGL(fifoConsumer, dim3(c->grid), dim3(kBlock), 0, s, (uint64_t *)fifoDevicePointer, c->mirror,
                      c->capacity, startSeq, (uint64_t)maxIdlePolls);
   FX_HIP(hipGetLastError());

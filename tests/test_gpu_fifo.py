@@ -128,3 +128,46 @@ def test_consumer_ends_by_itself_when_idle(dev):
     assert time.time() - t0 < DEADLINE
     reason, done, bad = ring.close()
     assert (reason, done, bad) == (2, 0, 0)                          # FX_FIFO_EXIT_IDLE
+
+
+def test_triggers_enqueued_before_the_launch_are_served(dev):
+    """The consumer starts at the ring's `consumed` index, so what the host put in
+    the ring before launching it is executed first."""
+    cap, n = 8, 70001
+    host = dev.malloc(lib.fx_fifo_bytes(cap), N.MEM_HOST)
+    N.check(lib.fx_fifo_init(host, cap))
+    a, c = seeded_inputs(N.DT_FP32, 2, n, seed=3)
+    with DevBufs(dev) as b:
+        da, dc = b.put(a), b.put(c)
+        outs = [b.alloc(n * 4) for _ in range(3)]
+        idx = C.c_int(-1)
+        slots = []
+        for o, op in zip(outs[:2], (N.OP_SUM, N.OP_MIN)):            # two triggers wait in the ring
+            N.check(lib.fx_fifo_enqueue(host, da, dc, o, n, 32, N.DT_FP32, op, C.byref(idx)))
+            assert idx.value >= 0
+            slots.append(idx.value)
+        dptr = C.c_void_p()
+        N.check(dev.t.hostGetDevicePointer(C.byref(dptr), host))
+        stream = dev.stream_create()
+        cons = C.c_void_p()
+        N.check(lib.fx_fifo_consumer_create(C.byref(cons), cap))
+        N.check(lib.fx_fifo_consumer_launch(cons, dptr, host, POLL_LIMIT, dev.raw_stream(stream)))
+        N.check(lib.fx_fifo_enqueue(host, da, dc, outs[2], n, 32, N.DT_FP32, N.OP_MAX, C.byref(idx)))   # and one after
+        slots.append(idx.value)
+        t0 = time.time()
+        try:
+            for s in slots:
+                while lib.fx_fifo_poll_state(host, s) != COMPLETE:
+                    assert time.time() - t0 < DEADLINE, "a trigger enqueued before the launch was never served"
+                N.check(lib.fx_fifo_set_state(host, s, AVAILABLE))
+        finally:
+            lib.fx_fifo_terminate(host)
+            dev.stream_sync(stream)
+        for o, op in zip(outs, (N.OP_SUM, N.OP_MIN, N.OP_MAX)):
+            assert_parity(dev.to_host(o, n, np.float32), O.reduce2(a, c, N.DT_FP32, op), N.DT_FP32, op, f"op {op}")
+        reason, done, bad = C.c_int(-1), C.c_uint64(), C.c_uint64()
+        N.check(lib.fx_fifo_consumer_status(cons, C.byref(reason), C.byref(done), C.byref(bad)))
+        assert (reason.value, done.value, bad.value) == (1, 3, 0)
+        lib.fx_fifo_consumer_destroy(cons)
+        dev.stream_destroy(stream)
+    dev.free(host, N.MEM_HOST)

@@ -260,3 +260,30 @@ def test_counts_beyond_32_bit_offsets(dev, dname, dtype, count):
                     want[lo - off:hi - off] = O.reduce2(a[0], a[1], dtype, N.OP_SUM)
             assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), f"{dname}: window at element {off}"
         assert (dev.to_host(dout + nbytes, 256, np.uint8) == 0xEE).all(), "wrote past the end"
+
+
+def test_cfg5_through_the_collective(dev, stream):
+    """The headline workload as one flagcxAllReduce over 8 simulated ranks (every
+    rank sends 512 MiB of bf16, every rank receives the 8-way sum): first and
+    last rank's results hash to the committed digest, the others agree with them
+    on sampled windows."""
+    c = W.CFG5
+    n, k = c["n"], c["k"]
+    gold = GOLDEN["cfg5_bf16_sum_8x268435456"]
+    with DevBufs(dev) as b, S.SimGroup(k) as g:
+        ds = []
+        for p in range(k):
+            host = K.synth(n, c["dtype"], *c["dist"], c["seed"], p, THREADS)
+            ds.append(b.put(host))
+        del host
+        dr = [b.alloc(n * 2) for _ in range(k)]
+        N.check(g.all_reduce(ds, dr, n, c["dtype"], N.OP_SUM, stream), "flagcxAllReduce")
+        dev.stream_sync(stream)
+        first = dev.to_host(dr[0], n, np.uint16)
+        assert W.digest(first) == gold["out_sha256"], "rank 0"
+        assert W.digest(dev.to_host(dr[k - 1], n, np.uint16)) == gold["out_sha256"], f"rank {k - 1}"
+        win = 1 << 19
+        for r in range(1, k - 1):
+            for pos in np.linspace(0, n - win, 9).astype(np.int64):
+                got = dev.to_host(dr[r] + int(pos) * 2, win, np.uint16)
+                assert np.array_equal(got, first[pos:pos + win]), f"rank {r} window at {pos}"

@@ -1,6 +1,6 @@
 """MI355X-native reduce / slice / pack path behind FlagCX's plugin boundary.
 
-The product is the three shared libraries under ``flagcx_amd/lib`` (built from
+The product is the shared libraries under ``flagcx_amd/lib`` (built from
 ``flagcx_amd/csrc`` by ``python -m flagcx_amd.build``).  This package is the thin
 ctypes glue the tests and the benchmark use to call their C ABI; it contains no
 arithmetic and has no CPU fallback: a missing library is an ImportError.

@@ -38,6 +38,22 @@ def test_kernel_library_exports_every_declared_symbol():
     assert set(N.exported_symbols()) <= declared          # the binding uses nothing undeclared
 
 
+def test_kernels_only_library_exports_fx_and_nothing_flagcx():
+    """The library a FlagCX build links into libflagcx.so must not bring a second
+    flagcxAllReduce: it exports every fx_* function of the kernel header and of
+    the partition API, and no other dynamic symbol."""
+    import subprocess
+    path = os.path.join(N.LIB_DIR, "libflagcx-kernels-mi355x.so")
+    out = subprocess.run(["nm", "-D", "--defined-only", path], check=True, capture_output=True, text=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    assert exported and all(s.startswith("fx_") for s in exported), sorted(exported)[:10]
+    wanted = {n for n in _declared_functions() if n.startswith("fx_") and n != "fx_synth_fill"}
+    assert wanted <= exported, sorted(wanted - exported)
+    lib = C.CDLL(path)
+    lib.fx_version.restype = C.c_char_p
+    assert lib.fx_version().startswith(b"flagcx_amd")
+
+
 def test_plugin_passes_the_reference_loader_checks():
     t = adaptor.load_plugin()
     assert t.name == b"MI355X"

@@ -1,0 +1,22 @@
+"""PyTorch-ROCm tensors and streams driving the library, the way the reference's
+torch backend does (plugin/torch/flagcx/src/backend_flagcx.cpp: data_ptr(),
+numel(), dtype / ReduceOp mapped to FlagCX enums, the current stream wrapped
+with streamCopy).  The client runs in a process of its own so that torch's
+bundled HIP runtime is loaded there and not under the other GPU tests."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_torch_tensors_through_the_wrapper(dev):
+    pytest.importorskip("torch")
+    env = dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    r = subprocess.run([sys.executable, "-u", os.path.join(ROOT, "tests", "torch_client.py")], cwd=ROOT, env=env,
+                       capture_output=True, text=True, timeout=420)
+    assert r.returncode == 0 and "torch client ok" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]

@@ -270,6 +270,13 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
     const uint64_t state = sh[0];
     if (state != kWork) {
       if (threadIdx.x == 0 && blockIdx.x == 0) {
+        // Workers may still be inside the last triggers.  `consumed` is where the
+        // next launch starts, so it must not be published short of them: wait
+        // (bounded, like every loop here) until all mirrored triggers are complete.
+        const uint64_t owed = mirrored - startSeq;
+        const uint64_t patience = (maxIdlePolls > (~0ull >> 5)) ? maxIdlePolls : maxIdlePolls * 32;
+        for (uint64_t spins = 0; pollDev(&m->completed) < owed && spins <= patience; spins++)
+          __builtin_amdgcn_s_sleep(32);
         storeSys(host + 1, startSeq + pollDev(&m->completed));
         storeDev(&m->exitReason, state);
       }

@@ -64,6 +64,7 @@ struct Group {
   std::mutex mu;
   std::string id;          // non-empty when created rank by rank (fxSimCommInitRank)
   int joined = 0, alive = 0;
+  std::vector<char> taken;  // ranks that have joined
   std::vector<PendingP2p> p2p;
   uint64_t nextP2pId = 1;
   std::map<uint64_t, flagcxResult_t> p2pMatched;  // rendezvous mode: verdicts awaiting their sleeping poster
@@ -531,6 +532,7 @@ flagcxResult_t runAlltoAllv(const Ctx &c) {
       const size_t cnt = g->posts[r].sendcounts[i];
       if (cnt != g->posts[i].recvcounts[r]) return flagcxInvalidArgument;
       tot += cnt;
+      if (cnt && (!c.send(r) || !c.recv(i))) return flagcxInvalidArgument;
       if (cnt) {
         const uintptr_t s = (uintptr_t)c.send(r) + g->posts[r].sdispls[i] * ts;
         const uintptr_t d = (uintptr_t)c.recv(i) + g->posts[i].rdispls[r] * ts;
@@ -821,6 +823,7 @@ flagcxResult_t newGroup(int nranks, Group **out) {
   try {
     g->posts.resize(nranks);
     g->ready.assign(nranks, nullptr);
+    g->taken.assign(nranks, 0);
   } catch (...) {
     delete g;
     throw;
@@ -992,11 +995,12 @@ flagcxResult_t fxSimCommInitRank(flagcxComm_t *comm, int nranks, const void *id,
       }
     } else {
       g = it->second;
-      if (g->n != nranks) {
+      if (g->n != nranks || g->taken[rank]) {  // a different group size, or this rank has joined already
         delete c;
         return flagcxInvalidArgument;
       }
     }
+    g->taken[rank] = 1;
     g->joined++;
     g->alive++;
     if (g->joined == nranks) gRegistry.erase(key);  // complete: the id may be reused for a new group

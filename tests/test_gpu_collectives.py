@@ -197,6 +197,8 @@ def test_alltoallv_matches_oracle(dev, stream):
         bad = counts.T.copy()
         bad[0, 1] += 1                                             # receiver expects more than is sent
         assert g.all_to_allv(ds, counts, sd, dr, bad, rd, N.DT_FP32, stream) == N.INVALID_ARGUMENT
+        # a rank with something to send and no send buffer is refused before anything is launched
+        assert g.all_to_allv([None] + ds[1:], counts, sd, dr, counts.T, rd, N.DT_FP32, stream) == N.INVALID_ARGUMENT
         # in place (send == recv, uneven blocks laid out back to back): goes through the staging slots
         blk = np.array([[1000 + 37 * ((r + i) % n) for i in range(n)] for r in range(n)], np.int64)   # symmetric
         disp = np.concatenate([np.zeros((n, 1), np.int64), np.cumsum(blk, axis=1)[:, :-1]], axis=1)

@@ -171,3 +171,54 @@ def test_triggers_enqueued_before_the_launch_are_served(dev):
         lib.fx_fifo_consumer_destroy(cons)
         dev.stream_destroy(stream)
     dev.free(host, N.MEM_HOST)
+
+
+def test_second_launch_does_not_repeat_a_trigger_that_was_running_at_terminate(dev):
+    """terminate right behind a large in-place trigger: the consumer leaves only
+    after that trigger is complete and `consumed` says so, so a second consumer
+    on the same ring starts behind it (a repeat would add input 2 twice)."""
+    cap, n = 4, 24 << 20
+    host = dev.malloc(lib.fx_fifo_bytes(cap), N.MEM_HOST)
+    N.check(lib.fx_fifo_init(host, cap))
+    words = np.ctypeslib.as_array(C.cast(host, C.POINTER(C.c_uint64)), shape=(4,))
+    a, c = seeded_inputs(N.DT_FP32, 2, n, seed=21)
+    small = seeded_inputs(N.DT_INT32, 2, 1000, seed=22)
+    with DevBufs(dev) as b:
+        da, dc = b.put(a), b.put(c)
+        ds0, ds1, dso = b.put(small[0]), b.put(small[1]), b.alloc(4000)
+        dptr = C.c_void_p()
+        N.check(dev.t.hostGetDevicePointer(C.byref(dptr), host))
+        stream = dev.stream_create()
+        cons = C.c_void_p()
+        N.check(lib.fx_fifo_consumer_create(C.byref(cons), cap))
+        idx = C.c_int(-1)
+        try:
+            N.check(lib.fx_fifo_consumer_launch(cons, dptr, host, POLL_LIMIT, dev.raw_stream(stream)))
+            N.check(lib.fx_fifo_enqueue(host, da, dc, da, n, 32, N.DT_FP32, N.OP_SUM, C.byref(idx)))   # a += c
+            assert idx.value == 0
+        finally:
+            lib.fx_fifo_terminate(host)                               # without waiting for Complete
+            dev.stream_sync(stream)
+        assert lib.fx_fifo_poll_state(host, 0) == COMPLETE
+        assert int(words[1]) == int(words[2]) == 1                    # consumed == produced
+        N.check(lib.fx_fifo_set_state(host, 0, AVAILABLE))
+        words[3] = 0                                                  # same ring, new session
+        try:
+            N.check(lib.fx_fifo_consumer_launch(cons, dptr, host, POLL_LIMIT, dev.raw_stream(stream)))
+            N.check(lib.fx_fifo_enqueue(host, ds0, ds1, dso, 1000, 32, N.DT_INT32, N.OP_MAX, C.byref(idx)))
+            assert idx.value == 1
+            t0 = time.time()
+            while lib.fx_fifo_poll_state(host, 1) != COMPLETE:
+                assert time.time() - t0 < DEADLINE, "second session's trigger never completed"
+        finally:
+            lib.fx_fifo_terminate(host)
+            dev.stream_sync(stream)
+        assert_parity(dev.to_host(da, n, np.float32), O.reduce2(a, c, N.DT_FP32, N.OP_SUM), N.DT_FP32, N.OP_SUM, "once")
+        assert_parity(dev.to_host(dso, 1000, np.int32), O.reduce2(small[0], small[1], N.DT_INT32, N.OP_MAX), N.DT_INT32,
+                      N.OP_MAX, "second session")
+        reason, done, bad = C.c_int(-1), C.c_uint64(), C.c_uint64()
+        N.check(lib.fx_fifo_consumer_status(cons, C.byref(reason), C.byref(done), C.byref(bad)))
+        assert (reason.value, done.value, bad.value) == (1, 1, 0)     # the second session completed one trigger
+        lib.fx_fifo_consumer_destroy(cons)
+        dev.stream_destroy(stream)
+    dev.free(host, N.MEM_HOST)

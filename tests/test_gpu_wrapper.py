@@ -37,6 +37,15 @@ def test_life_cycle_and_errors(dev, fx):
         fx.flagcxAllReduce(None, None, 4, DT.flagcxFloat, OP.flagcxSum, comms[0], stream)
     with pytest.raises(ValueError):
         fx.unique_id_from_bytes(b"short")
+    # a rank joins a communicator once; a late joiner must agree on its size
+    uid = fx.flagcxGetUniqueId()
+    half = fx.flagcxCommInitRank(2, uid, 0)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        fx.flagcxCommInitRank(2, uid, 0)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        fx.flagcxCommInitRank(3, uid, 1)
+    other = fx.flagcxCommInitRank(2, uid, 1)
+    comms += [half, other]
     for c in comms:
         fx.flagcxCommDestroy(c)
     fx.adaptor_stream_destroy(stream)

@@ -67,7 +67,7 @@ struct Group {
   std::vector<char> taken;  // ranks that have joined
   std::vector<PendingP2p> p2p;
   uint64_t nextP2pId = 1;
-  std::map<uint64_t, flagcxResult_t> p2pMatched;  // rendezvous mode: verdicts awaiting their sleeping poster
+  std::map<uint64_t, flagcxResult_t> p2pMatched;  // rendezvous mode: results awaiting their sleeping poster
   // pending collective
   Kind kind = kNone;
   size_t count = 0;
@@ -196,9 +196,10 @@ void hostChunk(size_t count, int n, int i, size_t *cnt, size_t *off) {
 // chunk c.  The ring computes x_c (op) (x_{c-1} (op) (.. (x_{c+2} (op) x_{c+1}))),
 // local operand first (bootstrap.cc:805-871).  For sum / prod / avg the operands
 // of one step commute bit for bit, so the fold runs c+1, c+2, .., c.  For max /
-// min ((a < b) ? b : a keeps the LOCAL value on a tie) the fold keeps its
-// accumulator on a tie instead, so it runs c, c-1, .., c+1: either way the last
-// rank of the ring wins ties.
+// min of integers ((a < b) ? b : a keeps the LOCAL value on a tie) the fold keeps
+// its accumulator on a tie instead, so it runs c, c-1, .., c+1: either way the
+// last rank of the ring wins ties.  (Floating max / min do not come here: NaN
+// makes them order-dependent in a way only the step-by-step chain reproduces.)
 void hostOrder(int c, int n, int op, std::vector<int> &order) {
   order.resize(n);
   const bool select = (op == flagcxMax || op == flagcxMin);
@@ -213,7 +214,74 @@ struct HostPiece {
   std::vector<void *> outs;
 };
 
+// max / min of floating types, exactly as the host ring evaluates them: n-1
+// two-input steps res = local (op) received (bootstrap.cc:853-871), the local
+// operand first, so that a NaN met on the way decides the result the way it
+// does there (std::max / std::min return their FIRST argument whenever the
+// comparison is false).  A left-to-right k-way fold cannot express that: once
+// rank j's NaN has been kept by rank j, everything folded before it is lost.
+// Step j of chunk c: local rank c+1+j, received = the previous partial (rank
+// c+1's data in step 1).  Partials travel through scratch; the last step, whose
+// local rank is c itself, writes the outputs.  One launch per step for all chunks.
+flagcxResult_t chainHostPieces(const Ctx &c, const std::vector<HostPiece> &pieces) {
+  Group *g = c.g;
+  const int n = c.n;
+  std::vector<size_t> soff(pieces.size(), 0);
+  size_t total = 0;
+  for (size_t i = 0; i < pieces.size(); i++) {
+    soff[i] = total;
+    total += (pieces[i].cnt * c.ts + 255) & ~(size_t)255;
+  }
+  if (total == 0) return flagcxSuccess;
+  if (n > 2) {
+    flagcxResult_t rc = ensureScratch(g, total);
+    if (rc != flagcxSuccess) return rc;
+  }
+  std::vector<fxSliceDesc> plain, copies;
+  std::vector<fxBcastDesc> bcast;
+  int nout = 1;
+  for (int j = 1; j < n; j++) {
+    plain.clear();
+    for (size_t i = 0; i < pieces.size(); i++) {
+      const HostPiece &p = pieces[i];
+      if (p.cnt == 0) continue;
+      const void *local = cadd(c.send(mod(p.chunk + 1 + j, n)), p.off * c.ts);
+      const void *received = (j == 1) ? cadd(c.send(mod(p.chunk + 1, n)), p.off * c.ts)
+                                      : (const void *)madd(g->scratch, soff[i]);
+      nout = (int)p.outs.size();
+      if (j == n - 1 && nout > 1 && nout <= FX_MAX_SLICE_INPUTS) {
+        fxBcastDesc d;
+        memset(&d, 0, sizeof(d));
+        d.in[0] = local;
+        d.in[1] = received;
+        for (int o = 0; o < nout; o++) d.out[o] = p.outs[o];
+        d.count = p.cnt;
+        bcast.push_back(d);
+        continue;
+      }
+      fxSliceDesc d;
+      memset(&d, 0, sizeof(d));
+      d.in[0] = local;
+      d.in[1] = received;
+      d.out = (j == n - 1) ? p.outs[0] : madd(g->scratch, soff[i]);
+      d.count = p.cnt;
+      plain.push_back(d);
+      if (j == n - 1)
+        for (int o = 1; o < nout; o++) copies.push_back(copyDesc(p.outs[0], p.outs[o], p.cnt * c.ts));
+    }
+    flagcxResult_t rc = R(fx_reduce_slices(plain.data(), plain.size(), 2, g->dtype, g->op, c.s));
+    if (rc != flagcxSuccess) return rc;
+  }
+  if (!bcast.empty()) return R(fx_reduce_bcast_slices(bcast.data(), bcast.size(), 2, nout, g->dtype, g->op, c.s));
+  return R(fx_copy_slices(copies.data(), copies.size(), c.s));
+}
+
+inline bool isFloating(int dtype) {
+  return dtype == flagcxFloat16 || dtype == flagcxBfloat16 || dtype == flagcxFloat32 || dtype == flagcxFloat64;
+}
+
 flagcxResult_t reduceHostPieces(const Ctx &c, const std::vector<HostPiece> &pieces) {
+  if ((c.g->op == flagcxMax || c.g->op == flagcxMin) && isFloating(c.g->dtype)) return chainHostPieces(c, pieces);
   std::vector<int> order;
   std::vector<fxBcastDesc> bcast;
   std::vector<fxSliceDesc> plain;
@@ -677,7 +745,7 @@ void resetPending(Group *g) {
 }
 
 // Drop the pending collective because of a caller error; ranks asleep in a
-// rendezvous get the same verdict.
+// rendezvous get the same result.
 void abandonPending(Group *g, flagcxResult_t why) {
   resetPending(g);
   g->lastResult = why;
@@ -806,7 +874,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   return res;
 }
 
-// Argument screening shared by the reducing collectives: same verdicts as the
+// Argument screening shared by the reducing collectives: same results as the
 // kernel layer (unsupported-but-known -> flagcxNotSupported).
 flagcxResult_t screenReduce(int dtype, int op) {
   if (dtype < 0 || dtype >= flagcxNumTypes || op < 0 || op >= flagcxNumRedOps) return flagcxInvalidArgument;

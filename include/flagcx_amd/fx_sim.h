@@ -106,8 +106,10 @@ enum {
                         element, chunk c folded along the ring c+1, c+2, .., c
                         as local (op) received.  AllReduce, Reduce and
                         ReduceScatter; bit-identical to that path for every type
-                        it carries, +-0 ties of max / min included (a NaN operand
-                        of max / min is the one case not reproduced)           */
+                        it carries, +-0 ties and NaN operands of max / min
+                        included (floating max / min run as the ring's n-1
+                        two-input steps for that; everything else as one k-way
+                        launch per collective)                                 */
 };
 flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value);
 

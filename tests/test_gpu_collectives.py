@@ -427,6 +427,8 @@ def test_host_order_matches_the_reference_host_ring(dev, stream, dname, n, count
         sends = [(a * 10.0 ** rng.integers(-3, 9, count)).astype(npdt) for a in sends]
         for r, a in enumerate(sends):                 # and plant zeros of both signs for the tie rule
             a[:min(count, 8)] = [(0.0, -0.0)[(r + i) % 2] for i in range(min(count, 8))]
+        for i in range(8, min(count, 8 + 3 * n)):     # one NaN per position, on a rank that moves along the ring:
+            sends[i % n][i] = np.nan                  # which operands survive it depends on where it enters the chain
     for op in (N.OP_SUM, N.OP_MAX, N.OP_MIN):
         want = O.bootstrap_allreduce(sends, dtype, op)[0]
         for inplace in (False, True):
@@ -447,14 +449,34 @@ def test_host_order_matches_the_reference_host_ring(dev, stream, dname, n, count
     ln = (C.c_size_t * n)(*[rc * es] * n)
     outs = [np.empty(rc, npdt) for _ in range(n)]
     vp = lambda arrs: (C.c_void_p * n)(*[a.ctypes.data for a in arrs])
-    assert O.lib.oracle_bootstrap_reduce_scatter(vp(outs), vp(part), n, off, ln, dtype, N.OP_SUM) == 0
-    with DevBufs(dev) as b, S.SimGroup(n, order=3) as g:
-        ds = [b.put(a) for a in part]
-        dr = [b.alloc(rc * es) for _ in range(n)]
-        N.check(g.reduce_scatter(ds, dr, rc, dtype, N.OP_SUM, stream))
-        dev.stream_sync(stream)
-        for r in range(n):
-            assert_parity(dev.to_host(dr[r], rc, npdt), outs[r], dtype, N.OP_SUM, f"host order reduce-scatter rank {r}")
+    for op in (N.OP_SUM, N.OP_MIN):
+        assert O.lib.oracle_bootstrap_reduce_scatter(vp(outs), vp(part), n, off, ln, dtype, op) == 0
+        with DevBufs(dev) as b, S.SimGroup(n, order=3) as g:
+            ds = [b.put(a) for a in part]
+            dr = [b.alloc(rc * es) for _ in range(n)]
+            N.check(g.reduce_scatter(ds, dr, rc, dtype, op, stream))
+            dev.stream_sync(stream)
+            for r in range(n):
+                assert_parity(dev.to_host(dr[r], rc, npdt), outs[r], dtype, op, f"host order reduce-scatter rank {r}")
+
+
+@pytest.mark.parametrize("dname", ["bf16", "fp16"])
+def test_host_order_max_min_of_16_bit_floats_with_nan(dev, stream, dname):
+    """max / min select an input's bits, so the host ring's step-by-step result is
+    defined for the 16-bit types too (their sums are not comparable: the ring would
+    round at every hop).  NaNs enter the chain at every position."""
+    dtype, n, count = DTYPES[dname], 5, 30011
+    sends = seeded_inputs(dtype, n, count, seed=17)
+    nan = 0x7fc0 if dname == "bf16" else 0x7e00
+    for i in range(4 * n):
+        sends[i % n][i] = nan
+        sends[(i + 2) % n][i + 100] = nan ^ 0x8000          # negative NaN, two ranks further on
+    for op in (N.OP_MAX, N.OP_MIN):
+        want = O.bootstrap_allreduce(sends, dtype, op)[0]
+        for inplace in (False, True):
+            got = _allreduce(dev, stream, sends, dtype, op, inplace=inplace, order=3)
+            for r in range(n):
+                assert np.array_equal(got[r], want), f"{dname} op={op} rank {r} inplace={inplace}"
 
 
 def test_single_rank_and_empty_collectives(dev, stream):

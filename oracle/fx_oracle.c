@@ -38,7 +38,8 @@
  *   oracle_bootstrap_* (the host ring) ........ chunk table against the quoted
  *       formula's literal cases; association and operand order derived by hand
  *       from the reference loop for n = 3 and 4 on values where every other
- *       association / tie rule gives a different answer; closed forms.
+ *       association / tie rule gives a different answer, and on NaN operands,
+ *       which show which argument of each step is the local one; closed forms.
  *   oracle_pack / oracle_unpack ............... round-trip identity and the
  *       displacement arithmetic of service/bootstrap.cc:1253-1258.
  *   trigger encode/decode ..................... bit constants of

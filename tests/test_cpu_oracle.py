@@ -337,6 +337,25 @@ def test_bootstrap_ring_association_derived_by_hand():
         got = O.bootstrap_allreduce(sends, F32, op)[0]
         want = np.concatenate([sends[c][2 * c:2 * c + 2] for c in range(n)])          # chunk c = elements 2c, 2c+1
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), op
+    # A NaN pins the operand order of each step: std::max(local, received) is (local < received) ? received : local,
+    # false whenever either is NaN, so it returns LOCAL.  n = 4, one element per chunk; chunk c travels c+1, c+2, c+3, c.
+    # NaN on the second rank of the chain: that rank keeps its NaN, the next rank keeps its own value over the NaN,
+    # and the first rank's value -- however large -- is never seen again.
+    nan, big = f(np.nan), f(1e30)
+    sends = [np.zeros(4, f) for _ in range(4)]
+    for c in range(4):
+        sends[(c + 1) % 4][c] = big            # first on the chain: lost behind the NaN
+        sends[(c + 2) % 4][c] = nan            # second: max(NaN, big) = NaN
+        sends[(c + 3) % 4][c] = f(2.0)         # third: max(2, NaN) = 2
+        sends[c][c] = f(1.0)                   # last: max(1, 2) = 2
+    got = O.bootstrap_allreduce(sends, F32, MAX)[0]
+    assert np.array_equal(got, np.full(4, 2.0, f))
+    got = O.bootstrap_allreduce(sends, F32, MIN)[0]          # min(2, NaN) = 2, min(1, 2) = 1
+    assert np.array_equal(got, np.full(4, 1.0, f))
+    for c in range(4):                                        # NaN on the LAST rank of the chain is the result
+        sends[(c + 2) % 4][c], sends[c][c] = f(3.0), nan
+    got = O.bootstrap_allreduce(sends, F32, MAX)[0]
+    assert np.isnan(got).all()
     # closed form of the reference's collective tests holds on this path too
     i = np.arange(1001)
     sends = [(r * 1000 + i % 10).astype(f) for r in range(8)]

@@ -145,8 +145,8 @@ def cpu_baseline(ins, threads_all):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--synthetic-fill", choices=["seeded", "memset"], default="seeded",
                     help="memset skips host generation (profiling runs)")

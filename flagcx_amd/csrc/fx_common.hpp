@@ -53,9 +53,14 @@ inline int guarded(F body) noexcept {
 }
 
 // 128-bit streaming accesses: every byte is touched once, so keep it out of
-// the caches' way (nontemporal).
+// the caches' way (nontemporal).  Loads may start at any byte: gfx950 under HSA
+// serves global loads of every width at unaligned addresses (the compiler itself
+// emits one 128-bit load for an under-aligned pointer), so an input that is only
+// element-aligned relative to the output's 16-byte grid costs no extra
+// instructions.  Stores are always whole aligned vectors.
+typedef u32x4 u32x4_anywhere __attribute__((aligned(1)));
 __device__ __forceinline__ u32x4 ldg_stream(const void *p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4_anywhere *>(p));
 }
 __device__ __forceinline__ void stg_stream(void *p, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));

@@ -22,9 +22,9 @@
 // flight per input, all K*U loads issued before the first use.  The index
 // space is anchored at the output pointer rounded down to 16 bytes, so stores
 // are always whole aligned vectors except in the first and last vector of a
-// segment, which fall back to element accesses.  Inputs that share the
-// output's misalignment take the vector-load path; others are gathered
-// element by element (coalesced across lanes, still one pass).  Large
+// segment, which fall back to element accesses.  An input need not share the
+// output's misalignment: its vectors are fetched with 128-bit loads that start
+// wherever the matching elements start (see ldg_stream).  Large
 // segments are handed to workgroups as 512-byte pieces 32 KiB apart (see
 // TilePlan) instead of contiguous 16 KiB runs.
 #pragma once
@@ -389,7 +389,10 @@ struct CopyRed {
 // write stream mixed into reads is expensive (measured: 5.9 TB/s for 8 inputs).
 // The same bytes moved as 512-byte pieces 32 KiB apart reach 6.4-6.5 TB/s.  So
 // the part of a segment that consists of whole regions of kStripeTiles tiles,
-// aligned in ABSOLUTE address, is handed out striped: tile i of a region owns
+// aligned in ABSOLUTE address, is handed out striped when every input shares
+// the output's alignment within 16 bytes (an input that does not would have a
+// cache line straddle every 512-byte piece, fetched by two workgroups; measured,
+// such segments do better contiguous: 6.1-6.5 against 5.5-6.0 TB/s): tile i of a region owns
 // piece i of every 32 KiB row of that region.  The rest (head before the first
 // region boundary, tail after the last) is handed out contiguously.
 constexpr uint32_t kPieceVecs = 32;                           // 512 bytes
@@ -437,7 +440,6 @@ struct Seg {
   const char *in[K];
   char *out;
   uint64_t lead, end;
-  bool coAligned;   // every input is 16-byte aligned like out
   __device__ __forceinline__ const char *inp(int p) const { return in[p]; }
   __device__ __forceinline__ int inputs() const { return K; }
 };
@@ -451,7 +453,6 @@ struct Seg<0> {
   char *out;
   uint64_t lead, end;
   int k;
-  bool coAligned;
   __device__ __forceinline__ const char *inp(int p) const { return (const char *)raw[p] - mis; }
   __device__ __forceinline__ int inputs() const { return k; }
 };
@@ -532,28 +533,6 @@ __device__ __forceinline__ void storeElems(const SegB<K> &sg, uint64_t e0, int l
     if (o < sg.nmore) scatterElems<ES>(sg.more[o], e0, lo, hi, v);
 }
 
-// A whole 16-byte vector from an address that is only element-aligned: aligned
-// dword loads plus a funnel shift.  The dword holding the first (last) byte may
-// start before (end after) the vector, but never leaves the 4-byte word that
-// holds valid data, so it cannot touch an unmapped page.
-template <int ES>
-__device__ __forceinline__ u32x4 loadVectorUnaligned(const char *p) {
-  const uint32_t sh = (uint32_t)(uintptr_t)p & 3u;  // 0 when ES == 4
-  const uint32_t *q = reinterpret_cast<const uint32_t *>(p - sh);
-  u32x4 r;
-  if (ES == 4 || sh == 0) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = __builtin_nontemporal_load(q + i);
-  } else {
-    uint32_t d[5];
-#pragma unroll
-    for (int i = 0; i < 5; i++) d[i] = __builtin_nontemporal_load(q + i);
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], sh);
-  }
-  return r;
-}
-
 // Reduce vector j of the segment with full bounds / alignment handling.
 template <class R, int K, class SG>
 __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
@@ -567,7 +546,7 @@ __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
   const int k = sg.inputs();
   auto fetch = [&](int p) -> u32x4 {
     if (!full) return gatherElems<R::ES>(sg.inp(p), e0, lo, hi);
-    return sg.coAligned ? ldg_stream(sg.inp(p) + j * 16) : loadVectorUnaligned<R::ES>(sg.inp(p) + j * 16);
+    return ldg_stream(sg.inp(p) + j * 16);
   };
   R::init(acc, fetch(0));
   for (int p = 1; p < k; p++) R::fold(acc, fetch(p));
@@ -615,16 +594,15 @@ __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, ui
 
 // Which vectors lane `tid` of the workgroup that owns tile `tile` handles:
 // j, j + stride, .., U of them.  `fast` (the same for the whole workgroup) says
-// that all U * kBlock vectors of the tile are whole, inside the segment and
-// loadable with aligned vector loads; otherwise every vector below `limit` goes
-// through the checked path.  Shared by the kernels and by the host-side check of
+// that all U * kBlock vectors of the tile are whole and inside the segment;
+// otherwise every vector below `limit` goes through the checked path.  Shared by the kernels and by the host-side check of
 // this index arithmetic.
 struct TileLane {
   uint64_t j, stride, limit;
   bool fast;
 };
 
-__host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile, uint32_t tid, int U, bool coAligned) {
+__host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile, uint32_t tid, int U) {
   const uint64_t V = (uint64_t)U * kBlock;
   TileLane tl;
   if (tile < tp.zoneTiles) {
@@ -650,14 +628,14 @@ __host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile
   const uint64_t fastEnd = (tl.limit < tp.endFull) ? tl.limit : tp.endFull;
   tl.j = j0 + tid;
   tl.stride = kBlock;
-  tl.fast = coAligned && j0 >= tp.firstFull && j0 + V <= fastEnd;
+  tl.fast = j0 >= tp.firstFull && j0 + V <= fastEnd;
   return tl;
 }
 
 // Tile `tile` of the segment: striped zone first, then head, then tail.
 template <class R, int K, int U, class SG>
 __device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uint32_t tile) {
-  const TileLane tl = laneOfTile(tp, tile, threadIdx.x, U, sg.coAligned);
+  const TileLane tl = laneOfTile(tp, tile, threadIdx.x, U);
   if (tl.fast) {
     reduceVectorsFast<R, K, U>(sg, tl.j * 16, tl.stride * 16);
   } else {
@@ -682,7 +660,6 @@ __device__ __forceinline__ TilePlan makeSeg(Seg<K> &sg, const void *const *in, v
     co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
     sg.in[p] = (const char *)in[p] - mis;
   }
-  sg.coAligned = co;
   return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
 }
 
@@ -697,7 +674,6 @@ __device__ __forceinline__ TilePlan makeSeg(Seg<0> &sg, const void *const *in, v
   sg.k = k;
   bool co = true;
   for (int p = 0; p < k; p++) co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
-  sg.coAligned = co;
   return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
 }
 

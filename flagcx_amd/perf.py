@@ -244,7 +244,7 @@ def main(argv=None):
     ap.add_argument("-f", "--factor", type=int, default=2)
     ap.add_argument("--inplace", action="store_true")
     ap.add_argument("--misalign", type=int, default=0, help="shift buffers by this many elements")
-    ap.add_argument("--mixed", action="store_true", help="shift only every other input (gather path)")
+    ap.add_argument("--mixed", action="store_true", help="shift only every other input (inputs not aligned like the output)")
     ap.add_argument("--in-shift", type=int, default=0,
                     help="start input i at byte offset i*IN_SHIFT of its allocation (multiple of 16 keeps vector loads)")
     a = ap.parse_args(argv)

@@ -21,13 +21,13 @@ static long checkOne(uint64_t outAddr, uint64_t count, int es, int U, bool co) {
   for (uint64_t tile = 0; tile < tiles; tile++) {
     bool fast0 = false;
     for (uint32_t tid = 0; tid < (uint32_t)kBlock; tid++) {
-      const TileLane tl = laneOfTile(tp, (uint32_t)tile, tid, U, co);
+      const TileLane tl = laneOfTile(tp, (uint32_t)tile, tid, U);
       if (tid == 0) fast0 = tl.fast;
       if (tl.fast != fast0) return 2;                       // the path must be uniform in a workgroup
       for (int u = 0; u < U; u++) {
         const uint64_t j = tl.j + (uint64_t)u * tl.stride;
         if (tl.fast) {
-          if (!co) return 3;                                  // vector loads need co-aligned inputs
+          if (!co && tile < tp.zoneTiles) return 3;           // striped tiles only for co-aligned inputs
           if (j < tp.firstFull || j >= tp.endFull) return 4;  // whole vectors inside the segment only
           if (seen[j]++) return 5;
         } else {

@@ -87,7 +87,7 @@ def test_rotated_order(dev, dname):
 @pytest.mark.parametrize("dname", list(DTYPES))
 def test_unaligned_buffers(dev, dname):
     """Output / inputs at element offsets that are not 16-byte aligned, both
-    all-equal (vector path with a peeled head) and mixed (gather path)."""
+    all-equal (a peeled head, then aligned vectors) and mixed (unaligned vector loads)."""
     dtype = DTYPES[dname]
     es = N.DTYPE_SIZE[dtype]
     k = 3
@@ -119,7 +119,7 @@ def test_striped_zone_boundaries(dev, dname):
             assert_parity(got, want, dtype, N.OP_SUM, f"zone {dname} n={n} off={off_el} k={k}")
             got = run_reduce(dev, ins, dtype, N.OP_SUM, offs=offs, inplace=True)
             assert_parity(got, want, dtype, N.OP_SUM, f"zone in-place {dname} n={n} off={off_el} k={k}")
-    # inputs NOT co-aligned with the output: no zone, gather path over a long segment
+    # inputs NOT co-aligned with the output: no zone, unaligned vector loads over a long segment
     n = 3 * mib + 9
     ins = seeded_inputs(dtype, 3, n, seed=4)
     got = run_reduce(dev, ins, dtype, N.OP_MAX, offs=[0, es, 0, 3 * es])

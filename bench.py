@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the same counter's reading for a
 # plain copy of known size; numbers and commands in
 # profiles/reduceCopyDirect_bf16_sum_k8_512MiB.txt.
-MEASURED_TRAFFIC_BYTES = 4_831_515_000
+MEASURED_TRAFFIC_BYTES = 4_831_503_000
 K_INPUTS = 8
 ELEMS = 268_435_456            # per input: 512 MiB of bf16
 SEED = 4                       # values N(0, 0.02)

@@ -86,8 +86,8 @@ template <int DT, int OP>
 __device__ __forceinline__ void runShare(const void *in1, const void *in2, void *out, uint64_t count, Share sh) {
   using R = Red<DT, OP>;
   const void *in[2] = {in1, in2};
-  Seg<2> sg;
-  const TilePlan tp = makeSeg<R::ES, kFifoU>(sg, in, out, count, 2);
+  SegWT<2> sg;  // written through: see the count-in below
+  const TilePlan tp = makeSeg<R::ES, kFifoU>(static_cast<Seg<2> &>(sg), in, out, count, 2);
   const uint64_t tiles = tp.tiles();
   for (uint64_t t = sh.idx; t < tiles; t += sh.takers) reduceTile<R, 2, kFifoU>(sg, tp, (uint32_t)t);
 }
@@ -282,8 +282,10 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       }
       break;
     }
-    const void *in1 = (const void *)(uintptr_t)sh[1], *in2 = (const void *)(uintptr_t)sh[2];
-    void *out = (void *)(uintptr_t)sh[3];
+    // the trigger's addresses are device (global) memory: say so, or every access below is a flat one
+    typedef __attribute__((address_space(1))) char GlobalByte;
+    const void *in1 = (const void *)(GlobalByte *)(uintptr_t)sh[1], *in2 = (const void *)(GlobalByte *)(uintptr_t)sh[2];
+    void *out = (void *)(GlobalByte *)(uintptr_t)sh[3];
     const uint64_t w3 = sh[4];
     const uint64_t count = w3 & 0xffffffffull;
     const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
@@ -294,8 +296,13 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       continue;
     }
     // The trigger's buffers may have been written by other agents since this
-    // kernel last looked: drop stale cache lines before reading them.
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    // kernel last looked: drop stale cache lines before reading them.  The caches
+    // are the compute unit's and the die's, not a wavefront's, so one wavefront
+    // invalidates for the whole workgroup and the barrier orders the others'
+    // loads behind it (four invalidates per workgroup cost 5 us more per large
+    // trigger than one).
+    if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    __syncthreads();
     bool ok = true;
     if (count) {
       switch (dtype) {
@@ -312,13 +319,19 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
         default: ok = false;
       }
     }
+    // Every wavefront waits until its own stores are acknowledged (s_waitcnt
+    // vmcnt(0); a workgroup barrier alone does not make a wavefront wait for
+    // its vector stores), then the barrier collects the four of them.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt left alone
     __syncthreads();
     if (threadIdx.x == 0) {
       const uint32_t slot = (uint32_t)(seq % cap);
-      // Release: with the barrier above, this workgroup's stores are out before
-      // it reports in.  Only the last one in pays for the acquire that puts
-      // everybody's stores behind it (an L2 invalidate per workgroup otherwise).
-      const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      // The results were stored through the caches (SegWT) and every wavefront
+      // waited for its stores before the barrier above, so they are in memory
+      // before this workgroup reports in: no cache write-back here (one per
+      // workgroup and trigger cost 7 us on a 16 MiB trigger).  Only the last one in pays
+      // for the acquire that puts everybody's count-ins behind it.
+      const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (prev == share.takers - 1) {  // last one out completes the trigger
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         __hip_atomic_store(&m->done[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

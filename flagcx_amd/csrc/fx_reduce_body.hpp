@@ -525,6 +525,51 @@ template <int ES, int K>
 __device__ __forceinline__ void storeElems(const Seg<K> &sg, uint64_t e0, int lo, int hi, u32x4 v) {
   scatterElems<ES>(sg.out, e0, lo, hi, v);
 }
+
+// Segment whose results are written THROUGH the caches (system-scope stores):
+// nothing of it stays dirty in a die's L2, so a kernel that must publish its
+// results to other agents while it keeps running (the FIFO consumer) needs no
+// cache write-back afterwards, only to wait for its stores.
+template <int K>
+struct SegWT : Seg<K> {};
+
+template <class T>
+__device__ __forceinline__ void storeThrough(void *p, T v) {
+  __hip_atomic_store(reinterpret_cast<T *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+// A whole vector: one 128-bit buffer store carrying the system-scope and
+// streaming cache-policy bits (two 64-bit atomic stores reach only 3.7 TB/s on
+// a large segment).  The buffer descriptor is based at the first active lane's
+// address; lane addresses only grow with the lane number in every tiling used
+// here, so the 32-bit offsets are small and non-negative.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+template <int K>
+__device__ __forceinline__ void storeVector(const SegWT<K> &sg, uint64_t byteOff, u32x4 v) {
+  const uint64_t a = (uint64_t)(uintptr_t)(sg.out + byteOff);
+  const uint64_t base = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
+  __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)base, 0, 0x7fffffff, 0x00020000);
+  constexpr int kSc0 = 1, kNt = 2, kSc1 = 16;
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)(uint32_t)(a - base), 0,
+                                         kSc0 | kSc1 | kNt);
+}
+template <int ES, int K>
+__device__ __forceinline__ void storeElems(const SegWT<K> &sg, uint64_t e0, int lo, int hi, u32x4 v) {
+  constexpr int VE = 16 / ES;
+#pragma unroll
+  for (int s = 0; s < VE; s++) {
+    if (s >= lo && s < hi) {
+      if constexpr (ES == 8)
+        storeThrough<uint64_t>(sg.out + (e0 + s) * 8, (uint64_t)v[2 * s] | ((uint64_t)v[2 * s + 1] << 32));
+      else if constexpr (ES == 4)
+        storeThrough<uint32_t>(sg.out + (e0 + s) * 4, v[s]);
+      else if constexpr (ES == 2)
+        storeThrough<uint16_t>(sg.out + (e0 + s) * 2, (uint16_t)(v[s / 2] >> (16 * (s & 1))));
+      else
+        storeThrough<uint8_t>(sg.out + e0 + s, (uint8_t)(v[s / 4] >> (8 * (s & 3))));
+    }
+  }
+}
 template <int ES, int K>
 __device__ __forceinline__ void storeElems(const SegB<K> &sg, uint64_t e0, int lo, int hi, u32x4 v) {
   scatterElems<ES>(sg.out, e0, lo, hi, v);

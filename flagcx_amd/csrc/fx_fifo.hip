@@ -282,10 +282,8 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       }
       break;
     }
-    // the trigger's addresses are device (global) memory: say so, or every access below is a flat one
-    typedef __attribute__((address_space(1))) char GlobalByte;
-    const void *in1 = (const void *)(GlobalByte *)(uintptr_t)sh[1], *in2 = (const void *)(GlobalByte *)(uintptr_t)sh[2];
-    void *out = (void *)(GlobalByte *)(uintptr_t)sh[3];
+    const void *in1 = (const void *)(uintptr_t)sh[1], *in2 = (const void *)(uintptr_t)sh[2];
+    void *out = (void *)(uintptr_t)sh[3];
     const uint64_t w3 = sh[4];
     const uint64_t count = w3 & 0xffffffffull;
     const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);

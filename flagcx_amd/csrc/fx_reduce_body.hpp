@@ -435,6 +435,16 @@ __host__ __device__ inline TilePlan planTiles(uint64_t outAddr, uint64_t count, 
   return tp;
 }
 
+// Every buffer these kernels touch is device-visible global memory.  Pointers
+// that reach a kernel through a table in memory or through LDS carry no address
+// space, and the compiler would then use flat instructions for them; passing
+// them through the global address space once lets it pick global ones.
+typedef __attribute__((address_space(1))) char GlobalByte;
+__device__ __forceinline__ const char *asGlobal(const void *p) {
+  return (const char *)(const GlobalByte *)(uintptr_t)p;
+}
+__device__ __forceinline__ char *asGlobal(void *p) { return (char *)(GlobalByte *)(uintptr_t)p; }
+
 template <int K>
 struct Seg {
   const char *in[K];
@@ -453,7 +463,7 @@ struct Seg<0> {
   char *out;
   uint64_t lead, end;
   int k;
-  __device__ __forceinline__ const char *inp(int p) const { return (const char *)raw[p] - mis; }
+  __device__ __forceinline__ const char *inp(int p) const { return asGlobal(raw[p]) - mis; }
   __device__ __forceinline__ int inputs() const { return k; }
 };
 
@@ -696,14 +706,14 @@ __device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uin
 template <int ES, int U, int K>
 __device__ __forceinline__ TilePlan makeSeg(Seg<K> &sg, const void *const *in, void *out, uint64_t count, int) {
   const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
-  sg.out = (char *)out - mis;
+  sg.out = asGlobal(out) - mis;
   sg.lead = mis / ES;
   sg.end = sg.lead + count;
   bool co = true;
 #pragma unroll
   for (int p = 0; p < K; p++) {
     co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
-    sg.in[p] = (const char *)in[p] - mis;
+    sg.in[p] = asGlobal(in[p]) - mis;
   }
   return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
 }
@@ -713,7 +723,7 @@ __device__ __forceinline__ TilePlan makeSeg(Seg<0> &sg, const void *const *in, v
   const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
   sg.raw = in;
   sg.mis = mis;
-  sg.out = (char *)out - mis;
+  sg.out = asGlobal(out) - mis;
   sg.lead = mis / ES;
   sg.end = sg.lead + count;
   sg.k = k;
@@ -835,7 +845,7 @@ __global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable t) 
   const uint64_t mis = (uint64_t)(uintptr_t)d.out[0] & 15u;
   sg.nmore = (int)d.nout - 1;
 #pragma unroll
-  for (int o = 0; o < kMaxFixedK - 1; o++) sg.more[o] = (o < sg.nmore) ? (char *)d.out[o + 1] - mis : nullptr;
+  for (int o = 0; o < kMaxFixedK - 1; o++) sg.more[o] = (o < sg.nmore) ? asGlobal(d.out[o + 1]) - mis : nullptr;
   reduceTile<R, K, U>(sg, tp, b - t.tileStart[i]);
 }
 

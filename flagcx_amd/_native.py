@@ -80,6 +80,7 @@ _SIGS = {
     "fx_fifo_poll_state": (_i, [_vp, _i]),
     "fx_fifo_set_state": (_i, [_vp, _i, _i]),
     "fx_fifo_terminate": (_i, [_vp]),
+    "fx_fifo_run_batch": (_i, [_vp, _vp, _sz, C.c_ulonglong]),
     "fx_fifo_consumer_create": (_i, [C.POINTER(_vp), _sz]),
     "fx_fifo_consumer_launch": (_i, [_vp, _vp, _vp, C.c_ulonglong, _vp]),
     "fx_fifo_consumer_status": (_i, [_vp, C.POINTER(_i), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),

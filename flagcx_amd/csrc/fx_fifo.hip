@@ -17,7 +17,9 @@
 // trigger, taking tiles idx, idx + takers, ... -- and the last workgroup to
 // finish marks it Complete.  Workgroup 0 does no arithmetic: it alone reads the
 // pinned host ring (over PCIe) and mirrors it into device memory, where the
-// other workgroups poll it.  Nothing waits on another
+// other workgroups poll it and read up to kBatch upcoming triggers per round
+// of reads.  Results are stored through the caches, so reporting in needs no
+// cache write-back.  Nothing waits on another
 // workgroup, so the kernel cannot deadlock on residency; every polling loop is
 // bounded by maxIdlePolls.  Triggers that are in the ring at the same time must
 // be independent of each other, which is how the reference's scheduler uses it
@@ -37,6 +39,7 @@ using namespace fx;
 namespace {
 
 constexpr int kFifoU = 4;
+constexpr int kBatch = 16;  // triggers a workgroup inspects per round of mirror reads
 constexpr uint32_t kMaxCapacity = 1024;
 
 struct FifoMirror {              // device memory, zeroed at creation
@@ -149,7 +152,9 @@ __global__ void __launch_bounds__(kBlock) clearMirror(uint64_t *words, uint32_t 
 
 __global__ void __launch_bounds__(kBlock)
 fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uint64_t maxIdlePolls) {
-  __shared__ uint64_t sh[6];  // [0] state, [1..4] trigger words, [5] words valid
+  __shared__ uint64_t sh[2];                  // [0] state, [1] triggers in this batch
+  __shared__ uint64_t shTrig[kBatch][4];     // their words
+  __shared__ uint32_t shValid[kBatch];       // and whether the words are theirs (sequence lock)
   enum { kWork = 0, kExitTerminate = FX_FIFO_EXIT_TERMINATE, kExitIdle = FX_FIFO_EXIT_IDLE };
   uint64_t seq = startSeq;
   uint64_t *hostTrig = host + 4;
@@ -164,10 +169,10 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       // Wavefront 0 does the polling.  Reads over PCIe cost microseconds each, so
       // they are issued by different lanes of one instruction and the results are
       // broadcast; every branch below depends on broadcast values only.
-      uint64_t idle = 0, state;
+      uint64_t idle = 0, state, p = 0;  // p: triggers published so far, as last polled
       bool termSeen = false;
       for (;;) {
-        uint64_t p, term;
+        uint64_t term;
         if (blockIdx.x == 0) {
           if (mirrored <= seq) {  // nothing mirrored is waiting for this workgroup: talk to the host
             uint64_t v = 0;
@@ -199,6 +204,7 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
               __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // every lane's copies before the new count
               mirrored = hp;
               if (lane == 0) __hip_atomic_store(&m->produced, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              idle = 0;  // the host is alive
             }
             // The host sets terminate after its last enqueue, but two relaxed
             // polls may be served out of order: act on terminate only on the poll
@@ -213,11 +219,16 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
             if (c != lastPublished) {
               if (lane == 0) storeSys(host + 1, startSeq + c);  // consumed
               lastPublished = c;
+              idle = 0;  // so are the workers
             }
           }
           uint64_t t = 0;
           if (lane == 0) t = pollDev(&m->terminate);
           term = fromLane(t, 0);
+          // With workers in the grid this workgroup never takes a tile, so it does
+          // not look at the triggers it has mirrored at all (three dependent reads
+          // each): it goes straight back to the host.
+          if (gridDim.x > 1) seq = mirrored;
           p = mirrored;
         } else {
           uint64_t t = 0, q = 0;
@@ -245,25 +256,35 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
         }
         __builtin_amdgcn_s_sleep(32);
       }
-      if (lane == 0) {
-        sh[0] = state;
-        if (state == kWork) {
-          // Reader side of the sequence lock.  If the slot still carries number
-          // seq after the words were read, they are trigger seq's.  If not, the
-          // ring has come round: trigger seq is complete, which it could not be
-          // had this workgroup been one of its workers -- so there is nothing to do.
-          // (agent-scope atomic loads read the coherent cache level; the
-          // workgroup-scope fences make each step's loads return before the next
-          // step's are issued, without invalidating anything.)
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-          const uint32_t slot = (uint32_t)(seq % cap);
-          const uint64_t before = pollDev(&m->trigSeq[slot]);
-          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
-          for (int w = 0; w < 4; w++) sh[1 + w] = pollDev(&m->trig[slot][w]);
-          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
-          const uint64_t after = pollDev(&m->trigSeq[slot]);
-          sh[5] = (before == seq && after == seq) ? 1 : 0;
+      if (lane == 0) sh[0] = state;
+      if (state == kWork) {
+        // Reader side of the sequence lock, for up to kBatch triggers at once (lane
+        // i looks at trigger seq + i): three dependent rounds of reads serve the
+        // whole batch instead of one trigger.  If a slot still carries the expected
+        // number after its words were read, they are that trigger's.  If not, the
+        // ring has come round: the trigger is complete, which it could not be had
+        // this workgroup been one of its workers -- so there is nothing to do.
+        // (agent-scope atomic loads read the coherent cache level; the
+        // workgroup-scope fences make each step's loads return before the next
+        // step's are issued, without invalidating anything.)
+        const uint64_t ahead = p - seq;
+        const uint32_t batch = (uint32_t)(ahead < (uint64_t)kBatch ? ahead : (uint64_t)kBatch);
+        const bool mine = lane < batch;
+        const uint64_t want = seq + lane;
+        const uint32_t slot = (uint32_t)(want % cap);
+        uint64_t before = kNoTrigger, after = kNoTrigger, w[4] = {0, 0, 0, 0};
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (mine) before = pollDev(&m->trigSeq[slot]);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+        if (mine)
+          for (int q = 0; q < 4; q++) w[q] = pollDev(&m->trig[slot][q]);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+        if (mine) after = pollDev(&m->trigSeq[slot]);
+        if (mine) {
+          for (int q = 0; q < 4; q++) shTrig[lane][q] = w[q];
+          shValid[lane] = (before == want && after == want) ? 1u : 0u;
         }
+        if (lane == 0) sh[1] = batch;
       }
     }
     __syncthreads();
@@ -282,17 +303,15 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       }
       break;
     }
-    const void *in1 = (const void *)(uintptr_t)sh[1], *in2 = (const void *)(uintptr_t)sh[2];
-    void *out = (void *)(uintptr_t)sh[3];
-    const uint64_t w3 = sh[4];
+    const uint32_t batch = (uint32_t)sh[1];
+    for (uint32_t bi = 0; bi < batch; bi++, seq++) {
+    const void *in1 = (const void *)(uintptr_t)shTrig[bi][0], *in2 = (const void *)(uintptr_t)shTrig[bi][1];
+    void *out = (void *)(uintptr_t)shTrig[bi][2];
+    const uint64_t w3 = shTrig[bi][3];
     const uint64_t count = w3 & 0xffffffffull;
     const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
     const Share share = shareOf(seq, in1, in2, out, count, dtype, op);
-    if (sh[5] == 0 || share.idx >= share.takers) {  // overtaken by the ring, or not needed for this trigger
-      seq++;
-      __syncthreads();
-      continue;
-    }
+    if (shValid[bi] == 0 || share.idx >= share.takers) continue;  // overtaken by the ring, or not needed for this trigger
     // The trigger's buffers may have been written by other agents since this
     // kernel last looked: drop stale cache lines before reading them.  The caches
     // are the compute unit's and the die's, not a wavefront's, so one wavefront
@@ -339,8 +358,8 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
         __hip_atomic_fetch_add(&m->completed, 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    seq++;
-    __syncthreads();
+    }  // batch
+    __syncthreads();  // the batch arrays are rewritten next
   }
 }
 
@@ -411,6 +430,40 @@ int fx_fifo_set_state(uint64_t *fifo, int idx, int state) {
 int fx_fifo_terminate(uint64_t *fifo) {
   if (!fifo) return flagcxInvalidArgument;
   __atomic_store_n(&fifo[3], 1ull, __ATOMIC_RELEASE);
+  return flagcxSuccess;
+}
+
+int fx_fifo_run_batch(uint64_t *fifo, const fxReduceTrigger *triggers, size_t n, unsigned long long spinLimit) {
+  if (!fifo || (n && !triggers) || spinLimit == 0) return flagcxInvalidArgument;
+  const uint64_t cap = fifo[0];
+  if (cap == 0 || cap > kMaxCapacity) return flagcxInvalidArgument;
+  // Slots are handed out in ring order and collected in the same order, so the
+  // in-flight ones are a window [collected, issued) of the batch.
+  int slotOf[kMaxCapacity];
+  size_t issued = 0, collected = 0;
+  unsigned long long idle = 0;
+  while (collected < n) {
+    bool progress = false;
+    if (issued < n && issued - collected < cap) {
+      uint64_t in1, in2, out, count, nthreads;
+      int dtype, op, idx = -1;
+      fx_trigger_get(&triggers[issued], &in1, &in2, &out, &count, &nthreads, &dtype, &op, nullptr);
+      int rc = fx_fifo_enqueue(fifo, in1, in2, out, count, nthreads, dtype, op, &idx);
+      if (rc != flagcxSuccess) return rc;
+      if (idx >= 0) {
+        slotOf[issued % cap] = idx;
+        issued++;
+        progress = true;
+      }
+    }
+    while (collected < issued && fx_fifo_poll_state(fifo, slotOf[collected % cap]) == fxTriggerComplete) {
+      fx_fifo_set_state(fifo, slotOf[collected % cap], fxTriggerAvailable);
+      collected++;
+      progress = true;
+    }
+    if (progress) idle = 0;
+    else if (++idle > spinLimit) return flagcxInternalError;
+  }
   return flagcxSuccess;
 }
 

@@ -186,24 +186,21 @@ def run_fifo(dev, a):
                 one(n)
             ms = (time.perf_counter() - t0) * 1e3 / 20
             row("fifo round trip, fp32 sum, 2 inputs", nbytes, ms, 3 * nbytes)
-            # the ring kept full: 256 independent triggers, collected as they complete
+            # the ring kept full: 1024 independent triggers through the library's own producer loop
+            # (enqueue as slots free up, collect as they complete)
             if 3 * nbytes * 64 <= emax * 3:
                 span = emax // (64 * 4) * 4                      # 64 disjoint windows of the buffers
                 n = min(n, span // 4)
-                pending, done, t0 = [], 0, time.perf_counter()
-                issued = 0
-                while done < 256:
-                    if issued < 256:
-                        off = (issued % 64) * span
-                        lib.fx_fifo_enqueue(host, bufs[0] + off, bufs[1] + off, bufs[2] + off, n, 32, N.DT_FP32,
-                                            N.OP_SUM, C.byref(idx))
-                        if idx.value >= 0:
-                            pending.append(idx.value)
-                            issued += 1
-                    if pending and lib.fx_fifo_poll_state(host, pending[0]) == 3:
-                        lib.fx_fifo_set_state(host, pending.pop(0), 0)
-                        done += 1
-                ms = (time.perf_counter() - t0) * 1e3 / 256
+                total = 1024
+                trig = (N.ReduceTrigger * total)()
+                for i in range(total):
+                    off = (i % 64) * span
+                    lib.fx_trigger_set(C.byref(trig[i]), bufs[0] + off, bufs[1] + off, bufs[2] + off, n, 32, N.DT_FP32,
+                                       N.OP_SUM, 1)
+                N.check(lib.fx_fifo_run_batch(host, trig, 64, 50_000_000))          # warm-up
+                t0 = time.perf_counter()
+                N.check(lib.fx_fifo_run_batch(host, trig, total, 50_000_000))
+                ms = (time.perf_counter() - t0) * 1e3 / total
                 row("fifo ring kept full, per trigger", n * 4, ms, 3 * n * 4)
             nbytes *= a.factor
     finally:

@@ -101,6 +101,17 @@ int fx_fifo_enqueue(uint64_t *fifo, uint64_t in1, uint64_t in2, uint64_t out,
 int fx_fifo_poll_state(const uint64_t *fifo, int idx);
 int fx_fifo_set_state(uint64_t *fifo, int idx, int state);
 int fx_fifo_terminate(uint64_t *fifo);
+/*
+ * The producer loop of the reference's scheduler for a set of independent
+ * triggers (processReadyQueue + processInflightQueue,
+ * flagcx/runner/uni_runner_impl.cc:1701-1794): enqueue all n, as slots free up,
+ * poll each for Complete and hand its slot back (state Available).  Returns when
+ * all n are complete, or flagcxInternalError after spinLimit consecutive polls
+ * without progress (no consumer running).  The state field of the triggers
+ * passed in is ignored.
+ */
+int fx_fifo_run_batch(uint64_t *fifo, const fxReduceTrigger *triggers, size_t n,
+                      unsigned long long spinLimit);
 
 /*
  * FIFO-compatible consumer: the drop-in for flagcxLaunchCollectiveKernel

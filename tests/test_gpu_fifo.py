@@ -222,3 +222,45 @@ def test_second_launch_does_not_repeat_a_trigger_that_was_running_at_terminate(d
         lib.fx_fifo_consumer_destroy(cons)
         dev.stream_destroy(stream)
     dev.free(host, N.MEM_HOST)
+
+
+def test_batch_of_independent_triggers_through_the_producer_loop(dev):
+    """fx_fifo_run_batch: 300 independent triggers of mixed sizes, types and ops
+    through a 16-slot ring (the ring wraps 18 times, many triggers in flight at
+    once, workgroups inspect them in batches); every output against the oracle.
+    With no consumer running the loop gives up instead of spinning for ever."""
+    cap, total = 16, 300
+    ring = Ring(dev, cap)
+    closed = False
+    try:
+        rng = np.random.default_rng(9)
+        kinds = [(N.DT_FP32, N.OP_SUM), (N.DT_BF16, N.OP_MAX), (N.DT_INT32, N.OP_PROD), (N.DT_UINT8, N.OP_MIN),
+                 (N.DT_FP64, N.OP_SUM), (N.DT_FP16, N.OP_AVG)]
+        with DevBufs(dev) as b:
+            trig = (N.ReduceTrigger * total)()
+            cases = []
+            for i in range(total):
+                dtype, op = kinds[i % len(kinds)]
+                n = int(rng.choice([1, 7, 1000, 4096, 70001, 300000]))
+                a, c = seeded_inputs(dtype, 2, n, seed=1000 + i)
+                da, dc, do = b.put(a), b.put(c), b.alloc(n * N.DTYPE_SIZE[dtype])
+                lib.fx_trigger_set(C.byref(trig[i]), da, dc, do, n, 32, dtype, op, ENQUEUED)
+                cases.append((dtype, op, n, a, c, do))
+            N.check(lib.fx_fifo_run_batch(ring.host, trig, total, 200_000_000))
+            assert int(ring.words()[2]) == total                       # produced
+            reason, done, bad = ring.close()                           # before the slow checking: the consumer would idle out
+            closed = True
+            assert (reason, done, bad) == (1, total, 0)
+            for i, (dtype, op, n, a, c, do) in enumerate(cases):
+                assert_parity(dev.to_host(do, n, N.NP_DTYPE[dtype]), O.reduce2(a, c, dtype, op), dtype, op, f"trigger {i}")
+    finally:
+        if not closed:
+            ring.close()
+    # no consumer: nothing ever completes, the producer loop reports it
+    host = dev.malloc(lib.fx_fifo_bytes(4), N.MEM_HOST)
+    N.check(lib.fx_fifo_init(host, 4))
+    one = (N.ReduceTrigger * 1)()
+    lib.fx_trigger_set(C.byref(one[0]), 4096, 8192, 12288, 0, 32, N.DT_FP32, N.OP_SUM, ENQUEUED)
+    assert lib.fx_fifo_run_batch(host, one, 1, 1000) == N.INTERNAL_ERROR
+    assert lib.fx_fifo_run_batch(None, one, 1, 1000) == N.INVALID_ARGUMENT
+    dev.free(host, N.MEM_HOST)

@@ -67,3 +67,47 @@ def test_reduce_entry_points_replay_correctly_in_a_graph(dev):
         hip.hipGraphExecDestroy(gexec)
         hip.hipGraphDestroy(graph)
     dev.stream_destroy(stream)
+
+
+def test_simulated_rank_allreduce_replays_correctly_in_a_graph(dev):
+    """All ranks post on the one captured stream, so the collective is a single
+    kernel node (no events, no scratch): an 8-rank all-reduce and a reduce-scatter
+    captured once, replayed on new data."""
+    from flagcx_amd import sim as S
+    n, count = 8, 8 * 40001
+    dtype = N.DT_FP32
+    stream = dev.stream_create()
+    raw = dev.raw_stream(stream)
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        sends = seeded_inputs(dtype, n, count, seed=3)
+        ds = [b.put(a) for a in sends]
+        dr = [b.alloc(count * 4) for _ in range(n)]
+        dp = [b.alloc(count // n * 4) for _ in range(n)]
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(raw, 0) == 0
+        try:
+            N.check(g.all_reduce(ds, dr, count, dtype, N.OP_SUM, stream))
+            N.check(g.reduce_scatter(ds, dp, count // n, dtype, N.OP_MAX, stream))
+        finally:
+            assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for rep in range(3):
+            if rep:
+                sends = seeded_inputs(dtype, n, count, seed=3 + rep)
+                for d, a in zip(ds, sends):
+                    dev.upload(d, a)
+                for d in dr:
+                    dev.memset(d, 0xEE, count * 4)
+                dev.sync()
+            assert hip.hipGraphLaunch(gexec, raw) == 0
+            dev.stream_sync(stream)
+            want = O.reduce_copy(sends, dtype, N.OP_SUM)
+            wmax = O.reduce_copy(sends, dtype, N.OP_MAX)
+            for r in (0, 3, n - 1):
+                assert_parity(dev.to_host(dr[r], count, np.float32), want, dtype, N.OP_SUM, f"replay {rep} rank {r}")
+                part = count // n
+                assert_parity(dev.to_host(dp[r], part, np.float32), wmax[r * part:(r + 1) * part], dtype, N.OP_MAX,
+                              f"replay {rep} reduce-scatter rank {r}")
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+    dev.stream_destroy(stream)

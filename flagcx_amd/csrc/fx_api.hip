@@ -103,6 +103,9 @@ flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slices
     tiles.push_back((uint32_t)t);
   }
   if (kept == 0) return flagcxSuccess;
+  // A single segment needs no table: the direct kernel's argument block is 100
+  // bytes instead of 4 KiB, which is 1.3 us of an 11 us launch.
+  if (kept == 1) return ks->direct[k](merged[0].out, merged[0].in, k, merged[0].count, s);
   return ks->slicesInline[k](merged.data(), tiles.data(), kept, s);
 }
 

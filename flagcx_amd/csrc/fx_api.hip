@@ -302,15 +302,8 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
       merged.push_back(d);
     }
     std::vector<fxSliceDesc> plainReduce, plainCopy;  // slices whose outputs are not co-aligned
-    InlineBcastTable t;
-    t.n = 0;
-    t.tileStart[0] = 0;
-    auto flush = [&]() -> flagcxResult_t {
-      if (t.n == 0) return flagcxSuccess;
-      flagcxResult_t rc = ks->bcastInline[k](t, s);
-      t.n = 0;
-      return rc;
-    };
+    std::vector<BcastDescDev> dev;
+    std::vector<uint32_t> devTiles;
     for (const fxBcastDesc &d : merged) {
       bool same = true;
       for (int o = 1; o < nout; o++) same = same && (((uintptr_t)d.out[o] & 15u) == ((uintptr_t)d.out[0] & 15u));
@@ -333,19 +326,15 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
       }
       const uint64_t tiles = tilesFor(d.out[0], d.in, k, d.count, es, U);
       if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
-      if (t.n == (uint32_t)kInlineBcast || (uint64_t)t.tileStart[t.n] + tiles > 0x7ffffff0ull) {
-        flagcxResult_t rc = flush();
-        if (rc != flagcxSuccess) return rc;
-      }
-      BcastDescDev &dd = t.d[t.n];
+      BcastDescDev dd;
       for (int p = 0; p < kMaxFixedK; p++) dd.in[p] = (p < k) ? d.in[p] : nullptr;
       for (int o = 0; o < kMaxFixedK; o++) dd.out[o] = (o < nout) ? d.out[o] : nullptr;
       dd.count = d.count;
       dd.nout = (uint32_t)nout;
-      t.tileStart[t.n + 1] = t.tileStart[t.n] + (uint32_t)tiles;
-      t.n++;
+      dev.push_back(dd);
+      devTiles.push_back((uint32_t)tiles);
     }
-    flagcxResult_t rc = flush();
+    flagcxResult_t rc = dev.empty() ? flagcxSuccess : ks->bcastInline[k](dev.data(), devTiles.data(), dev.size(), s);
     if (rc != flagcxSuccess) return rc;
     if (!plainReduce.empty()) {
       rc = launchSliceBatches(ks, plainReduce.data(), plainReduce.size(), k, s);

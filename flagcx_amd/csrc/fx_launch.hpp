@@ -23,7 +23,8 @@ struct KernelSet {
                                                  hipStream_t s);
   flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
                                                 uint32_t grid, hipStream_t s);
-  flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const InlineBcastTable &t, hipStream_t s);
+  // n multi-output slices with their tile counts (all non-zero)
+  flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const BcastDescDev *d, const uint32_t *tiles, size_t n, hipStream_t s);
   int elemSize;
 };
 
@@ -94,12 +95,33 @@ flagcxResult_t launchSlicesTable(const SliceDescDev *d, const uint32_t *tileStar
 }
 
 template <class R, int K>
-flagcxResult_t launchBcastInline(const InlineBcastTable &t, hipStream_t s) {
+flagcxResult_t launchBcastInline(const BcastDescDev *d, const uint32_t *tiles, size_t n, hipStream_t s) {
   constexpr int U = unrollFor(K);
-  uint32_t grid = t.tileStart[t.n];
-  if (grid == 0) return flagcxSuccess;
-  hipLaunchKernelGGL((reduceBcastInline<R, K, U>), dim3(grid), dim3(kBlock), 0, s, t);
-  FX_HIP(hipGetLastError());
+  if (n == 1) {  // the small table
+    InlineBcastTable<1> t;
+    t.d[0] = d[0];
+    t.tileStart[0] = 0;
+    t.tileStart[1] = tiles[0];
+    t.n = 1;
+    hipLaunchKernelGGL((reduceBcastInline<R, K, U, 1>), dim3(tiles[0]), dim3(kBlock), 0, s, t);
+    FX_HIP(hipGetLastError());
+    return flagcxSuccess;
+  }
+  InlineBcastTable<kInlineBcast> t;
+  t.n = 0;
+  t.tileStart[0] = 0;
+  for (size_t i = 0; i <= n; i++) {
+    const bool full = t.n == (uint32_t)kInlineBcast || (i < n && (uint64_t)t.tileStart[t.n] + tiles[i] > 0x7ffffff0ull);
+    if ((i == n || full) && t.n > 0) {
+      hipLaunchKernelGGL((reduceBcastInline<R, K, U, kInlineBcast>), dim3(t.tileStart[t.n]), dim3(kBlock), 0, s, t);
+      FX_HIP(hipGetLastError());
+      t.n = 0;
+    }
+    if (i == n) break;
+    t.d[t.n] = d[i];
+    t.tileStart[t.n + 1] = t.tileStart[t.n] + tiles[i];
+    t.n++;
+  }
   return flagcxSuccess;
 }
 

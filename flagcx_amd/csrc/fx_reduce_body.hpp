@@ -827,16 +827,20 @@ struct BcastDescDev {
   uint32_t nout;
 };
 
+// Two table sizes: the kernel-argument block is copied at every launch (about
+// 0.3 us per KiB), and the common case -- a whole all-reduce merged into one
+// descriptor -- should not carry fifteen empty slots.
 constexpr int kInlineBcast = 16;
 
+template <int NS>
 struct InlineBcastTable {
-  BcastDescDev d[kInlineBcast];
-  uint32_t tileStart[kInlineBcast + 1];
+  BcastDescDev d[NS];
+  uint32_t tileStart[NS + 1];
   uint32_t n;
 };
 
-template <class R, int K, int U>
-__global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable t) {
+template <class R, int K, int U, int NS>
+__global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable<NS> t) {
   const uint32_t b = blockIdx.x;
   const uint32_t i = findSlice(t.tileStart, t.n, b);
   const BcastDescDev &d = t.d[i];

@@ -59,17 +59,17 @@ flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t co
   return launchDirectU<R, K, unrollFor(K)>(out, in, k, count, s);
 }
 
-template <class R, int K>
-flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, const uint32_t *tiles, size_t n, hipStream_t s) {
+template <class R, int K, int NS>
+flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, const uint32_t *tiles, size_t n, hipStream_t s) {
   constexpr int U = unrollFor(K);
-  InlineSliceTable<K> t;
+  InlineSliceTable<K, NS> t;
   t.n = 0;
   t.tileStart[0] = 0;
   for (size_t i = 0; i <= n; i++) {
-    const bool full = t.n == (uint32_t)InlineSliceTable<K>::kSlots ||
+    const bool full = t.n == (uint32_t)InlineSliceTable<K, NS>::kSlots ||
                       (i < n && (uint64_t)t.tileStart[t.n] + tiles[i] > 0x7ffffff0ull);
     if ((i == n || full) && t.n > 0) {
-      hipLaunchKernelGGL((reduceSlicesInline<R, K, U>), dim3(t.tileStart[t.n]), dim3(kBlock), 0, s, t);
+      hipLaunchKernelGGL((reduceSlicesInline<R, K, U, NS>), dim3(t.tileStart[t.n]), dim3(kBlock), 0, s, t);
       FX_HIP(hipGetLastError());
       t.n = 0;
     }
@@ -82,6 +82,12 @@ flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, const uint32_t *til
     t.n++;
   }
   return flagcxSuccess;
+}
+
+template <class R, int K>
+flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, const uint32_t *tiles, size_t n, hipStream_t s) {
+  if (n <= (size_t)kSmallSliceTable) return launchSlicesInlineSized<R, K, kSmallSliceTable>(slices, tiles, n, s);
+  return launchSlicesInlineSized<R, K, 0>(slices, tiles, n, s);
 }
 
 template <class R, int K>

@@ -781,9 +781,15 @@ constexpr int inlineSlicesFor() {
   return (4000 - 8) / (int)(sizeof(SliceDescK<K>) + sizeof(uint32_t));
 }
 
-template <int K>
+// NS = 0 means as many slots as fit under 4 KiB.  A second, small size exists
+// because the argument block is copied at every launch (about 0.3 us per KiB)
+// and most batches -- one descriptor per rank or per peer -- have eight
+// entries or fewer.
+constexpr int kSmallSliceTable = 8;
+
+template <int K, int NS = 0>
 struct InlineSliceTable {
-  static constexpr int kSlots = inlineSlicesFor<K>();
+  static constexpr int kSlots = NS > 0 ? NS : inlineSlicesFor<K>();
   SliceDescK<K> d[kSlots];
   uint32_t tileStart[kSlots + 1];
   uint32_t n;
@@ -807,8 +813,8 @@ __device__ __forceinline__ void reduceSlicesBody(const D *d, const uint32_t *til
   reduceTile<R, K, U>(sg, tp, b - tileStart[i]);
 }
 
-template <class R, int K, int U>
-__global__ void __launch_bounds__(kBlock) reduceSlicesInline(InlineSliceTable<K> t) {
+template <class R, int K, int U, int NS>
+__global__ void __launch_bounds__(kBlock) reduceSlicesInline(InlineSliceTable<K, NS> t) {
   reduceSlicesBody<R, K, U>(t.d, t.tileStart, t.n);
 }
 

@@ -264,3 +264,39 @@ def test_batch_of_independent_triggers_through_the_producer_loop(dev):
     assert lib.fx_fifo_run_batch(host, one, 1, 1000) == N.INTERNAL_ERROR
     assert lib.fx_fifo_run_batch(None, one, 1, 1000) == N.INVALID_ARGUMENT
     dev.free(host, N.MEM_HOST)
+
+
+def test_long_chain_of_dependent_triggers_sees_every_previous_result(dev):
+    """acc = acc + x_i forty times over 3 Mi elements (every workgroup of every die
+    takes part in each trigger, and trigger i + 1 reads what trigger i wrote, most of
+    it from another die): the results are stored through the caches and the next
+    trigger's workgroups invalidate before they load, so nothing stale is read."""
+    n, steps = 3 << 20, 40
+    ring = Ring(dev, capacity=8)
+    closed = False
+    try:
+        rng = np.random.default_rng(31)
+        acc = rng.integers(-1000, 1000, n).astype(np.int32)
+        xs = [rng.integers(-1000, 1000, n).astype(np.int32) for _ in range(4)]
+        with DevBufs(dev) as b:
+            dacc = b.put(acc)
+            dxs = [b.put(x) for x in xs]
+            want = acc.copy()
+            for i in range(steps):
+                ring.wait(ring.enqueue(dacc, dxs[i % 4], dacc, n, N.DT_INT32, N.OP_SUM))      # output == input 1
+                want += xs[i % 4]
+            # ping-pong between two buffers, max: a stale read would let an old, smaller value survive
+            da, db2 = b.put(acc), b.alloc(n * 4)
+            hi = acc.copy()
+            for i in range(steps):
+                src, dst = (da, db2) if i % 2 == 0 else (db2, da)
+                ring.wait(ring.enqueue(src, dxs[i % 4], dst, n, N.DT_INT32, N.OP_MAX))
+                hi = np.maximum(hi, xs[i % 4])
+            reason, done, bad = ring.close()
+            closed = True
+            assert (reason, done, bad) == (1, 2 * steps, 0)
+            assert np.array_equal(dev.to_host(dacc, n, np.int32), want)
+            assert np.array_equal(dev.to_host(da, n, np.int32), hi)
+    finally:
+        if not closed:
+            ring.close()

@@ -130,7 +130,8 @@ __device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b,
   }
 }
 
-// Who works on trigger number seq.  One workgroup per 16 KiB tile, at least one
+// Who works on trigger number seq.  One workgroup per 16 KiB tile (per eight
+// tiles for a trigger that arrived in bulk, see kBulkArrivals), at least one
 // (which completes empty and unsupported triggers), at most G-1: workgroup 0
 // never computes, so it is always free to talk to the host, and the workers of
 // a small trigger start at a position that rotates with seq, so consecutive

@@ -92,7 +92,8 @@ int fx_reduce_triggers(const fxReduceTrigger *triggers, size_t n, void *stream);
  * a pinned buffer of uint64 words [capacity, consumed, produced, terminate]
  * followed by `capacity` triggers.  fx_fifo_enqueue returns idx = -1 when the
  * ring is full or the slot has not been collected yet (the caller retries);
- * fx_fifo_poll_state / fx_fifo_set_state are pollState / setState.
+ * fx_fifo_poll_state / fx_fifo_set_state are pollState / setState.  One
+ * producer thread per ring, as in the reference.
  */
 size_t fx_fifo_bytes(size_t capacity);
 int fx_fifo_init(uint64_t *fifo, size_t capacity);

@@ -300,3 +300,61 @@ def test_long_chain_of_dependent_triggers_sees_every_previous_result(dev):
     finally:
         if not closed:
             ring.close()
+
+
+def test_ring_allreduce_driven_through_the_fifo(dev):
+    """What an unmodified uniRunner does with this consumer behind its FIFO
+    (uni_runner_impl.cc:661-1007): n-1 reduce-scatter steps whose reduce nodes --
+    one per rank, slice and red-slice: in1 = the previous rank's partial, in2 = own
+    data, out = own receive buffer -- go through the ring as triggers, each step
+    waiting for the one before; then the all-gather copies.  fp32, so the result
+    must equal the hop-by-hop ring oracle bit for bit."""
+    from flagcx_amd import kernels as K
+    n, count, nslices, nred = 8, 8 * 50021 + 5, 2, 3
+    dtype, es = N.DT_FP32, 4
+    sends = seeded_inputs(dtype, n, count, seed=41)
+    rng = np.random.default_rng(41)
+    sends = [(a * 10.0 ** rng.integers(-3, 9, count)).astype(np.float32) for a in sends]     # make the order matter
+    want = O.ring_allreduce(sends, dtype, N.OP_SUM)
+    ring = Ring(dev, capacity=128)
+    closed = False
+    try:
+        with DevBufs(dev) as b:
+            ds = [b.put(a) for a in sends]
+            dr = [b.alloc(count * es) for _ in range(n)]
+            ntrig = 0
+            for i in range(n - 1):                                   # reduce-scatter steps
+                trig = (N.ReduceTrigger * (n * nslices * nred))()
+                t = 0
+                for r in range(n):
+                    prev, rx = (r - 1) % n, (r - i - 1) % n
+                    ccnt, coff = K.split(count, n, rx)
+                    partial = ds[prev] if i == 0 else dr[prev]
+                    for s in range(nslices):
+                        scnt, soff = K.split(ccnt, nslices, s)
+                        for q in range(nred):
+                            rcnt, roff = K.split(scnt, nred, q)
+                            off = (coff + soff + roff) * es
+                            lib.fx_trigger_set(C.byref(trig[t]), partial + off, ds[r] + off, dr[r] + off, rcnt, 32, dtype,
+                                               N.OP_SUM, ENQUEUED)
+                            t += 1
+                N.check(lib.fx_fifo_run_batch(ring.host, trig, t, 200_000_000))
+                ntrig += t
+            reason, done, bad = ring.close()
+            closed = True
+            assert (reason, done, bad) == (1, ntrig, 0)
+            stream = dev.stream_create()
+            for i in range(n - 1):                                   # all-gather steps: chunk (r - i) % n from the previous rank
+                copies = []
+                for r in range(n):
+                    ccnt, coff = K.split(count, n, (r - i) % n)
+                    copies.append((dr[(r - 1) % n] + coff * es, dr[r] + coff * es, ccnt * es))
+                N.check(K.copy_slices(copies, dev.raw_stream(stream)))
+            dev.stream_sync(stream)
+            dev.stream_destroy(stream)
+            for r in range(n):
+                got = dev.to_host(dr[r], count, np.float32)
+                assert np.array_equal(got.view(np.uint32), want[r].view(np.uint32)), f"rank {r}"
+    finally:
+        if not closed:
+            ring.close()

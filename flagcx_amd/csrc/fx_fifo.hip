@@ -185,7 +185,7 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
   uint64_t *hostTrig = host + 4;
   // workgroup 0, wavefront 0 (all of these stay wave-uniform):
   uint64_t mirrored = startSeq;      // triggers copied to the mirror so far
-  uint64_t lastPublished = ~0ull;    // last `completed` written to the host's `consumed`
+  uint64_t lastSeenCompleted = 0;    // progress of the workers, for the idle count
   bool hostTermSeen = false;
   const uint32_t lane = threadIdx.x;
   const uint64_t idleLimit = (blockIdx.x == 0 || maxIdlePolls > (~0ull >> 5)) ? maxIdlePolls : maxIdlePolls * 32;
@@ -229,7 +229,15 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
                                      __HIP_MEMORY_SCOPE_AGENT);
               waitVectorMemory();  // every lane's copies are acknowledged before the new count goes out
               mirrored = hp;
-              if (lane == 0) __hip_atomic_store(&m->produced, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              if (lane == 0) {
+                __hip_atomic_store(&m->produced, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // `consumed` counts triggers TAKEN from the ring, as the reference's
+                // dequeue does (flagcx_reduce_kernel_device.cu:53-73); the producer only
+                // uses it to see whether the ring is full, the slot's state word says
+                // when a slot is free again.  Published at once, so that the producer is
+                // never held up by this loop's pace.
+                __hip_atomic_store(host + 1, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+              }
               idle = 0;  // the host is alive
             }
             // The host sets terminate after its last enqueue, but two relaxed
@@ -242,10 +250,8 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
             uint64_t c = 0;
             if (lane == 0) c = pollDev(&m->completed);
             c = fromLane(c, 0);
-            if (c != lastPublished) {
-              if (lane == 0)  // consumed: a progress report; the exact figure is published on the way out
-                __hip_atomic_store(host + 1, startSeq + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-              lastPublished = c;
+            if (c != lastSeenCompleted) {
+              lastSeenCompleted = c;
               idle = 0;  // so are the workers
             }
           }

@@ -203,6 +203,27 @@ def run_fifo(dev, a):
                 ms = (time.perf_counter() - t0) * 1e3 / total
                 row("fifo ring kept full, per trigger", n * 4, ms, 3 * n * 4)
             nbytes *= a.factor
+        # BASELINE config 2 as the reference's scheduler would run it through this ring: one reduce-scatter step of
+        # the ring all-reduce for all 8 simulated ranks = 8 x 8 slices x 2 pieces = 128 two-input bf16 triggers of
+        # 262,144 elements (512 KiB), all independent; 7 such steps make the reduce-scatter.
+        n, k, piece = 33_554_432, 8, 262_144
+        if emax >= n * 2:
+            chunk = n // k
+            total = k * (chunk // piece)
+            trig = (N.ReduceTrigger * total)()
+            t = 0
+            for r in range(k):
+                for q in range(chunk // piece):
+                    off = (r * chunk + q * piece) * 2
+                    lib.fx_trigger_set(C.byref(trig[t]), bufs[0] + off, bufs[1] + off, bufs[2] + off, piece, 32,
+                                       N.DT_BF16, N.OP_SUM, 1)
+                    t += 1
+            N.check(lib.fx_fifo_run_batch(host, trig, total, 50_000_000))          # warm-up
+            t0 = time.perf_counter()
+            for _ in range(7):
+                N.check(lib.fx_fifo_run_batch(host, trig, total, 50_000_000))
+            ms = (time.perf_counter() - t0) * 1e3 / 7
+            row("config-2 ring step, 128 triggers of 512 KiB", total * piece * 2, ms, 3 * total * piece * 2)
     finally:
         lib.fx_fifo_terminate(host)
         dev.stream_sync(stream)

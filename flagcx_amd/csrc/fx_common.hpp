@@ -4,6 +4,8 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <new>
+#include <tuple>
+#include <utility>
 
 #include "flagcx_amd/fx_types.h"
 
@@ -33,11 +35,24 @@ __host__ __device__ inline size_t dtypeSize(int dt) {
 
 inline bool opSupported(int op) { return op >= flagcxSum && op <= flagcxAvg; }
 
-#define FX_HIP(call)                                                           \
-  do {                                                                         \
-    hipError_t e_ = (call);                                                    \
-    if (e_ != hipSuccess) return flagcxUnhandledDeviceError;                   \
-  } while (0)
+// Launch `kernel` on a grid of `grid` workgroups of kBlock threads and report
+// THIS launch's own status: the return value of hipLaunchKernel, not the
+// thread's last-error slot, which an unrelated earlier call (say an allocation
+// the caller saw fail and handled) may still occupy.
+template <class Tuple, size_t... I>
+inline void argPointers(Tuple &vals, void **argv, std::index_sequence<I...>) {
+  ((argv[I] = static_cast<void *>(&std::get<I>(vals))), ...);
+}
+template <class... P, class... A>
+inline flagcxResult_t launchKernel(void (*kernel)(P...), uint32_t grid, hipStream_t s, const A &...args) {
+  static_assert(sizeof...(P) == sizeof...(A), "one argument per kernel parameter");
+  std::tuple<P...> vals{static_cast<P>(args)...};  // each argument in the kernel's own parameter type
+  void *argv[sizeof...(P)];
+  argPointers(vals, argv, std::index_sequence_for<P...>{});
+  return hipLaunchKernel(reinterpret_cast<const void *>(kernel), dim3(grid), dim3(kBlock), argv, 0, s) == hipSuccess
+             ? flagcxSuccess
+             : flagcxUnhandledDeviceError;
+}
 
 // No C++ exception may cross the C ABI: host entry points that allocate run
 // their body through this.

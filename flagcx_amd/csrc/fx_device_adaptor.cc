@@ -27,7 +27,14 @@ struct flagcxIpcMemHandle {
 
 namespace {
 
-inline flagcxResult_t dev(hipError_t e) { return e == hipSuccess ? flagcxSuccess : flagcxUnhandledDeviceError; }
+// The error is handed to the caller as a return code; it is also taken out of
+// the runtime's per-thread last-error slot so that it cannot be mistaken for the
+// result of a later, unrelated call.
+inline flagcxResult_t dev(hipError_t e) {
+  if (e == hipSuccess) return flagcxSuccess;
+  (void)hipGetLastError();
+  return flagcxUnhandledDeviceError;
+}
 
 inline flagcxResult_t ready(hipError_t e) {
   if (e == hipSuccess) return flagcxSuccess;

@@ -536,14 +536,14 @@ int fx_fifo_consumer_launch(fxFifoConsumer_t c, void *fifoDevicePointer, const u
   hipStream_t s = (hipStream_t)stream;
   static_assert(sizeof(FifoMirror) % sizeof(uint64_t) == 0, "FifoMirror is cleared in 8-byte words");
   const uint32_t words = (uint32_t)(sizeof(FifoMirror) / sizeof(uint64_t));
-  hipLaunchKernelGGL(clearMirror, dim3((words + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (uint64_t *)c->mirror, words);
-  FX_HIP(hipGetLastError());
+  flagcxResult_t rc = launchKernel(clearMirror, (words + kBlock - 1) / kBlock, s, (uint64_t *)c->mirror, words);
+  if (rc != flagcxSuccess) return rc;
   // Start where the last consumer stopped: triggers enqueued before this launch
   // are waiting between `consumed` and `produced` and are served first.
   const uint64_t startSeq = __atomic_load_n(&fifoHost[1], __ATOMIC_ACQUIRE);
-  hipLaunchKernelGGL(fifoConsumer, dim3(c->grid), dim3(kBlock), 0, s, (uint64_t *)fifoDevicePointer, c->mirror,
-                     c->capacity, startSeq, (uint64_t)maxIdlePolls);
-  FX_HIP(hipGetLastError());
+  rc = launchKernel(fifoConsumer, c->grid, s, (uint64_t *)fifoDevicePointer, c->mirror, c->capacity, startSeq,
+                    (uint64_t)maxIdlePolls);
+  if (rc != flagcxSuccess) return rc;
   return flagcxSuccess;
 }
 

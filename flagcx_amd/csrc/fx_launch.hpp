@@ -45,9 +45,7 @@ flagcxResult_t launchDirectU(void *out, const void *const *in, int k, uint64_t c
   uint64_t ntiles = tilesFor(out, in, kk, count, R::ES, U);
   if (ntiles == 0) return flagcxSuccess;
   if (ntiles > 0x7ffffff0ull) return flagcxInvalidArgument;
-  hipLaunchKernelGGL((reduceCopyDirect<R, K, U>), dim3((uint32_t)ntiles), dim3(kBlock), 0, s, a);
-  FX_HIP(hipGetLastError());
-  return flagcxSuccess;
+  return launchKernel(reduceCopyDirect<R, K, U>, (uint32_t)ntiles, s, a);
 }
 
 template <class R, int K>
@@ -69,8 +67,8 @@ flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, const uint32_t
     const bool full = t.n == (uint32_t)InlineSliceTable<K, NS>::kSlots ||
                       (i < n && (uint64_t)t.tileStart[t.n] + tiles[i] > 0x7ffffff0ull);
     if ((i == n || full) && t.n > 0) {
-      hipLaunchKernelGGL((reduceSlicesInline<R, K, U, NS>), dim3(t.tileStart[t.n]), dim3(kBlock), 0, s, t);
-      FX_HIP(hipGetLastError());
+      const flagcxResult_t rc = launchKernel(reduceSlicesInline<R, K, U, NS>, t.tileStart[t.n], s, t);
+      if (rc != flagcxSuccess) return rc;
       t.n = 0;
     }
     if (i == n) break;
@@ -95,9 +93,7 @@ flagcxResult_t launchSlicesTable(const SliceDescDev *d, const uint32_t *tileStar
                                  hipStream_t s) {
   constexpr int U = unrollFor(K);
   if (grid == 0) return flagcxSuccess;
-  hipLaunchKernelGGL((reduceSlicesTable<R, K, U>), dim3(grid), dim3(kBlock), 0, s, d, tileStart, n);
-  FX_HIP(hipGetLastError());
-  return flagcxSuccess;
+  return launchKernel(reduceSlicesTable<R, K, U>, grid, s, d, tileStart, n);
 }
 
 template <class R, int K>
@@ -109,9 +105,7 @@ flagcxResult_t launchBcastInline(const BcastDescDev *d, const uint32_t *tiles, s
     t.tileStart[0] = 0;
     t.tileStart[1] = tiles[0];
     t.n = 1;
-    hipLaunchKernelGGL((reduceBcastInline<R, K, U, 1>), dim3(tiles[0]), dim3(kBlock), 0, s, t);
-    FX_HIP(hipGetLastError());
-    return flagcxSuccess;
+    return launchKernel(reduceBcastInline<R, K, U, 1>, tiles[0], s, t);
   }
   InlineBcastTable<kInlineBcast> t;
   t.n = 0;
@@ -119,8 +113,8 @@ flagcxResult_t launchBcastInline(const BcastDescDev *d, const uint32_t *tiles, s
   for (size_t i = 0; i <= n; i++) {
     const bool full = t.n == (uint32_t)kInlineBcast || (i < n && (uint64_t)t.tileStart[t.n] + tiles[i] > 0x7ffffff0ull);
     if ((i == n || full) && t.n > 0) {
-      hipLaunchKernelGGL((reduceBcastInline<R, K, U, kInlineBcast>), dim3(t.tileStart[t.n]), dim3(kBlock), 0, s, t);
-      FX_HIP(hipGetLastError());
+      const flagcxResult_t rc = launchKernel(reduceBcastInline<R, K, U, kInlineBcast>, t.tileStart[t.n], s, t);
+      if (rc != flagcxSuccess) return rc;
       t.n = 0;
     }
     if (i == n) break;

@@ -287,3 +287,51 @@ def test_cfg5_through_the_collective(dev, stream):
             for pos in np.linspace(0, n - win, 9).astype(np.int64):
                 got = dev.to_host(dr[r] + int(pos) * 2, win, np.uint16)
                 assert np.array_equal(got, first[pos:pos + win]), f"rank {r} window at {pos}"
+
+
+def test_half_the_hbm_in_one_launch(dev):
+    """Sized for the part: 8 inputs of 16 GiB (2^33 + 12,345 bf16 elements each) and
+    a 16 GiB output -- 144 GiB resident, 524,289 workgroups, element counts and byte
+    offsets far beyond 32 bits -- in ONE fx_reduce_copy.  Inputs are byte patterns
+    with seeded random patches at the start, across every 4 GiB boundary and at
+    the ragged end; the whole output is downloaded window by window and compared
+    with the oracle, and the bytes behind it must be untouched."""
+    k, dtype, es = 8, N.DT_BF16, 2
+    count = (1 << 33) + 12345
+    nbytes = count * es
+    patch_el = 1 << 19                                                   # 1 MiB of bf16
+    starts = sorted({0, count - patch_el} | {(g << 32) // es - patch_el // 2 for g in range(1, 4)})
+    rng = np.random.default_rng(8)
+    fills = [0x3c + p for p in range(k)]                                  # bf16 0x3c3c .. 0x4343: finite, distinct
+    with DevBufs(dev) as b:
+        try:
+            dins = [b.alloc(nbytes + 256) for _ in range(k)]
+            dout = b.alloc(nbytes + 256)
+        except RuntimeError as e:                                        # a smaller part, or memory in use
+            pytest.skip(f"cannot hold 144 GiB on this device: {e}")
+        patches = []
+        for p in range(k):
+            dev.memset(dins[p], fills[p], nbytes)
+            mine = {}
+            for s in starts:
+                bits = rng.integers(0, 1 << 16, patch_el, dtype=np.uint16)
+                bits[(bits & 0x7f80) == 0x7f80] = 0x3f80                 # no inf / NaN: keep the sum's bits defined
+                mine[s] = bits
+                dev.upload(dins[p] + s * es, bits)
+            patches.append(mine)
+        dev.memset(dout, 0xEE, nbytes + 256)
+        N.check(K.reduce_copy(dout, dins, count, dtype, N.OP_SUM), "fx_reduce_copy")
+        dev.sync()
+        base = [np.uint16(f << 8 | f) for f in fills]
+        plain = O.reduce_copy([np.full(4, v, np.uint16) for v in base], dtype, N.OP_SUM)[0]
+        step = 1 << 27                                                   # 256 MiB of bf16 per download
+        for off in range(0, count, step):
+            n = min(step, count - off)
+            got = dev.to_host(dout + off * es, n, np.uint16)
+            want = np.full(n, plain, np.uint16)
+            for s in starts:
+                lo, hi = max(s, off), min(s + patch_el, off + n)
+                if lo < hi:
+                    want[lo - off:hi - off] = O.reduce_copy([patches[p][s][lo - s:hi - s] for p in range(k)], dtype, N.OP_SUM)
+            assert np.array_equal(got, want), f"window at element {off}"
+        assert (dev.to_host(dout + nbytes, 256, np.uint8) == 0xEE).all(), "wrote past the end"

@@ -44,9 +44,10 @@ constexpr int kBatch = 16;  // triggers a workgroup inspects per round of mirror
 // an eighth of the workgroups each, eight tiles per workgroup, so that eight
 // times as many triggers run side by side and each workgroup's fixed cost per
 // trigger is spread over eight tiles (2 MiB triggers with the ring kept full:
-// 2.2 us each shared out fully, 1.6 us at a quarter, 1.5 us at an eighth).  Workgroup 0 decides (it sees how many
-// arrived together) and marks the mirrored copy in a bit the ring format leaves
-// unused; the bit never reaches the host.
+// 2.2 us each shared out fully, 1.6 us at a quarter, 1.5 us at an eighth).
+// Workgroup 0 decides (it sees how many arrived together) and marks the
+// mirrored copy in a bit the ring format leaves unused; the bit never reaches
+// the host.
 constexpr uint64_t kBulkArrivals = 4;
 constexpr uint64_t kBulkBit = 1ull << 63;
 constexpr int kBulkShift = 3;

@@ -255,6 +255,44 @@ def test_reduce_fifo_host_protocol():
     assert N.lib.fx_fifo_poll_state(buf, 5) == -1
 
 
+def test_reduce_fifo_producer_loop_against_a_host_side_consumer():
+    """fx_fifo_run_batch (the scheduler's enqueue-and-collect loop) with a Python
+    thread playing the consumer on the same ring: 200 triggers through 8 slots are
+    all delivered once, in order, with the fields they were given; with nobody
+    consuming, the loop gives up after its spin limit."""
+    import threading
+    cap, total = 8, 200
+    buf = (C.c_uint64 * (N.lib.fx_fifo_bytes(cap) // 8))()
+    N.check(N.lib.fx_fifo_init(buf, cap))
+    trig = (N.ReduceTrigger * total)()
+    for i in range(total):
+        N.lib.fx_trigger_set(C.byref(trig[i]), 1000 + i, 2000 + i, 3000 + i, i, 32, i % 10, i % 5, 1)
+    seen, stop = [], threading.Event()
+
+    def consumer():                                   # the protocol of flagcx_reduce_kernel_device.cu:53-186, in Python
+        taken = 0
+        while not stop.is_set() and taken < total:
+            if buf[2] > taken:                        # produced
+                w = 4 + 4 * (taken % cap)
+                seen.append((buf[w], buf[w + 1], buf[w + 2], buf[w + 3] & 0xffffffff, (buf[w + 3] >> 48) & 0xf,
+                             (buf[w + 3] >> 52) & 0xf))
+                taken += 1
+                buf[1] = taken                        # consumed
+                buf[w + 3] |= 3 << 56                 # Complete
+    t = threading.Thread(target=consumer)
+    t.start()
+    try:
+        assert N.lib.fx_fifo_run_batch(buf, trig, total, 2_000_000_000) == N.SUCCESS
+    finally:
+        stop.set()
+        t.join(timeout=30)
+    assert seen == [(1000 + i, 2000 + i, 3000 + i, i, i % 10, i % 5) for i in range(total)]
+    assert buf[2] == total and all((buf[4 + 4 * s + 3] >> 56) & 3 == 0 for s in range(cap))     # every slot handed back
+    assert N.lib.fx_fifo_run_batch(buf, trig, 1, 1000) == N.INTERNAL_ERROR                       # nobody consumes
+    assert N.lib.fx_fifo_run_batch(buf, None, 1, 1000) == N.INVALID_ARGUMENT
+    assert N.lib.fx_fifo_run_batch(buf, trig, 0, 1000) == N.SUCCESS
+
+
 def test_headers_are_plain_c_and_a_c_client_links(tmp_path):
     """The boundary is a C ABI: every header compiles as strict C11, a C program
     links against the kernel library and the host-only entry points answer."""

@@ -52,6 +52,7 @@ constexpr uint64_t kBulkArrivals = 4;
 constexpr uint64_t kBulkBit = 1ull << 63;
 constexpr int kBulkShift = 3;
 constexpr uint32_t kMaxCapacity = 1024;
+constexpr uint64_t kMirrorBatch = 64;  // triggers workgroup 0 mirrors per pass
 
 struct FifoMirror {              // device memory, zeroed at creation
   uint64_t produced;             // triggers mirrored so far (written by workgroup 0)
@@ -206,22 +207,42 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
             const uint64_t hp = fromLane(v, 0), ht = fromLane(v, 1);
             if (mirrored < hp) {
               __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // the triggers behind `produced`
-              const uint64_t words = 4 * (hp - mirrored);     // at most 4 * capacity
+              // at most kMirrorBatch triggers per pass (four words per lane); the rest next time round
+              const uint64_t arrived = hp - mirrored;
+              const uint64_t upTo = mirrored + (arrived < kMirrorBatch ? arrived : kMirrorBatch);
+              const uint64_t words = 4 * (upTo - mirrored);
               // Refill the slots like a sequence lock: number invalid, words, number
               // valid.  All of these are agent-scope atomic stores (they go to the
               // coherent cache level themselves); between the phases the wavefront
               // waits for one phase's stores to be acknowledged before it issues the
-              // next -- no cache write-back each.
+              // next -- no cache write-back each.  The words come over PCIe (over a
+              // microsecond); the stores that take the slots out of service -- number
+              // invalid, count-in counter back to zero: the previous trigger in a slot
+              // is long complete, or the host could not have reused it -- are issued
+              // behind those reads and acknowledged while they are in flight.
+              uint64_t fetched[4];
+#pragma unroll
+              for (int r = 0; r < 4; r++) {
+                const uint64_t w = lane + 64ull * r;
+                fetched[r] = 0;
+                if (w < words) fetched[r] = pollSys(hostTrig + 4 * ((mirrored + w / 4) % cap) + (w & 3));
+              }
               for (uint64_t w = lane; w < words; w += 64)
-                if ((w & 3) == 0)
-                  __hip_atomic_store(&m->trigSeq[(mirrored + w / 4) % cap], kNoTrigger, __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT);
+                if ((w & 3) == 0) {
+                  const uint32_t slot = (uint32_t)((mirrored + w / 4) % cap);
+                  __hip_atomic_store(&m->trigSeq[slot], kNoTrigger, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                  __hip_atomic_store(&m->done[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
               waitVectorMemory();
-              for (uint64_t w = lane; w < words; w += 64) {
-                const uint32_t slot = (uint32_t)((mirrored + w / 4) % cap);
-                uint64_t word = pollSys(hostTrig + 4 * slot + (w & 3));
-                if ((w & 3) == 3) word = (hp - mirrored >= kBulkArrivals) ? (word | kBulkBit) : (word & ~kBulkBit);
-                __hip_atomic_store(&m->trig[slot][w & 3], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+              for (int r = 0; r < 4; r++) {
+                const uint64_t w = lane + 64ull * r;
+                if (w < words) {
+                  const uint32_t slot = (uint32_t)((mirrored + w / 4) % cap);
+                  uint64_t word = fetched[r];
+                  if ((w & 3) == 3) word = (arrived >= kBulkArrivals) ? (word | kBulkBit) : (word & ~kBulkBit);
+                  __hip_atomic_store(&m->trig[slot][w & 3], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
               }
               waitVectorMemory();
               for (uint64_t w = lane; w < words; w += 64)
@@ -229,22 +250,24 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
                   __hip_atomic_store(&m->trigSeq[(mirrored + w / 4) % cap], mirrored + w / 4, __ATOMIC_RELAXED,
                                      __HIP_MEMORY_SCOPE_AGENT);
               waitVectorMemory();  // every lane's copies are acknowledged before the new count goes out
-              mirrored = hp;
+              mirrored = upTo;
               if (lane == 0) {
-                __hip_atomic_store(&m->produced, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&m->produced, upTo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 // `consumed` counts triggers TAKEN from the ring, as the reference's
                 // dequeue does (flagcx_reduce_kernel_device.cu:53-73); the producer only
                 // uses it to see whether the ring is full, the slot's state word says
                 // when a slot is free again.  Published at once, so that the producer is
                 // never held up by this loop's pace.
-                __hip_atomic_store(host + 1, hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                __hip_atomic_store(host + 1, upTo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
               }
               idle = 0;  // the host is alive
             }
             // The host sets terminate after its last enqueue, but two relaxed
             // polls may be served out of order: act on terminate only on the poll
             // AFTER the one that first saw it, when `produced` has been re-read.
-            if (ht) {
+            // And only once everything the host has produced is mirrored (a pass
+            // takes at most kMirrorBatch triggers).
+            if (ht && mirrored >= hp) {
               if (hostTermSeen && lane == 0) storeDev(&m->terminate, ht);
               hostTermSeen = true;
             }
@@ -293,9 +316,10 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       if (lane == 0) sh[0] = state;
       if (state == kWork) {
         // Reader side of the sequence lock, for up to kBatch triggers at once (lane
-        // i looks at trigger seq + i): three dependent rounds of reads serve the
-        // whole batch instead of one trigger.  If a slot still carries the expected
-        // number after its words were read, they are that trigger's.  If not, the
+        // i looks at trigger seq + i): two dependent rounds of reads serve the whole
+        // batch.  The writer takes a slot out of service BEFORE it touches the words
+        // and puts the new number in AFTER, so if a slot carries the expected number
+        // after its words were read, the words are that trigger's.  If not, the
         // ring has come round: the trigger is complete, which it could not be had
         // this workgroup been one of its workers -- so there is nothing to do.
         // (agent-scope atomic loads read the coherent cache level; each step's
@@ -306,16 +330,14 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
         const bool mine = lane < batch;
         const uint64_t want = seq + lane;
         const uint32_t slot = (uint32_t)(want % cap);
-        uint64_t before = kNoTrigger, after = kNoTrigger, w[4] = {0, 0, 0, 0};
-        if (mine) before = pollDev(&m->trigSeq[slot]);
-        waitVectorMemory();
+        uint64_t after = kNoTrigger, w[4] = {0, 0, 0, 0};
         if (mine)
           for (int q = 0; q < 4; q++) w[q] = pollDev(&m->trig[slot][q]);
         waitVectorMemory();
         if (mine) after = pollDev(&m->trigSeq[slot]);
         if (mine) {
           for (int q = 0; q < 4; q++) shTrig[lane][q] = w[q];
-          shValid[lane] = (before == want && after == want) ? 1u : 0u;
+          shValid[lane] = (after == want) ? 1u : 0u;
         }
         if (lane == 0) sh[1] = batch;
       }
@@ -347,11 +369,11 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
     const Share share = shareOf(seq, in1, in2, out, count, dtype, op, bulk);
     if (shValid[bi] == 0 || share.idx >= share.takers) continue;  // overtaken by the ring, or not needed for this trigger
     // The trigger's buffers may have been written by other agents since this
-    // kernel last looked: drop stale cache lines before reading them.  The caches
-    // are the compute unit's and the die's, not a wavefront's, so one wavefront
-    // invalidates for the whole workgroup and the barrier orders the others'
-    // loads behind it (four invalidates per workgroup cost 5 us more per large
-    // trigger than one).
+    // kernel last looked: drop stale cache lines before reading them.  Only a
+    // workgroup that takes tiles does so (every workgroup doing it for every batch
+    // it inspects costs more than a microsecond per round trip), and one wavefront
+    // does it for the workgroup: the caches are the compute unit's and the die's,
+    // and the barrier orders the other wavefronts' loads behind it.
     if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
     __syncthreads();
     bool ok = true;
@@ -384,14 +406,12 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (prev == share.takers - 1) {  // last one out completes the trigger
         // Everybody else has counted in, so everybody's results are in memory; this
-        // thread reads none of them.  What must be ordered is its own bookkeeping:
-        // the counter is back at zero (acknowledged) before the host can learn that
-        // the slot is free again.  No cache-wide write-back or invalidate here --
-        // either would stall every workgroup of this die that is busy with another
-        // trigger (0.78 against 1.3 us per 256 KiB trigger with the ring kept full).
-        __hip_atomic_store(&m->done[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // thread reads none of them, and the counter is put back to zero by workgroup
+        // 0 when it next fills the slot: Complete can go out at once.  No cache-wide
+        // write-back or invalidate here -- either would stall every workgroup of this
+        // die that is busy with another trigger (0.78 against 1.3 us per 256 KiB
+        // trigger with the ring kept full).
         if (!ok) __hip_atomic_fetch_add(&m->badTriggers, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        waitVectorMemory();
         __hip_atomic_store(hostTrig + 4 * slot + 3, w3 | ((uint64_t)fxTriggerComplete << 56), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_SYSTEM);
         __hip_atomic_fetch_add(&m->completed, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

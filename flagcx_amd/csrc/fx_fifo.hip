@@ -199,12 +199,18 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
       uint64_t idle = 0, state, p = 0;  // p: triggers published so far, as last polled
       bool termSeen = false;
       for (;;) {
-        uint64_t term;
+        uint64_t term, termMirror = 0;
         if (blockIdx.x == 0) {
           if (mirrored <= seq) {  // nothing mirrored is waiting for this workgroup: talk to the host
+            // one round of reads: the host's `produced` and `terminate` over PCIe and,
+            // alongside them, the workers' progress and the mirror's terminate word
             uint64_t v = 0;
             if (lane < 2) v = pollSys(host + 2 + lane);
+            else if (lane == 2) v = pollDev(&m->completed);
+            else if (lane == 3) v = pollDev(&m->terminate);
             const uint64_t hp = fromLane(v, 0), ht = fromLane(v, 1);
+            const uint64_t c = fromLane(v, 2);
+            termMirror = fromLane(v, 3);
             if (mirrored < hp) {
               __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // the triggers behind `produced`
               // at most kMirrorBatch triggers per pass (four words per lane); the rest next time round
@@ -271,17 +277,17 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
               if (hostTermSeen && lane == 0) storeDev(&m->terminate, ht);
               hostTermSeen = true;
             }
-            uint64_t c = 0;
-            if (lane == 0) c = pollDev(&m->completed);
-            c = fromLane(c, 0);
             if (c != lastSeenCompleted) {
               lastSeenCompleted = c;
               idle = 0;  // so are the workers
             }
           }
-          uint64_t t = 0;
-          if (lane == 0) t = pollDev(&m->terminate);
-          term = fromLane(t, 0);
+          if (mirrored > seq) {  // a one-workgroup grid working off its own backlog: no host round this time
+            uint64_t t = 0;
+            if (lane == 0) t = pollDev(&m->terminate);
+            termMirror = fromLane(t, 0);
+          }
+          term = termMirror;
           // With workers in the grid this workgroup never takes a tile, so it does
           // not look at the triggers it has mirrored at all (three dependent reads
           // each): it goes straight back to the host.
@@ -311,7 +317,10 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
           state = kExitIdle;
           break;
         }
-        __builtin_amdgcn_s_sleep(32);
+        // Workgroup 0 is alone on the PCIe link and each of its rounds already takes
+        // over a microsecond; the workers poll device memory, 255 of them.
+        if (blockIdx.x == 0) __builtin_amdgcn_s_sleep(4);
+        else __builtin_amdgcn_s_sleep(32);
       }
       if (lane == 0) sh[0] = state;
       if (state == kWork) {

@@ -120,7 +120,7 @@ int fx_fifo_run_batch(uint64_t *fifo, const fxReduceTrigger *triggers, size_t n,
  * persistent full-width kernel executes every trigger the host enqueues, for
  * every op and type, and marks it Complete; it returns when `terminate`
  * is set and the ring is drained, or after maxIdlePolls consecutive empty
- * polls of the host ring (a few microseconds each; so it always ends).
+ * polls of the host ring (one to two microseconds each; so it always ends).
  * fifoDevicePointer is hostGetDevicePointer() of the pinned ring, fifoHost
  * the ring itself.  Triggers that sit in the ring at
  * the same time must not depend on each other.  Capacity <= 1024.  The grid is

@@ -364,3 +364,13 @@ def test_kernel_index_arithmetic_on_the_host(tmp_path):
                    capture_output=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.startswith("ok"), out.stdout
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Nothing in this build uses a second GPU; the benchmark says so instead of
+    pretending to scale."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "--gpus must be 1" in r.stderr and r.stdout == ""

@@ -33,7 +33,7 @@ SEED = 4                       # values N(0, 0.02)
 
 
 def cfg1(args):
-    """BASELINE configs[0]: out = a + b, fp32, 16,777,216 elements, uniform[-1,1)
+    """BASELINE.json configs[0]: out = a + b, fp32, 16,777,216 elements, uniform[-1,1)
     seed 0 -- on the GPU and, as the reference runs it, as one scalar host loop."""
     import numpy as np
 

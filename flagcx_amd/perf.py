@@ -3,8 +3,8 @@
 algBw = bytes / 1e9 / t).  Usage:
 
     python -m flagcx_amd.perf reduce  -k 4 -d fp16 -o sum -b 1K -e 1G -f 2 [--inplace]
-    python -m flagcx_amd.perf slices            # BASELINE config 2: rank shares in 512 KiB pieces + all-gather copy
-    python -m flagcx_amd.perf pack              # BASELINE config 4: alltoallv pack / unpack
+    python -m flagcx_amd.perf slices            # BASELINE.json configs[1]: rank shares in 512 KiB pieces + all-gather copy
+    python -m flagcx_amd.perf pack              # BASELINE.json configs[3]: alltoallv pack / unpack
     python -m flagcx_amd.perf allreduce -n 8 -d bf16 -b 1M -e 64M
     python -m flagcx_amd.perf fifo -b 4K -e 256M -f 8   # round trips through the reduce FIFO
 """
@@ -203,7 +203,7 @@ def run_fifo(dev, a):
                 ms = (time.perf_counter() - t0) * 1e3 / total
                 row("fifo ring kept full, per trigger", n * 4, ms, 3 * n * 4)
             nbytes *= a.factor
-        # BASELINE config 2 as the reference's scheduler would run it through this ring: one reduce-scatter step of
+        # BASELINE.json configs[1] as the reference's scheduler would run it through this ring: one reduce-scatter step of
         # the ring all-reduce for all 8 simulated ranks = 8 x 8 slices x 2 pieces = 128 two-input bf16 triggers of
         # 262,144 elements (512 KiB), all independent; 7 such steps make the reduce-scatter.
         n, k, piece = 33_554_432, 8, 262_144

@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Writes tests/golden/golden.json: digests of the CPU oracle's outputs on the
-seeded inputs of every BASELINE configuration.
+seeded inputs of every configuration of BASELINE.json.
 
     python tests/golden/make_golden.py [--full]
 

@@ -1,4 +1,4 @@
-"""The BASELINE configurations as data: shapes, seeds, distributions.  Shared by
+"""The configurations of BASELINE.json as data: shapes, seeds, distributions.  Shared by
 the fixture generator, the parity tests and nothing else."""
 import hashlib
 

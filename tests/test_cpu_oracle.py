@@ -431,7 +431,7 @@ def test_split_tiles_exactly_and_is_balanced():
 
 
 def test_nredslices_reference_cases():
-    # BASELINE config 2: 33,554,432 elements, 8 ranks, 8 slices, 262,144-element pieces -> 2
+    # BASELINE.json configs[1]: 33,554,432 elements, 8 ranks, 8 slices, 262,144-element pieces -> 2
     assert O.lib.oracle_nredslices(33554432, 8, 8, 0, 262144) == 2
     assert O.lib.oracle_nredslices(33554432, 8, 1, 0, 65536) == 64
     assert O.lib.oracle_nredslices(0, 8, 1, 0, 65536) == 1

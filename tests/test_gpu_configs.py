@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their FULL sizes on the GPU: bit-exact
+"""The five configurations of BASELINE.json at their FULL sizes on the GPU: bit-exact
 against committed digests of the oracle's output, against the oracle run live on
 this box's host cores, and through size-independent properties."""
 import json

@@ -11,7 +11,7 @@ OPS = {"sum": N.OP_SUM, "prod": N.OP_PROD, "max": N.OP_MAX, "min": N.OP_MIN, "av
 
 
 def seeded_inputs(dtype, k, n, seed, dist=None):
-    """k host arrays of n elements in the distribution BASELINE's configs name
+    """k host arrays of n elements in the distribution BASELINE.json's configs name
     for the type: fp32 uniform[-1,1), 16-bit N(0,1), int32 uniform[-2^20,2^20].
     The other host types of the reference (8/64-bit and unsigned integers over
     their whole range so that sums and products wrap, fp64 uniform[-1,1)) come

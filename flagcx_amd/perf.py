@@ -5,7 +5,7 @@ algBw = bytes / 1e9 / t).  Usage:
     python -m flagcx_amd.perf reduce  -k 4 -d fp16 -o sum -b 1K -e 1G -f 2 [--inplace]
     python -m flagcx_amd.perf slices            # BASELINE.json configs[1]: rank shares in 512 KiB pieces + all-gather copy
     python -m flagcx_amd.perf pack              # BASELINE.json configs[3]: alltoallv pack / unpack
-    python -m flagcx_amd.perf allreduce -n 8 -d bf16 -b 1M -e 64M
+    python -m flagcx_amd.perf allreduce -n 8 -d bf16 -b 1M -e 64M [--graph]
     python -m flagcx_amd.perf fifo -b 4K -e 256M -f 8   # round trips through the reduce FIFO
 """
 import argparse
@@ -230,6 +230,32 @@ def run_fifo(dev, a):
         lib.fx_fifo_consumer_destroy(cons)
 
 
+def _replay_of(t, post):
+    """Capture what `post` enqueues on the timer's stream into a HIP graph once; the returned function replays it."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so.7")          # the runtime the library is linked against (same mapping)
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    post()                                    # first call outside the capture: one-time set-up
+    t.dev.stream_sync(t.stream)
+    if hip.hipStreamBeginCapture(t.raw, 0) != 0:
+        raise RuntimeError("hipStreamBeginCapture failed")
+    try:
+        post()
+    finally:
+        rc = hip.hipStreamEndCapture(t.raw, C.byref(graph))
+    if rc != 0 or hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) != 0:
+        raise RuntimeError("the call could not be captured into a graph")
+
+    def replay():
+        if hip.hipGraphLaunch(gexec, t.raw) != 0:
+            raise RuntimeError("hipGraphLaunch failed")
+    return replay                             # graph and executable live until the process ends
+
+
 def run_allreduce(dev, a):
     t = Timer(dev)
     dtype, n = DT[a.dtype], a.nranks
@@ -242,10 +268,11 @@ def run_allreduce(dev, a):
             nbytes = size(a.min)
             while nbytes <= emax:
                 cnt = nbytes // es
-                ms = t.ms(lambda: N.check(g.all_reduce(ds, dr, cnt, dtype, OP[a.op], t.stream)))
+                post = lambda: N.check(g.all_reduce(ds, dr, cnt, dtype, OP[a.op], t.stream))
+                ms = t.ms(_replay_of(t, post)) if a.graph else t.ms(post)
                 alg = nbytes / ms / 1e6
                 # algBw = size / time, busBw = algBw * 2 (n - 1) / n, as test/perf/host_api/test_allreduce.cpp:11
-                print(f"{'allreduce n=%d %s %s' % (n, a.dtype, 'ring' if algo else 'direct'):<44s} size {nbytes:>12d} B   "
+                print(f"{'allreduce n=%d %s %s' % (n, a.dtype, ('ring' if algo else 'direct') + (' graph' if a.graph else '')):<44s} size {nbytes:>12d} B   "
                       f"{ms * 1e3:10.2f} us   algBw {alg:9.1f} GB/s   busBw {alg * 2 * (n - 1) / n:9.1f} GB/s", flush=True)
                 nbytes *= a.factor
 
@@ -261,6 +288,7 @@ def main(argv=None):
     ap.add_argument("-e", "--max", default="1G")
     ap.add_argument("-f", "--factor", type=int, default=2)
     ap.add_argument("--inplace", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="allreduce: capture one call into a HIP graph and time replays")
     ap.add_argument("--misalign", type=int, default=0, help="shift buffers by this many elements")
     ap.add_argument("--mixed", action="store_true", help="shift only every other input (inputs not aligned like the output)")
     ap.add_argument("--in-shift", type=int, default=0,

@@ -126,6 +126,9 @@ int fx_fifo_run_batch(uint64_t *fifo, const fxReduceTrigger *triggers, size_t n,
  * the same time must not depend on each other.  Capacity <= 1024.  The grid is
  * one workgroup per compute unit; FX_FIFO_WGS_PER_CU (environment, 1..8, read
  * at fx_fifo_consumer_create) asks for more, which measured slower.
+ * A ring can be served again after its consumer has ended (the launch reads
+ * `consumed` on the host to know where to resume, so the earlier kernel must
+ * have finished); triggers enqueued in between are served first.
  * While the consumer runs, calls that wait for the whole device (hipFree,
  * hipDeviceSynchronize) block until it has ended: set `terminate` first.
  */

@@ -62,6 +62,22 @@ def test_seeded_parity_k_and_sizes(dev, dname, oname):
         assert_parity(got, want, dtype, op, f"{dname} {oname} k={k} n={n}")
 
 
+@pytest.mark.parametrize("dname", ["bf16", "fp32", "int8", "uint64"])
+def test_largest_input_counts(dev, dname):
+    """k = 33 and k = 64 (FX_MAX_INPUTS), rotated, aligned and not, across the
+    striped-zone threshold for the wider types."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    for k, n, first, shift in [(33, 70001, 0, 0), (64, 1, 63, 0), (64, 40007, 17, 0), (64, 40007, 0, es),
+                               (64, (4 << 20) // es + 5, 5, 0)]:
+        ins = seeded_inputs(dtype, k, n, seed=200 + k)
+        for op in (N.OP_SUM, N.OP_MAX, N.OP_AVG):
+            want = O.reduce_copy(ins, dtype, op, first=first)
+            offs = [0] + [shift * (p % 3) for p in range(k)]
+            got = run_reduce(dev, ins, dtype, op, first=first, offs=offs)
+            assert_parity(got, want, dtype, op, f"{dname} op={op} k={k} n={n} first={first} shift={shift}")
+
+
 @pytest.mark.parametrize("dname", list(DTYPES))
 def test_inplace_matches_out_of_place(dev, dname):
     dtype = DTYPES[dname]

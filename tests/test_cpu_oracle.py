@@ -504,6 +504,13 @@ def test_ring_allreduce_closed_forms(n):
     want = sum(s.astype(np.float64) for s in sends).astype(np.float32)
     for recv in O.ring_allreduce(sends, F32, SUM):
         assert np.array_equal(recv, want)
+    # the intra-node kernel's own checks: (rank+1) -> n(n+1)/2 through the k-way fold in rank order
+    # (test/unittest/device_api/test_device_api_intra.cpp:363-389, test/perf/device_api/test_allreduce_intranode.cpp:196-211)
+    assert (O.reduce_copy([np.full(count, r + 1, np.float32) for r in range(n)], F32, SUM) == n * (n + 1) / 2).all()
+    # fixture pattern (i%10) + seed with seed = rank, compared as verifyBuffer does (test/fixtures/test_utils.hpp:11-34)
+    got = O.reduce_copy([((i % 10) + r).astype(np.float32) for r in range(n)], F32, SUM)
+    want = (n * (i % 10) + n * (n - 1) // 2).astype(np.float64)
+    assert (np.abs(got - want) / np.maximum(np.abs(want), 1e-10)).max() <= 1e-5 and np.array_equal(got, want.astype(np.float32))
 
 
 def test_ring_allreduce_order_is_the_rotated_left_fold():

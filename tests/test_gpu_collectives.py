@@ -241,6 +241,42 @@ def test_custom_allreduce_hook(dev, stream):
         assert_parity(dev.to_host(dr[5], 1001, np.uint16), want, dtype, N.OP_SUM, "odd count")
 
 
+@pytest.mark.parametrize("n", [2, 4, 8])
+def test_custom_allreduce_reference_intranode_cases(dev, stream, n):
+    """The reference's own checks of its intra-node all-reduce kernel, run through
+    the hook on registered windows: every rank contributes rank + 1, the result is
+    n (n + 1) / 2 everywhere -- in place on the registered buffer
+    (test/unittest/device_api/test_device_api_intra.cpp:363-389, tolerance 1e-1
+    there) and out of place into a receive buffer
+    (test/perf/device_api/test_allreduce_intranode.cpp:196-211, tolerance 1e-3);
+    exact here.  Then the fixture pattern (i % 10) + seed of
+    test/fixtures/test_utils.hpp:28-34 with seed = rank, compared the way its
+    verifyBuffer does (relative 1e-5, :11-26) and exactly."""
+    count = 1 << 20                                     # 4 MiB of fp32, inside the 8 MiB window
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        wins = [b.alloc(8 << 20) for _ in range(n)]
+        N.check(g.register_windows(wins, 8 << 20))
+        dr = [b.alloc(count * 4) for _ in range(n)]
+        for r in range(n):
+            dev.upload(wins[r], np.full(count, r + 1, np.float32))
+        N.check(g.custom_all_reduce(wins, dr, count, N.DT_FP32, N.OP_SUM, stream))      # out of place
+        N.check(g.custom_all_reduce(wins, wins, count, N.DT_FP32, N.OP_SUM, stream))    # in place on the windows
+        dev.stream_sync(stream)
+        for r in range(n):
+            assert (dev.to_host(dr[r], count, np.float32) == n * (n + 1) / 2).all()
+            assert (dev.to_host(wins[r], count, np.float32) == n * (n + 1) / 2).all()
+        i = np.arange(count)
+        for r in range(n):
+            dev.upload(wins[r], ((i % 10) + r).astype(np.float32))
+        N.check(g.custom_all_reduce(wins, dr, count, N.DT_FP32, N.OP_SUM, stream))
+        dev.stream_sync(stream)
+        want = (n * (i % 10) + n * (n - 1) // 2).astype(np.float32)
+        for r in range(n):
+            got = dev.to_host(dr[r], count, np.float32)
+            rel = np.abs(got.astype(np.float64) - want) / np.maximum(np.abs(want.astype(np.float64)), 1e-10)
+            assert rel.max() <= 1e-5 and np.array_equal(got, want)
+
+
 def test_group_misuse_is_reported(dev, stream):
     with DevBufs(dev) as b, S.SimGroup(2) as g:
         p = b.alloc(64)

@@ -513,6 +513,24 @@ def test_ring_allreduce_closed_forms(n):
     assert (np.abs(got - want) / np.maximum(np.abs(want), 1e-10)).max() <= 1e-5 and np.array_equal(got, want.astype(np.float32))
 
 
+@pytest.mark.parametrize("n", [1, 2, 3, 8])
+def test_reference_data_file_identical_inputs(n):
+    """test/unittest/main.cpp:15-58: every rank sends i % 10, the all-reduced sum
+    divided by the rank count is the input again; the suite's data file
+    (test/unittest/baseline_result.txt, 1000 values) is that pattern."""
+    import os
+    fixture = np.loadtxt(os.path.join(os.path.dirname(__file__), "golden", "reference_baseline_result.txt"),
+                         dtype=np.float32)
+    assert fixture.shape == (1000,)
+    sends = [fixture.copy() for _ in range(n)]
+    for recv in O.ring_allreduce(sends, F32, SUM):
+        assert np.array_equal(recv / n, fixture)
+    assert np.array_equal(O.reduce_copy(sends, F32, SUM) / n, fixture)
+    assert np.array_equal(O.reduce_copy(sends, F32, 4), fixture)      # 4 = flagcxAvg
+    if n > 1:
+        assert np.array_equal(O.bootstrap_allreduce(sends, F32, SUM)[0] / n, fixture)
+
+
 def test_ring_allreduce_order_is_the_rotated_left_fold():
     """Chunk c of a ring allreduce equals the k-way fold starting at rank c."""
     rng = np.random.default_rng(6)

@@ -125,6 +125,63 @@ def test_reducing_collectives_closed_forms(dev, ccl, stream):
     destroy(ccl, comms)
 
 
+@pytest.mark.parametrize("n", [2, 8])
+def test_legacy_suite_identical_inputs(dev, ccl, stream, n):
+    """The reference's first collective suite (test/unittest/main.cpp:15-310): every
+    rank sends the pattern i % 10 as fp32 and the result, divided by the number of
+    ranks where it is a sum, is the pattern again.  The pattern's first 1000 values
+    are the data file that suite ships (test/unittest/baseline_result.txt, kept
+    here as tests/golden/reference_baseline_result.txt)."""
+    import os
+    fixture = np.loadtxt(os.path.join(os.path.dirname(__file__), "golden", "reference_baseline_result.txt"),
+                         dtype=np.float32)
+    count = 1000 * n
+    i = np.arange(count)
+    pattern = (i % 10).astype(np.float32)
+    assert fixture.shape == (1000,) and np.array_equal(pattern[:1000], fixture)
+    comms, _ = make_comms(ccl, n)
+    call = lambda f, *a: [f(*[x[r] if isinstance(x, list) else x for x in a], comms[r], stream) for r in range(n)]
+    with DevBufs(dev) as b:
+        ds = [b.put(pattern) for _ in range(n)]
+        dr = [b.alloc(count * 4) for _ in range(n)]
+        get = lambda r, cnt=count: dev.to_host(dr[r], cnt, np.float32)
+        assert set(call(ccl.allReduce, ds, dr, count, N.DT_FP32, N.OP_SUM)) == {OK}          # :15-58
+        dev.stream_sync(stream)
+        for r in range(n):
+            assert np.array_equal(get(r) / n, pattern) and np.array_equal((get(r) / n)[:1000], fixture)
+        assert set(call(ccl.allReduce, ds, dr, count, N.DT_FP32, N.OP_AVG)) == {OK}          # the division done by the op
+        dev.stream_sync(stream)
+        assert np.array_equal(get(n - 1)[:1000], fixture)
+        sc = count // n
+        assert set(call(ccl.allGather, ds, dr, sc, N.DT_FP32)) == {OK}                       # :60-102
+        dev.stream_sync(stream)
+        for r in range(n):                               # sc is a multiple of 10, so the gathered blocks continue the pattern
+            assert np.array_equal(get(r), pattern)
+        assert set(call(ccl.reduceScatter, ds, dr, sc, N.DT_FP32, N.OP_SUM)) == {OK}         # :104-146
+        dev.stream_sync(stream)
+        for r in range(n):
+            assert np.array_equal(get(r, sc) / n, pattern[r * sc:(r + 1) * sc])
+        dev.memset(dr[0], 0, count * 4)
+        assert set(call(ccl.reduce, ds, dr, count, N.DT_FP32, N.OP_SUM, 0)) == {OK}          # :148-190
+        dev.stream_sync(stream)
+        assert np.array_equal(get(0) / n, pattern)
+        dev.memset(dr[0], 0, count * 4)
+        assert set(call(ccl.gather, ds, dr, sc, N.DT_FP32, 0)) == {OK}                       # :192-234
+        dev.stream_sync(stream)
+        assert np.array_equal(get(0), pattern)
+        dev.upload(ds[0], i.astype(np.float32))                                              # :236-277: root sends 0, 1, 2, ...
+        assert set(call(ccl.scatter, ds, dr, sc, N.DT_FP32, 0)) == {OK}
+        dev.stream_sync(stream)
+        for r in range(n):
+            assert np.array_equal(get(r, sc), i[r * sc:(r + 1) * sc].astype(np.float32))
+        dev.upload(ds[0], pattern)
+        assert set(call(ccl.broadcast, ds, dr, count, N.DT_FP32, 0)) == {OK}                 # :279-310
+        dev.stream_sync(stream)
+        for r in range(n):
+            assert np.array_equal(get(r), pattern)
+    destroy(ccl, comms)
+
+
 def test_byte_moving_collectives(dev, ccl, stream):
     n, count = 4, 70001
     comms, _ = make_comms(ccl, n)

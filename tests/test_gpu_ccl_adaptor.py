@@ -197,12 +197,12 @@ def test_byte_moving_collectives(dev, ccl, stream):
         want = np.concatenate([a[:count] for a in blocks])
         for r in range(n):
             assert np.array_equal(dev.to_host(dr[r], n * count, np.uint32), want)
-        # broadcast from root 2
+        # broadcast (coll_broadcast.cpp:9-35 uses root 0; here root 2)
         assert set(call(ccl.broadcast, ds, dr, count, N.DT_FP32, 2)) == {OK}
         dev.stream_sync(stream)
         for r in range(n):
             assert np.array_equal(dev.to_host(dr[r], count, np.uint32), blocks[2][:count])
-        # gather to root 1; scatter from root 3
+        # gather (coll_gather.cpp:10-37: chunk r on the root is rank r's data) to root 1; scatter (coll_scatter.cpp:12-38) from root 3
         assert set(call(ccl.gather, ds, dr, count, N.DT_FP32, 1)) == {OK}
         dev.stream_sync(stream)
         assert np.array_equal(dev.to_host(dr[1], n * count, np.uint32), want)
@@ -232,7 +232,7 @@ def test_send_recv_pairs(dev, ccl, stream):
     with DevBufs(dev) as b:
         ds = [b.put(a) for a in data]
         dr = [b.alloc(count * 4) for _ in range(n)]
-        # ring shift: rank r sends to r+1; receives posted first for one pair, sends first for the others
+        # ring shift as coll_sendrecv.cpp:12-31: rank r sends to r+1; receives posted first for one pair, sends first for the others
         assert ccl.recv(dr[1], count, N.DT_FP32, 0, comms[1], s2) == OK
         for r in range(n):
             assert ccl.send(ds[r], count, N.DT_FP32, (r + 1) % n, comms[r], stream) == OK

@@ -17,6 +17,7 @@ DT_FP16, DT_FP32, DT_FP64, DT_BF16 = 6, 7, 8, 9
 OP_SUM, OP_PROD, OP_MAX, OP_MIN, OP_AVG = 0, 1, 2, 3, 4
 MEMCPY_H2D, MEMCPY_D2H, MEMCPY_D2D = 0, 1, 2
 MEM_HOST, MEM_DEVICE, MEM_MANAGED = 0, 1, 2
+STATIC_MAX_SLICES = 1024   # FX_STATIC_MAX_SLICES of include/flagcx_amd/fx_kernels.h
 
 DTYPE_SIZE = {DT_INT8: 1, DT_UINT8: 1, DT_INT32: 4, DT_UINT32: 4, DT_INT64: 8, DT_UINT64: 8,
               DT_FP16: 2, DT_FP32: 4, DT_FP64: 8, DT_BF16: 2}
@@ -72,6 +73,7 @@ _SIGS = {
     "fx_plan_create": (_i, [C.POINTER(_vp), C.POINTER(SliceDesc), _sz, _i, _i, _i]),
     "fx_plan_launch": (_i, [_vp, _vp]),
     "fx_plan_destroy": (_i, [_vp]),
+    "fx_reduce_slices_static": (_i, [C.POINTER(SliceDesc), _sz, _i, _i, _i, _vp]),
     "fx_pack": (_i, [_vp, _vp, C.POINTER(_sz), C.POINTER(_sz), _i, _i, _vp]),
     "fx_unpack": (_i, [_vp, _vp, C.POINTER(_sz), C.POINTER(_sz), _i, _i, _vp]),
     "fx_fifo_bytes": (_sz, [_sz]),

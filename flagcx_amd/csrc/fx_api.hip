@@ -119,6 +119,84 @@ int copyGranularity(const fxSliceDesc *slices, size_t n) {
   return (bits & 1) ? 1 : ((bits & 2) ? 2 : 4);
 }
 
+
+// ---------------------------------------------- table in static device memory
+
+// Descriptor table and tile-prefix table of fx_reduce_slices_static: the same
+// two arrays a plan keeps in allocated device memory, here in a file-scope
+// array so that the call path allocates nothing.  Every GPU holds its own copy
+// of the array, at its own address, until the process ends.
+constexpr size_t kStaticSlices = FX_STATIC_MAX_SLICES;
+constexpr size_t kStaticDescBytes = kStaticSlices * sizeof(SliceDescDev);
+constexpr size_t kStaticBytes = kStaticDescBytes + (kStaticSlices + 1) * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[(kStaticBytes + 255) / 256 * 256];
+
+// Descriptors travel to the table in the argument block of a small kernel
+// (an upload from pageable host memory would stage through the runtime's own
+// buffers and could not be captured).
+constexpr int kWriterSlots = 32;
+struct TableChunk {
+  SliceDescDev d[kWriterSlots];
+  uint32_t tileStart[kWriterSlots];  // first workgroup of descriptor base + i
+  uint32_t base, n, gridEnd;         // gridEnd = tileStart of the entry after this chunk
+};
+
+__global__ void __launch_bounds__(kBlock) writeSliceTable(TableChunk c, SliceDescDev *d, uint32_t *tileStart) {
+  constexpr uint32_t kWords = sizeof(SliceDescDev) / sizeof(uint64_t);
+  const uint64_t *src = reinterpret_cast<const uint64_t *>(c.d);
+  uint64_t *dst = reinterpret_cast<uint64_t *>(d + c.base);
+  for (uint32_t w = threadIdx.x; w < c.n * kWords; w += kBlock) dst[w] = src[w];
+  for (uint32_t i = threadIdx.x; i < c.n; i += kBlock) tileStart[c.base + i] = c.tileStart[i];
+  if (threadIdx.x == 0) tileStart[c.base + c.n] = c.gridEnd;   // the next chunk overwrites it with the same value
+}
+
+constexpr int kMaxDevices = 64;
+unsigned char *g_scratchOf[kMaxDevices];  // device address of `scratch` per GPU, filled on first use
+
+// Address of this GPU's copy of `scratch`.  In host code the array's name is
+// only a handle for the runtime; the address kernels and copies need comes from
+// hipGetSymbolAddress, asked once per device with that device current.
+flagcxResult_t staticTable(unsigned char **ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return flagcxUnhandledDeviceError;
+  unsigned char *p = __atomic_load_n(&g_scratchOf[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    if (hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return flagcxUnhandledDeviceError;
+    __atomic_store_n(&g_scratchOf[dev], p, __ATOMIC_RELEASE);   // racing first calls store the same value
+  }
+  *ptr = p;
+  return flagcxSuccess;
+}
+
+// Walk the descriptors the way launchSliceBatches / fx_plan_create see them:
+// empty ones dropped, counts divided by `div` (copies count bytes), runs that
+// continue each other in every stream merged.  emit(desc) is called once per
+// merged descriptor; a non-zero return stops the walk and is handed back.
+template <class F>
+int forEachMerged(const fxSliceDesc *slices, size_t n, int k, size_t es, uint64_t div, F emit) {
+  fxSliceDesc cur;
+  bool have = false;
+  for (size_t i = 0; i < n; i++) {
+    fxSliceDesc d = slices[i];
+    d.count /= div;
+    if (d.count == 0) continue;
+    if (have) {
+      const size_t bytes = cur.count * es;
+      bool cont = (const char *)d.out == (const char *)cur.out + bytes;
+      for (int p = 0; p < k && cont; p++) cont = (const char *)d.in[p] == (const char *)cur.in[p] + bytes;
+      if (cont) {
+        cur.count += d.count;
+        continue;
+      }
+      const int rc = emit(cur);
+      if (rc) return rc;
+    }
+    cur = d;
+    have = true;
+  }
+  return have ? emit(cur) : 0;
+}
+
 }  // namespace
 
 struct fxPlan {
@@ -426,6 +504,85 @@ int fx_plan_destroy(fxPlan_t plan) {
   if (plan->dTileStart) (void)hipFree(plan->dTileStart);
   delete plan;
   return flagcxSuccess;
+}
+
+int fx_reduce_slices_static(const fxSliceDesc *slices, size_t n, int k, int dtype, int op, void *stream) {
+  const KernelSet *ks;
+  uint64_t div = 1;
+  if (n && !slices) return flagcxInvalidArgument;
+  if (op == -1) {
+    k = 1;
+    for (size_t i = 0; i < n; i++)
+      if (slices[i].count && (!slices[i].in[0] || !slices[i].out)) return flagcxInvalidArgument;
+    const int es = copyGranularity(slices, n);
+    ks = copySetFor(es);
+    div = (uint64_t)es;
+  } else {
+    flagcxResult_t rc = screen(dtype, op);
+    if (rc != flagcxSuccess) return rc;
+    if (k < 1 || k > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
+    ks = setFor(dtype, op);
+  }
+  if (n == 0) return flagcxSuccess;
+  for (size_t i = 0; i < n; i++)
+    if (slices[i].count) {
+      if (!slices[i].out) return flagcxInvalidArgument;
+      for (int p = 0; p < k; p++)
+        if (!slices[i].in[p]) return flagcxInvalidArgument;
+    }
+  const int U = unrollFor(k);
+  const size_t es = (size_t)ks->elemSize;
+  // first walk: validate everything and size the table, so that an error leaves nothing enqueued
+  size_t entries = 0;
+  uint64_t grid = 0;
+  int rc = forEachMerged(slices, n, k, es, div, [&](const fxSliceDesc &d) -> int {
+    uint64_t t = 0;
+    const flagcxResult_t r = sliceTiles(d, k, (int)es, U, &t);
+    if (r != flagcxSuccess) return r;
+    if (t == 0) return 0;
+    entries++;
+    grid += t;
+    return (grid > 0x7ffffff0ull) ? (int)flagcxInvalidArgument : 0;
+  });
+  if (rc) return rc;
+  if (entries == 0) return flagcxSuccess;
+  if (entries > kStaticSlices) return flagcxInvalidArgument;   // more descriptors than the static table holds
+  unsigned char *base = nullptr;
+  flagcxResult_t st = staticTable(&base);
+  if (st != flagcxSuccess) return st;
+  SliceDescDev *dDesc = reinterpret_cast<SliceDescDev *>(base);
+  uint32_t *dTileStart = reinterpret_cast<uint32_t *>(base + kStaticDescBytes);
+  hipStream_t s = (hipStream_t)stream;
+  // second walk: fill the table chunk by chunk on the caller's stream
+  TableChunk c;
+  c.base = 0;
+  c.n = 0;
+  uint32_t next = 0;   // tileStart of the descriptor being added
+  auto flush = [&]() -> int {
+    if (c.n == 0) return 0;
+    c.gridEnd = next;
+    const flagcxResult_t r = launchKernel(writeSliceTable, 1, s, c, dDesc, dTileStart);
+    c.base += c.n;
+    c.n = 0;
+    return r;
+  };
+  rc = forEachMerged(slices, n, k, es, div, [&](const fxSliceDesc &d) -> int {
+    uint64_t t = 0;
+    (void)sliceTiles(d, k, (int)es, U, &t);
+    if (t == 0) return 0;
+    SliceDescDev &o = c.d[c.n];
+    for (int p = 0; p < kMaxFixedK; p++) o.in[p] = (p < k) ? d.in[p] : nullptr;
+    o.out = d.out;
+    o.count = d.count;
+    c.tileStart[c.n] = next;
+    next += (uint32_t)t;
+    c.n++;
+    return (c.n == (uint32_t)kWriterSlots) ? flush() : 0;
+  });
+  if (rc) return rc;
+  rc = flush();
+  if (rc) return rc;
+  return ks->slicesTable[k](dDesc, dTileStart, (uint32_t)entries, next, s);
 }
 
 static int packOrUnpack(bool pack, void *a, const void *b, const size_t *counts, const size_t *displs, int npeers,

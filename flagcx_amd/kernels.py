@@ -71,6 +71,12 @@ class Plan:
             self.h = C.c_void_p()
 
 
+def reduce_slices_static(descs, k, dtype, op, stream=None):
+    """fx_plan_create + fx_plan_launch without any allocation; op = -1 copies (count in bytes)."""
+    arr, n = make_slices(descs)
+    return lib.fx_reduce_slices_static(arr, n, k, dtype, op, stream)
+
+
 def make_trigger(in1, in2, out, count, nthreads, dtype, op, state=N.SUCCESS + 1):
     t = N.ReduceTrigger()
     lib.fx_trigger_set(C.byref(t), in1, in2, out, count, nthreads, dtype, op, state)

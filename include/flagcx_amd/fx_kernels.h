@@ -199,6 +199,28 @@ int fx_plan_launch(fxPlan_t plan, void *stream);
 int fx_plan_destroy(fxPlan_t plan);
 
 /*
+ * fx_plan_create + fx_plan_launch in one call that allocates nothing.  It has
+ * no counterpart in the reference: it is for callers that cannot allocate
+ * device memory at the call (code inside a HIP graph capture, tight serving
+ * loops, harnesses that forbid it).  The descriptor table and the tile-prefix
+ * table, which a plan keeps in memory it allocates, live in a static device
+ * array of FX_STATIC_MAX_SLICES descriptors (about 84 KiB per GPU, held until
+ * the process ends); the table is filled on `stream` by small kernels whose
+ * arguments carry the descriptors, then the same kernel as fx_plan_launch
+ * runs.  Same arguments, merging of adjacent slices and results as
+ * fx_plan_create (op = -1: copy, count in bytes).  More than
+ * FX_STATIC_MAX_SLICES descriptors after merging -> flagcxInvalidArgument (4)
+ * and nothing is enqueued.  All calls on one GPU share the one table: a call
+ * may be enqueued only when the previous call's kernels on that GPU are
+ * ordered before it (same stream, or an event between the streams);
+ * overlapping calls race.  The first call on a GPU looks the array's address
+ * up once (make it outside a capture).
+ */
+#define FX_STATIC_MAX_SLICES 1024
+int fx_reduce_slices_static(const fxSliceDesc *slices, size_t n, int k,
+                            int dtype, int op, void *stream);
+
+/*
  * alltoallv pack: gather npeers segments of sendbuff (element displacements
  * sdispls[i], element counts sendcounts[i]; host arrays) into contiguous
  * slots of `packed`, slot_i = sum_{j<i} sendcounts[j].  unpack is the inverse

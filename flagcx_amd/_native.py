@@ -5,7 +5,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_DIR = os.path.join(_HERE, "lib")
+# FLAGCX_AMD_LIB_DIR points at another build of the libraries (A/B measurements)
+LIB_DIR = os.environ.get("FLAGCX_AMD_LIB_DIR") or os.path.join(_HERE, "lib")
 KERNEL_LIB = os.path.join(LIB_DIR, "libflagcx_amd.so")
 PLUGIN_LIB = os.path.join(LIB_DIR, "libflagcx-device-mi355x.so")
 

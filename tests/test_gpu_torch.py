@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def test_torch_tensors_through_the_wrapper(dev):
+def test_torch_tensors_and_streams(dev):
     if importlib.util.find_spec("torch") is None:      # looked up, not imported: torch stays out of this process
         pytest.skip("torch is not installed")
     env = dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", ""))

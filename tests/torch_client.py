@@ -20,7 +20,7 @@ from torch.distributed import ReduceOp
 
 from flagcx_amd import _native as N
 from flagcx_amd import kernels as K
-from flagcx_amd.wrapper import FLAGCXLibrary, flagcxDataTypeEnum as DT, flagcxRedOpTypeEnum as OP
+from flagcx_amd import comm
 from oracle import fx_oracle as O
 
 BITS = {torch.bfloat16: torch.int16, torch.float16: torch.int16, torch.float32: torch.int32, torch.int32: torch.int32,
@@ -29,7 +29,7 @@ BITS = {torch.bfloat16: torch.int16, torch.float16: torch.int16, torch.float32: 
 
 def host_words(t):
     """The tensor's bytes as the numpy array the oracle takes for its dtype."""
-    dt = DT.from_torch(t.dtype)
+    dt = comm.dtype_code(t.dtype)
     raw = t.detach().contiguous().view(BITS[t.dtype]).cpu().numpy()
     return raw.view(N.NP_DTYPE[dt])
 
@@ -53,12 +53,10 @@ def main():
     assert torch.cuda.is_available(), "no GPU visible to torch"
     torch.cuda.set_device(0)
     gen = torch.Generator(device="cuda").manual_seed(11)
-    fx = FLAGCXLibrary()
     with open("/proc/self/maps") as f:
         print("HIP runtime in this process:", sorted({ln.split()[-1] for ln in f if "libamdhip64" in ln}), flush=True)
     nranks = 4
-    uid = fx.flagcxGetUniqueId()
-    comms = [fx.flagcxCommInitRank(nranks, uid, r) for r in range(nranks)]
+    ranks = comm.join(nranks)
     side = torch.cuda.Stream()
 
     # ---- the kernel layer on raw torch pointers and torch's current stream ----
@@ -66,7 +64,7 @@ def main():
         n = 1_000_003
         ins = [make(dtype, n, gen) for _ in range(5)]
         out = torch.empty_like(ins[0])
-        dt, rop = DT.from_torch(dtype), OP.from_torch(op)
+        dt, rop = comm.dtype_code(dtype), comm.op_code(op)
         print(f"run reduce_copy {dtype} {op} n={n}", flush=True)
         rc = K.reduce_copy(out.data_ptr(), [t.data_ptr() for t in ins], n, dt, rop, 0,
                            torch.cuda.current_stream().cuda_stream)
@@ -81,17 +79,17 @@ def main():
         n = 262_147
         sends = [make(dtype, n, gen) for _ in range(nranks)]
         recvs = [torch.empty_like(s) for s in sends]
-        dt, rop = DT.from_torch(dtype), OP.from_torch(op)
+        dt, rop = comm.dtype_code(dtype), comm.op_code(op)
         print(f"run allreduce {dtype} {op} n={n}", flush=True)
         stream.wait_stream(torch.cuda.current_stream())          # the fills above ran on the current stream
-        fs = fx.adaptor_stream_copy(stream)
+        fs = comm.borrow_stream(stream)
         for r in range(nranks):
-            fx.flagcxAllReduce(sends[r].data_ptr(), recvs[r].data_ptr(), n, dt, rop, comms[r], fs)
+            ranks[r].all_reduce(sends[r].data_ptr(), recvs[r].data_ptr(), n, dt, rop, fs)
         torch.cuda.current_stream().wait_stream(stream)
         want = O.reduce_copy([host_words(s) for s in sends], dt, rop)
         for r in range(nranks):
             check(host_words(recvs[r]), want, f"allreduce {dtype} {op} rank {r}")
-        fx.adaptor_stream_free(fs)
+        comm.return_stream(fs)
 
     # in place, then reduce-scatter + all-gather give the same words as the all-reduce
     n = nranks * 65_536
@@ -99,21 +97,21 @@ def main():
     want = O.reduce_copy([host_words(s) for s in sends], N.DT_BF16, N.OP_SUM)
     parts = [torch.empty(n // nranks, device="cuda", dtype=torch.bfloat16) for _ in range(nranks)]
     full = [torch.empty(n, device="cuda", dtype=torch.bfloat16) for _ in range(nranks)]
-    fs = fx.adaptor_stream_copy(torch.cuda.current_stream())
+    fs = comm.borrow_stream(torch.cuda.current_stream())
     print("run reducescatter + allgather bf16", flush=True)
     for r in range(nranks):
-        fx.flagcxReduceScatter(sends[r].data_ptr(), parts[r].data_ptr(), n // nranks, N.DT_BF16, N.OP_SUM, comms[r], fs)
+        ranks[r].reduce_scatter(sends[r].data_ptr(), parts[r].data_ptr(), n // nranks, N.DT_BF16, N.OP_SUM, fs)
     for r in range(nranks):
-        fx.flagcxAllGather(parts[r].data_ptr(), full[r].data_ptr(), n // nranks, N.DT_BF16, comms[r], fs)
+        ranks[r].all_gather(parts[r].data_ptr(), full[r].data_ptr(), n // nranks, N.DT_BF16, fs)
     for r in range(nranks):
-        fx.flagcxAllReduce(sends[r].data_ptr(), sends[r].data_ptr(), n, N.DT_BF16, N.OP_SUM, comms[r], fs)
+        ranks[r].all_reduce(sends[r].data_ptr(), sends[r].data_ptr(), n, N.DT_BF16, N.OP_SUM, fs)
     torch.cuda.synchronize()
     for r in range(nranks):
         check(host_words(full[r]), want, f"reducescatter+allgather rank {r}")
         check(host_words(sends[r]), want, f"allreduce in place rank {r}")
-    fx.adaptor_stream_free(fs)
-    for c in comms:
-        fx.flagcxCommDestroy(c)
+    comm.return_stream(fs)
+    for r in ranks:
+        r.close()
     print("torch client ok", flush=True)
 
 

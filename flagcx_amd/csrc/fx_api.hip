@@ -402,7 +402,7 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
         }
         continue;
       }
-      const uint64_t tiles = tilesFor(d.out[0], d.in, k, d.count, es, U);
+      const uint64_t tiles = tilesFor(d.out[0], d.in, k, d.count, es, U, d.out + 1, nout - 1);
       if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
       BcastDescDev dd;
       for (int p = 0; p < kMaxFixedK; p++) dd.in[p] = (p < k) ? d.in[p] : nullptr;

@@ -146,8 +146,8 @@ __device__ __forceinline__ Share shareOf(uint64_t seq, const void *in1, const vo
   const int es = (int)dtypeSize(dtype);
   uint64_t tiles = 1;
   if (es != 0 && count != 0 && op >= flagcxSum && op <= flagcxAvg) {
-    const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
-    const bool co = (((uint64_t)(uintptr_t)in1 & 15u) == mis) && (((uint64_t)(uintptr_t)in2 & 15u) == mis);
+    const bool co = sameLinePhase((uint64_t)(uintptr_t)in1, (uint64_t)(uintptr_t)out) &&
+                    sameLinePhase((uint64_t)(uintptr_t)in2, (uint64_t)(uintptr_t)out);
     tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, co).tiles();
     if (tiles == 0) tiles = 1;
   }

@@ -29,9 +29,10 @@ struct KernelSet {
 };
 
 // Tiles (workgroups) a segment of `count` elements needs with unroll U.
-inline uint64_t tilesFor(const void *out, const void *const *in, int k, uint64_t count, int es, int U) {
+inline uint64_t tilesFor(const void *out, const void *const *in, int k, uint64_t count, int es, int U,
+                         void *const *more = nullptr, int nmore = 0) {
   if (count == 0) return 0;
-  return planTiles((uint64_t)(uintptr_t)out, count, es, U, coAlignedHost(out, in, k)).tiles();
+  return planTiles((uint64_t)(uintptr_t)out, count, es, U, coAlignedHost(out, in, k, more, nmore)).tiles();
 }
 
 template <class R, int K, int U>

@@ -390,9 +390,10 @@ struct CopyRed {
 // The same bytes moved as 512-byte pieces 32 KiB apart reach 6.4-6.5 TB/s.  So
 // the part of a segment that consists of whole regions of kStripeTiles tiles,
 // aligned in ABSOLUTE address, is handed out striped when every input shares
-// the output's alignment within 16 bytes (an input that does not would have a
-// cache line straddle every 512-byte piece, fetched by two workgroups; measured,
-// such segments do better contiguous: 6.1-6.5 against 5.5-6.0 TB/s): tile i of a region owns
+// the output's position within a 128-byte cache line (an input that does not
+// would have a line straddle every 512-byte piece, fetched by two workgroups:
+// counter-measured 1.22-1.25 x the bytes for an input 16 bytes off, and 5.5-6.0
+// against 6.1-6.5 TB/s contiguous): tile i of a region owns
 // piece i of every 32 KiB row of that region.  The rest (head before the first
 // region boundary, tail after the last) is handed out contiguously.
 constexpr uint32_t kPieceVecs = 32;                           // 512 bytes
@@ -404,6 +405,10 @@ constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;      // 32 KiB
 // Segments shorter than this (output bytes) stay contiguous: with few
 // workgroups in flight the striped hand-out only adds latency.
 constexpr uint64_t kStripeMinBytes = FX_STRIPE_MIN_BYTES;
+
+// Streams a and b sit at the same offset within a cache line.
+constexpr uint64_t kLineBytes = 128;
+__host__ __device__ inline bool sameLinePhase(uint64_t a, uint64_t b) { return ((a ^ b) & (kLineBytes - 1)) == 0; }
 
 struct TilePlan {
   uint64_t nv;                 // vectors spanned by the segment
@@ -703,16 +708,18 @@ __device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uin
 }
 
 // Build the output-anchored segment from raw element pointers.
+// `co` carries what the caller already knows about further streams (the extra
+// outputs of a multi-output segment).
 template <int ES, int U, int K>
-__device__ __forceinline__ TilePlan makeSeg(Seg<K> &sg, const void *const *in, void *out, uint64_t count, int) {
+__device__ __forceinline__ TilePlan makeSeg(Seg<K> &sg, const void *const *in, void *out, uint64_t count, int,
+                                            bool co = true) {
   const uint64_t mis = (uint64_t)(uintptr_t)out & 15u;
   sg.out = asGlobal(out) - mis;
   sg.lead = mis / ES;
   sg.end = sg.lead + count;
-  bool co = true;
 #pragma unroll
   for (int p = 0; p < K; p++) {
-    co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
+    co = co && sameLinePhase((uint64_t)(uintptr_t)in[p], (uint64_t)(uintptr_t)out);
     sg.in[p] = asGlobal(in[p]) - mis;
   }
   return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
@@ -728,15 +735,16 @@ __device__ __forceinline__ TilePlan makeSeg(Seg<0> &sg, const void *const *in, v
   sg.end = sg.lead + count;
   sg.k = k;
   bool co = true;
-  for (int p = 0; p < k; p++) co = co && (((uint64_t)(uintptr_t)in[p] & 15u) == mis);
+  for (int p = 0; p < k; p++) co = co && sameLinePhase((uint64_t)(uintptr_t)in[p], (uint64_t)(uintptr_t)out);
   return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
 }
 
-// Host twin of the co-alignment test above.
-inline bool coAlignedHost(const void *out, const void *const *in, int k) {
-  const uintptr_t mis = (uintptr_t)out & 15u;
+// Host twin of the co-alignment test above; `more` are further outputs.
+inline bool coAlignedHost(const void *out, const void *const *in, int k, void *const *more = nullptr, int nmore = 0) {
   for (int p = 0; p < k; p++)
-    if (((uintptr_t)in[p] & 15u) != mis) return false;
+    if (!sameLinePhase((uint64_t)(uintptr_t)in[p], (uint64_t)(uintptr_t)out)) return false;
+  for (int o = 0; o < nmore; o++)
+    if (!sameLinePhase((uint64_t)(uintptr_t)more[o], (uint64_t)(uintptr_t)out)) return false;
   return true;
 }
 
@@ -851,11 +859,15 @@ __global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable<NS>
   const uint32_t i = findSlice(t.tileStart, t.n, b);
   const BcastDescDev &d = t.d[i];
   SegB<K> sg;
-  const TilePlan tp = makeSeg<R::ES, U>(static_cast<Seg<K> &>(sg), d.in, d.out[0], d.count, K);
   const uint64_t mis = (uint64_t)(uintptr_t)d.out[0] & 15u;
   sg.nmore = (int)d.nout - 1;
+  bool co = true;   // every output at the same place in its cache line, or the striped pieces would split lines
 #pragma unroll
-  for (int o = 0; o < kMaxFixedK - 1; o++) sg.more[o] = (o < sg.nmore) ? asGlobal(d.out[o + 1]) - mis : nullptr;
+  for (int o = 0; o < kMaxFixedK - 1; o++) {
+    sg.more[o] = (o < sg.nmore) ? asGlobal(d.out[o + 1]) - mis : nullptr;
+    if (o < sg.nmore) co = co && sameLinePhase((uint64_t)(uintptr_t)d.out[o + 1], (uint64_t)(uintptr_t)d.out[0]);
+  }
+  const TilePlan tp = makeSeg<R::ES, U>(static_cast<Seg<K> &>(sg), d.in, d.out[0], d.count, K, co);
   reduceTile<R, K, U>(sg, tp, b - t.tileStart[i]);
 }
 

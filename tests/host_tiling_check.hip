@@ -8,7 +8,7 @@
 #include <cstdlib>
 #include <vector>
 
-#include "fx_reduce_body.hpp"
+#include "fx_launch.hpp"
 
 using namespace fx;
 
@@ -75,6 +75,29 @@ int main() {
                 if (rc) { printf("FAIL rc=%ld es=%d U=%d co=%d addr=%llx count=%llu\n", rc, es, U, (int)co, (unsigned long long)(base + mis), (unsigned long long)c); return 1; }
               }
           }
+  // The striping criterion: every stream at the output's offset within a 128-byte line.  16 bytes apart is
+  // not enough (a 512-byte piece of such an input would cut five lines instead of covering four).
+  {
+    char *o = (char *)0x7f0000001000ull;
+    const void *same[3] = {o + 128, o + (1 << 20), o - 4096};
+    const void *off16[3] = {o + 128, o + 16, o};
+    const void *off4[2] = {o + 4, o};
+    void *outs[2] = {o + 256, o + 64};
+    if (!coAlignedHost(o, same, 3) || coAlignedHost(o, off16, 3) || coAlignedHost(o, off4, 2) ||
+        !coAlignedHost(o, same, 3, outs, 1) || coAlignedHost(o, same, 3, outs, 2)) {
+      printf("FAIL striping criterion\n");
+      return 1;
+    }
+    const uint64_t count = (16ull << 20) / 4;
+    const void *in1[1] = {o + 16};
+    if (tilesFor(o, in1, 1, count, 4, 4) != (count * 4 + 16383) / 16384 ||          // contiguous: one tile per 16 KiB
+        planTiles((uint64_t)(uintptr_t)o, count, 4, 4, coAlignedHost(o, in1, 1)).zoneTiles != 0 ||
+        planTiles((uint64_t)(uintptr_t)o, count, 4, 4, coAlignedHost(o, same, 3)).zoneTiles == 0) {
+      printf("FAIL striping decision\n");
+      return 1;
+    }
+    cases += 8;
+  }
   printf("ok %ld cases\n", cases);
   return 0;
 }

@@ -22,19 +22,41 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
-# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs
+# HBM bytes per launch of the headline kernel come from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the same counter's reading for a
-# plain copy of known size; numbers and commands in
-# profiles/reduceCopyDirect_bf16_sum_k8_512MiB.txt.
-MEASURED_TRAFFIC_BYTES = 4_831_503_000
+# plain copy of known size.  This run does not collect counters: the figure is
+# read from the committed summary of those runs and the JSON line names it.
+TRAFFIC_SOURCE = "profiles/reduceCopyDirect_bf16_sum_k8_512MiB.txt"
+GOLDEN_JSON = os.path.join("tests", "golden", "golden.json")
+GOLDEN_KEY = "cfg5_bf16_sum_8x268435456"
 K_INPUTS = 8
 ELEMS = 268_435_456            # per input: 512 MiB of bf16
 SEED = 4                       # values N(0, 0.02)
 
 
-def cfg1(args):
+def carried_traffic():
+    """(bytes per launch, source) from the line 'traffic per launch = N B' of the
+    profile summary, or (None, None) when the summary is not there."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_SOURCE)).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic per launch = ([0-9,]+) B", text)
+    return (int(m.group(1).replace(",", "")), TRAFFIC_SOURCE) if m else (None, None)
+
+
+def golden_digest():
+    try:
+        return json.load(open(os.path.join(ROOT, GOLDEN_JSON)))[GOLDEN_KEY]["out_sha256"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def cfg1(args, dev=None):
     """BASELINE.json configs[0]: out = a + b, fp32, 16,777,216 elements, uniform[-1,1)
-    seed 0 -- on the GPU and, as the reference runs it, as one scalar host loop."""
+    seed 0 -- on the GPU and, as the reference runs it, as one scalar host loop.
+    Returns the result object."""
     import numpy as np
 
     from flagcx_amd import _native as N
@@ -42,7 +64,7 @@ def cfg1(args):
     from flagcx_amd.adaptor import Device
 
     n, k = 16_777_216, 2
-    dev = Device(0)
+    dev = dev or Device(0)
     threads = min(16, len(os.sched_getaffinity(0)))
     host = [K.synth(n, N.DT_FP32, K.SYNTH_UNIFORM, -1.0, 1.0, 0, p, threads) for p in range(k)]
     dins = [dev.malloc(n * 4) for _ in range(k)]
@@ -108,7 +130,22 @@ def cfg1(args):
     for p in dins + [out]:
         dev.free(p)
     dev.stream_destroy(stream)
-    print(json.dumps(result))
+    return result
+
+
+def reference_case(dev, threads):
+    """The reference's own CPU-runnable case (BASELINE configs[0]) in short form,
+    for the default line: its arithmetic on its own types -- the fp32
+    c[i] = a[i] + b[i] loop of flagcx/service/include/utils.h:697-705 -- on one
+    host core and on all of them, with the GPU launch beside it."""
+    class A:
+        steps, warmup, no_cpu_baseline = 50, 10, False
+    r = cfg1(A, dev)
+    return {"kind": "reference-semantics", "workload": r["config"]["workload"],
+            "loop": "sum<float>, flagcx/service/include/utils.h:697-705 (restated in oracle/fx_oracle.c)",
+            "cpu_GBs_1_core": r["cpu_baseline"]["value"], "cpu_GBs_all_cores": r["cpu_baseline"]["all_cores"]["value"],
+            "cores": r["cpu_baseline"]["all_cores"]["cores"], "gpu_us_per_launch": round(r["roofline"]["avg_launch_ms"] * 1e3, 2),
+            "gpu_GBs": r["roofline"]["achieved"], "bytes": r["roofline"]["bytes_per_launch"], "parity": r["parity"]}
 
 
 def cpu_baseline(ins, threads_all):
@@ -162,7 +199,11 @@ def main():
         sys.exit(2)
 
     if args.workload == "cfg1":
-        return cfg1(args)
+        r = cfg1(args)
+        print(json.dumps(r))
+        if r.get("parity") == "MISMATCH":
+            sys.exit(1)
+        return
 
     from flagcx_amd import _native as N
     from flagcx_amd import kernels as K
@@ -232,9 +273,22 @@ def main():
             dev.event_destroy(e)
         return ms
 
+    import hashlib
+
+    import numpy as np
+
+    def digest_of(dptr):
+        return hashlib.sha256(dev.to_host(dptr, ELEMS, np.uint16).view(np.uint8)).hexdigest()
+
     wall_ms, kern_ms = timed(out, args.steps, args.warmup)
     each = per_launch(out, 20)
+    # The buffer the timed launches wrote, against the committed digest of the CPU oracle's output for these inputs.
+    want = golden_digest() if args.synthetic_fill == "seeded" else None
+    parity = "not checked (no committed digest for this fill)"
+    if want is not None:
+        parity = "bit-exact" if digest_of(out) == want else "MISMATCH"
     _, inplace_ms = timed(ins[0], max(args.steps // 2, 1), 2)      # out = in[0]; destroys input 0, run last
+    traffic, traffic_source = carried_traffic()
     gbs = algo_bytes / (wall_ms * 1e-3) / 1e9
     kern_gbs = algo_bytes / (kern_ms * 1e-3) / 1e9
     result = {
@@ -249,10 +303,15 @@ def main():
                    "arithmetic": "every input widened to f32, f32 accumulate, one round-to-nearest-even to bf16",
                    "in_place_GBs": round(algo_bytes / (inplace_ms * 1e-3) / 1e9, 1)},
         "roofline": {"bound": "hbm", "achieved": round(kern_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(kern_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "frac": round(kern_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": traffic_source,
+                     "traffic_note": "counter-measured in the profiling runs of that summary, not in this run",
                      "kernel": "reduceCopyDirect<Red<bf16,sum>,8,8>", "bytes_per_launch": algo_bytes,
                      "avg_launch_ms": round(kern_ms, 4), "min_launch_ms": round(each[0], 4),
                      "median_launch_ms": round(each[len(each) // 2], 4)},
+        "parity": parity,
+        "parity_check": "sha256 of the output buffer of the timed launches == tests/golden/golden.json"
+                        f"[{GOLDEN_KEY}].out_sha256 (the CPU oracle's output for the same seeded inputs)",
     }
     for p in ins + [out]:
         dev.free(p)
@@ -261,7 +320,11 @@ def main():
         if not host_ins:         # memset-filled profiling run: generate the sample now
             host_ins = [K.synth(sample, N.DT_BF16, K.SYNTH_NORMAL, 0.0, 0.02, SEED, p, threads) for p in range(K_INPUTS)]
         result["cpu_baseline"] = cpu_baseline(host_ins, threads)
+        del host_ins
+        result["cpu_baseline"]["reference_case"] = reference_case(dev, threads)
     print(json.dumps(result))
+    if parity == "MISMATCH":
+        sys.exit(1)
 
 
 if __name__ == "__main__":

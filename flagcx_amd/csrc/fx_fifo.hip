@@ -19,12 +19,18 @@
 // pinned host ring (over PCIe) and mirrors it into device memory, where the
 // other workgroups poll it and read up to kBatch upcoming triggers per round
 // of reads.  Results are stored through the caches, so reporting in needs no
-// cache write-back.  Nothing waits on another
-// workgroup, so the kernel cannot deadlock on residency; every polling loop is
-// bounded by maxIdlePolls.  Triggers that are in the ring at the same time must
-// be independent of each other, which is how the reference's scheduler uses it
-// (a node is enqueued only after its parents completed,
-// flagcx/runner/uni_runner_impl.cc:1727-1794).
+// cache write-back.  A trigger is Complete once every workgroup that takes part
+// of it has reported in, so all workgroups of the grid must be resident at the
+// same time: the grid is never larger than what the device holds at once
+// (occupancy x compute units, see fx_fifo_consumer_create).  Every polling loop
+// is bounded by maxIdlePolls, so even a grid that lost a workgroup ends.
+// Triggers that are in the ring at the same time must be independent of each
+// other, which is how the reference's scheduler uses it (a node is enqueued
+// only after its parents completed, flagcx/runner/uni_runner_impl.cc:1727-1794)
+// -- unless the consumer was created in order (FX_FIFO_IN_ORDER=1): then one
+// trigger at a time is handed to the workers, the next only after the previous
+// one is Complete, which is the reference consumer's own serial behaviour
+// (flagcx_reduce_kernel_device.cu:104-185).
 #include <sched.h>
 
 #include <cstddef>
@@ -32,6 +38,7 @@
 #include <new>
 
 #include "flagcx_amd/fx_kernels.h"
+#include "fx_fifo_share.hpp"
 #include "fx_launch.hpp"
 
 using namespace fx;
@@ -50,7 +57,6 @@ constexpr int kBatch = 16;  // triggers a workgroup inspects per round of mirror
 // the host.
 constexpr uint64_t kBulkArrivals = 4;
 constexpr uint64_t kBulkBit = 1ull << 63;
-constexpr int kBulkShift = 3;
 constexpr uint32_t kMaxCapacity = 1024;
 constexpr uint64_t kMirrorBatch = 64;  // triggers workgroup 0 mirrors per pass
 
@@ -60,7 +66,8 @@ struct FifoMirror {              // device memory, zeroed at creation
   uint64_t completed;            // triggers fully executed
   uint64_t exitReason;           // FX_FIFO_EXIT_*
   uint64_t badTriggers;          // triggers skipped because dtype / op is not carried
-  uint64_t pad[3];
+  uint64_t startPlus1;           // 1 + the ring's `consumed` when this launch began (0: not read yet)
+  uint64_t pad[2];
   uint32_t done[kMaxCapacity];   // per slot: workgroups that finished their share
   uint64_t trig[kMaxCapacity][4];
   // Which trigger number trig[slot] holds (kNoTrigger while it is being
@@ -103,12 +110,6 @@ __device__ __forceinline__ void waitVectorMemory() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
-// Which part of a trigger a workgroup takes: tiles idx, idx + takers, ...;
-// idx >= takers means none.
-struct Share {
-  uint32_t idx, takers;
-};
-
 // This workgroup's share of one two-input trigger.
 template <int DT, int OP>
 __device__ __forceinline__ void runShare(const void *in1, const void *in2, void *out, uint64_t count, Share sh) {
@@ -132,36 +133,19 @@ __device__ __forceinline__ bool runShareOp(int op, const void *a, const void *b,
   }
 }
 
-// Who works on trigger number seq.  One workgroup per 16 KiB tile (per eight
-// tiles for a trigger that arrived in bulk, see kBulkArrivals), at least one
-// (which completes empty and unsupported triggers), at most G-1: workgroup 0
-// never computes, so it is always free to talk to the host, and the workers of
-// a small trigger start at a position that rotates with seq, so consecutive
-// small triggers run side by side on different workgroups.  Every workgroup
-// computes the same answer from the trigger words alone, so the ones left out
-// neither work nor report in.
+// Who works on trigger number seq: one workgroup per 16 KiB tile (per eight
+// tiles for a trigger that arrived in bulk, see kBulkArrivals); the rest is
+// shareFor's.
 __device__ __forceinline__ Share shareOf(uint64_t seq, const void *in1, const void *in2, void *out, uint64_t count,
                                          int dtype, int op, bool bulk) {
-  const uint32_t grid = gridDim.x;
   const int es = (int)dtypeSize(dtype);
   uint64_t tiles = 1;
   if (es != 0 && count != 0 && op >= flagcxSum && op <= flagcxAvg) {
     const bool co = sameLinePhase((uint64_t)(uintptr_t)in1, (uint64_t)(uintptr_t)out) &&
                     sameLinePhase((uint64_t)(uintptr_t)in2, (uint64_t)(uintptr_t)out);
     tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, co).tiles();
-    if (tiles == 0) tiles = 1;
   }
-  Share sh;
-  if (grid == 1) {  // a one-workgroup launch does everything itself
-    sh.takers = 1;
-    sh.idx = 0;
-    return sh;
-  }
-  const uint32_t pool = grid - 1, rot = (uint32_t)((seq * 61u) % pool);
-  if (bulk) tiles = (tiles >> kBulkShift) ? (tiles >> kBulkShift) : 1;
-  sh.takers = (uint32_t)(tiles < pool ? tiles : pool);
-  sh.idx = (blockIdx.x == 0) ? sh.takers : (blockIdx.x - 1 + pool - rot) % pool;
-  return sh;
+  return shareFor(gridDim.x, blockIdx.x, seq, tiles, bulk);
 }
 
 // Value of lane `src` of the wavefront as a wave-uniform 64-bit scalar.
@@ -178,8 +162,30 @@ __global__ void __launch_bounds__(kBlock) clearMirror(uint64_t *words, uint32_t 
 }
 
 __global__ void __launch_bounds__(kBlock)
-fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uint64_t maxIdlePolls) {
+fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint32_t inOrder, uint64_t maxIdlePolls) {
   __shared__ uint64_t sh[2];                  // [0] state, [1] triggers in this batch
+  // Where this launch starts: the ring's `consumed` as the previous consumer
+  // left it.  Read here, not on the host at enqueue time, because an earlier
+  // consumer on the same stream may still be running then.  Workgroup 0 reads it
+  // (it is also the one that overwrites it later) and passes it on through the
+  // mirror; the others wait for it, bounded like every wait here.
+  if (threadIdx.x == 0) {
+    uint64_t s1 = 0;
+    if (blockIdx.x == 0) {
+      s1 = pollSys(host + 1) + 1;
+      storeDev(&m->startPlus1, s1);
+    } else {
+      const uint64_t patience = (maxIdlePolls > (~0ull >> 5)) ? maxIdlePolls : maxIdlePolls * 32;
+      for (uint64_t spins = 0; (s1 = pollDev(&m->startPlus1)) == 0 && spins <= patience; spins++)
+        __builtin_amdgcn_s_sleep(8);
+    }
+    sh[0] = s1;
+  }
+  __syncthreads();
+  const uint64_t startPlus1 = sh[0];
+  __syncthreads();
+  if (startPlus1 == 0) return;                // workgroup 0 never showed up: nothing can be done safely
+  const uint64_t startSeq = startPlus1 - 1;
   __shared__ uint64_t shTrig[kBatch][4];     // their words
   __shared__ uint32_t shValid[kBatch];       // and whether the words are theirs (sequence lock)
   enum { kWork = 0, kExitTerminate = FX_FIFO_EXIT_TERMINATE, kExitIdle = FX_FIFO_EXIT_IDLE };
@@ -211,10 +217,11 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint64_t startSeq, uin
             const uint64_t hp = fromLane(v, 0), ht = fromLane(v, 1);
             const uint64_t c = fromLane(v, 2);
             termMirror = fromLane(v, 3);
-            if (mirrored < hp) {
+            // In order: the next trigger goes out only when everything handed out so far is complete.
+            if (mirrored < hp && (!inOrder || c == mirrored - startSeq)) {
               __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // the triggers behind `produced`
               // at most kMirrorBatch triggers per pass (four words per lane); the rest next time round
-              const uint64_t arrived = hp - mirrored;
+              const uint64_t arrived = inOrder ? 1 : hp - mirrored;
               const uint64_t upTo = mirrored + (arrived < kMirrorBatch ? arrived : kMirrorBatch);
               const uint64_t words = 4 * (upTo - mirrored);
               // Refill the slots like a sequence lock: number invalid, words, number
@@ -437,6 +444,7 @@ struct fxFifoConsumer {
   FifoMirror *mirror;
   uint32_t capacity;
   uint32_t grid;
+  uint32_t inOrder;
 };
 
 extern "C" {
@@ -550,11 +558,18 @@ int fx_fifo_consumer_create(fxFifoConsumer_t *consumer, size_t capacity) {
     return flagcxUnhandledDeviceError;
   }
   c->capacity = (uint32_t)capacity;
-  int perCu = 1;  // resident workgroups per CU
-  if (const char *e = getenv("FX_FIFO_WGS_PER_CU")) perCu = atoi(e);
-  if (perCu < 1) perCu = 1;
-  if (perCu > 8) perCu = 8;
-  c->grid = (uint32_t)((cus > 0 ? cus : 1) * perCu);
+  int resident = 0;  // workgroups of this kernel one compute unit holds at the same time
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, fifoConsumer, kBlock, 0) != hipSuccess || resident < 1) {
+    (void)hipFree(c->mirror);
+    delete c;
+    return flagcxUnhandledDeviceError;
+  }
+  long wanted = 0;
+  if (const char *e = getenv("FX_FIFO_WGS")) wanted = atol(e);
+  else if (const char *e = getenv("FX_FIFO_WGS_PER_CU")) wanted = atol(e) * (long)(cus > 0 ? cus : 1);
+  c->grid = fifoGridFor(cus, resident, wanted);
+  const char *io = getenv("FX_FIFO_IN_ORDER");
+  c->inOrder = (io && atoi(io) != 0) ? 1u : 0u;
   *consumer = c;
   return flagcxSuccess;
 }
@@ -568,10 +583,10 @@ int fx_fifo_consumer_launch(fxFifoConsumer_t c, void *fifoDevicePointer, const u
   const uint32_t words = (uint32_t)(sizeof(FifoMirror) / sizeof(uint64_t));
   flagcxResult_t rc = launchKernel(clearMirror, (words + kBlock - 1) / kBlock, s, (uint64_t *)c->mirror, words);
   if (rc != flagcxSuccess) return rc;
-  // Start where the last consumer stopped: triggers enqueued before this launch
-  // are waiting between `consumed` and `produced` and are served first.
-  const uint64_t startSeq = __atomic_load_n(&fifoHost[1], __ATOMIC_ACQUIRE);
-  rc = launchKernel(fifoConsumer, c->grid, s, (uint64_t *)fifoDevicePointer, c->mirror, c->capacity, startSeq,
+  // The kernel starts where the last consumer stopped (it reads the ring's
+  // `consumed` itself): triggers enqueued before this launch are waiting between
+  // `consumed` and `produced` and are served first.
+  rc = launchKernel(fifoConsumer, c->grid, s, (uint64_t *)fifoDevicePointer, c->mirror, c->capacity, c->inOrder,
                     (uint64_t)maxIdlePolls);
   if (rc != flagcxSuccess) return rc;
   return flagcxSuccess;
@@ -579,7 +594,7 @@ int fx_fifo_consumer_launch(fxFifoConsumer_t c, void *fifoDevicePointer, const u
 
 int fx_fifo_consumer_status(fxFifoConsumer_t c, int *exitReason, uint64_t *completed, uint64_t *badTriggers) {
   if (!c) return flagcxInvalidArgument;
-  uint64_t head[8];  // produced, terminate, completed, exitReason, badTriggers, pad
+  uint64_t head[8];  // produced, terminate, completed, exitReason, badTriggers, startPlus1, pad
   static_assert(offsetof(FifoMirror, done) == sizeof(head), "FifoMirror header layout");
   if (hipMemcpy(head, c->mirror, sizeof(head), hipMemcpyDeviceToHost) != hipSuccess) return flagcxUnhandledDeviceError;
   if (completed) *completed = head[2];

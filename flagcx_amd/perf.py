@@ -188,16 +188,17 @@ def run_fifo(dev, a):
             row("fifo round trip, fp32 sum, 2 inputs", nbytes, ms, 3 * nbytes)
             # the ring kept full: 1024 independent triggers through the library's own producer loop
             # (enqueue as slots free up, collect as they complete)
-            if 3 * nbytes * 64 <= emax * 3:
-                span = emax // (64 * 4) * 4                      # 64 disjoint windows of the buffers
+            windows = min(64, emax // nbytes)                    # disjoint windows of the buffers
+            if windows >= 2:
+                span = emax // (windows * 4) * 4
                 n = min(n, span // 4)
-                total = 1024
+                total = max(32, min(1024, (8 << 30) // (3 * nbytes)))
                 trig = (N.ReduceTrigger * total)()
                 for i in range(total):
-                    off = (i % 64) * span
+                    off = (i % windows) * span
                     lib.fx_trigger_set(C.byref(trig[i]), bufs[0] + off, bufs[1] + off, bufs[2] + off, n, 32, N.DT_FP32,
                                        N.OP_SUM, 1)
-                N.check(lib.fx_fifo_run_batch(host, trig, 64, 50_000_000))          # warm-up
+                N.check(lib.fx_fifo_run_batch(host, trig, min(64, total), 50_000_000))          # warm-up
                 t0 = time.perf_counter()
                 N.check(lib.fx_fifo_run_batch(host, trig, total, 50_000_000))
                 ms = (time.perf_counter() - t0) * 1e3 / total

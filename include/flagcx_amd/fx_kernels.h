@@ -123,12 +123,20 @@ int fx_fifo_run_batch(uint64_t *fifo, const fxReduceTrigger *triggers, size_t n,
  * polls of the host ring (one to two microseconds each; so it always ends).
  * fifoDevicePointer is hostGetDevicePointer() of the pinned ring, fifoHost
  * the ring itself.  Triggers that sit in the ring at
- * the same time must not depend on each other.  Capacity <= 1024.  The grid is
- * one workgroup per compute unit; FX_FIFO_WGS_PER_CU (environment, 1..8, read
- * at fx_fifo_consumer_create) asks for more, which measured slower.
- * A ring can be served again after its consumer has ended (the launch reads
- * `consumed` on the host to know where to resume, so the earlier kernel must
- * have finished); triggers enqueued in between are served first.
+ * the same time must not depend on each other, unless the consumer was
+ * created with FX_FIFO_IN_ORDER=1 in the environment: then one trigger at a
+ * time is executed, the next only after the previous one is Complete, as the
+ * reference's single-block consumer does, and a trigger may read what an
+ * earlier one in the ring wrote.  Capacity <= 1024.  The grid is one
+ * workgroup per compute unit (the first talks to the host, the others work) and
+ * never more workgroups than the device holds at the same time (a trigger
+ * completes when all its workgroups have reported in); FX_FIFO_WGS or
+ * FX_FIFO_WGS_PER_CU (environment, read at fx_fifo_consumer_create) ask for
+ * another size within that limit.
+ * A ring can be served again after its consumer has ended: the new kernel
+ * reads `consumed` from the ring when it starts (so it may be enqueued on the
+ * same stream while the earlier one is still running); triggers enqueued in
+ * between are served first.
  * While the consumer runs, calls that wait for the whole device (hipFree,
  * hipDeviceSynchronize) block until it has ended: set `terminate` first.
  */

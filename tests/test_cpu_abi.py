@@ -366,6 +366,25 @@ def test_kernel_index_arithmetic_on_the_host(tmp_path):
     assert out.returncode == 0 and out.stdout.startswith("ok"), out.stdout
 
 
+def test_fifo_share_arithmetic_on_the_host(tmp_path):
+    """tests/host_fifo_check.cc drives fx::fifoGridFor and fx::shareFor -- the very
+    functions the FIFO consumer uses to size its grid and to decide which
+    workgroups take which tiles of a trigger -- on the CPU: the grid never exceeds
+    what the device holds at once, every taker index has exactly one workgroup,
+    workgroup 0 computes only when it is alone."""
+    import shutil
+    import subprocess
+    gxx = shutil.which("g++")
+    if not gxx:
+        pytest.skip("no g++")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = tmp_path / "host_fifo_check"
+    subprocess.run([gxx, "-O1", "-std=c++17", f"-I{root}/flagcx_amd/csrc", f"{root}/tests/host_fifo_check.cc", "-o",
+                    str(exe)], check=True, capture_output=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.startswith("ok"), out.stdout
+
+
 def test_bench_refuses_more_than_one_gpu():
     """Nothing in this build uses a second GPU; the benchmark says so instead of
     pretending to scale."""

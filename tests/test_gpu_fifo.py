@@ -302,6 +302,46 @@ def test_long_chain_of_dependent_triggers_sees_every_previous_result(dev):
             ring.close()
 
 
+def test_in_order_consumer_runs_dependent_triggers_enqueued_back_to_back(dev, monkeypatch):
+    """FX_FIFO_IN_ORDER=1: the reference consumer's serial semantics
+    (flagcx_reduce_kernel_device.cu:104-185).  Sixty triggers, each reading what
+    the one before it wrote, are pushed through a 16-slot ring by the producer
+    loop without waiting for any of them in between; sizes alternate between one
+    tile and every workgroup of every die.  A consumer that let two of them run
+    side by side, or read a stale line, would not reproduce the sequential result."""
+    monkeypatch.setenv("FX_FIFO_IN_ORDER", "1")
+    ring = Ring(dev, capacity=16)
+    monkeypatch.delenv("FX_FIFO_IN_ORDER")
+    closed = False
+    try:
+        rng = np.random.default_rng(77)
+        n, steps = 3 << 20, 60
+        acc = rng.integers(-1000, 1000, n).astype(np.int32)
+        xs = [rng.integers(-1000, 1000, n).astype(np.int32) for _ in range(3)]
+        with DevBufs(dev) as b:
+            dacc, dalt = b.put(acc), b.put(np.zeros(n, np.int32))     # (no memset / device-wide wait while the consumer runs)
+            dxs = [b.put(x) for x in xs]
+            trig = (N.ReduceTrigger * steps)()
+            want, other = acc.copy(), np.zeros(n, np.int32)
+            src, dst, hsrc, hdst = dacc, dalt, want, other
+            for i in range(steps):
+                cnt = n if i % 3 else 4096 + i            # a short trigger in between: only its first elements move on
+                op = N.OP_SUM if i % 2 else N.OP_MAX
+                lib.fx_trigger_set(C.byref(trig[i]), src, dxs[i % 3], dst, cnt, 32, N.DT_INT32, op, ENQUEUED)
+                hdst[:cnt] = (hsrc[:cnt] + xs[i % 3][:cnt]) if op == N.OP_SUM else np.maximum(hsrc[:cnt], xs[i % 3][:cnt])
+                src, dst, hsrc, hdst = dst, src, hdst, hsrc     # ping-pong: the next one reads what this one wrote
+            N.check(lib.fx_fifo_run_batch(ring.host, trig, steps, 400_000_000))
+            reason, done, bad = ring.close()
+            closed = True
+            assert (reason, done, bad) == (1, steps, 0)
+            got = {dacc: dev.to_host(dacc, n, np.int32), dalt: dev.to_host(dalt, n, np.int32)}
+            assert np.array_equal(got[src], hsrc), "last trigger's output differs from the sequential result"
+            assert np.array_equal(got[dst], hdst), "the other buffer (second-to-last output) differs"
+    finally:
+        if not closed:
+            ring.close()
+
+
 def test_ring_allreduce_driven_through_the_fifo(dev):
     """What an unmodified uniRunner does with this consumer behind its FIFO
     (uni_runner_impl.cc:661-1007): n-1 reduce-scatter steps whose reduce nodes --

@@ -59,11 +59,14 @@ flagcxResult_t sliceTiles(const fxSliceDesc &s, int k, int es, int U, uint64_t *
 // longer slice (the operation is element-wise).  Partitions such as the
 // reference's slice / red-slice split produce long runs of them, and a long
 // segment gets the striped hand-out where 512 KiB pieces would not.
-std::vector<fxSliceDesc> mergeAdjacent(const fxSliceDesc *slices, size_t n, int k, size_t es) {
-  std::vector<fxSliceDesc> out;
+constexpr size_t kFewSlices = 16;   // descriptor lists up to this length stay on the stack
+typedef SmallVec<fxSliceDesc, kFewSlices> SliceList;
+
+void mergeAdjacent(SliceList &out, const fxSliceDesc *slices, size_t n, int k, size_t es, uint64_t div = 1) {
   out.reserve(n);
   for (size_t i = 0; i < n; i++) {
-    const fxSliceDesc &d = slices[i];
+    fxSliceDesc d = slices[i];
+    d.count /= div;          // copies are given in bytes and moved in units of `div` bytes
     if (d.count == 0) continue;
     if (!out.empty()) {
       fxSliceDesc &l = out.back();
@@ -77,20 +80,21 @@ std::vector<fxSliceDesc> mergeAdjacent(const fxSliceDesc *slices, size_t n, int 
     }
     out.push_back(d);
   }
-  return out;
 }
 
 // Launch n slices through kernel-argument tables (as many launches as the tables need).
-flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slicesIn, size_t nIn, int k, hipStream_t s) {
+flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slicesIn, size_t nIn, int k, hipStream_t s,
+                                  uint64_t div = 1) {
   for (size_t i = 0; i < nIn; i++)   // validate before merging so a bad slice is still reported
     if (slicesIn[i].count) {
       if (!slicesIn[i].out) return flagcxInvalidArgument;
       for (int p = 0; p < k; p++)
         if (!slicesIn[i].in[p]) return flagcxInvalidArgument;
     }
-  std::vector<fxSliceDesc> merged = mergeAdjacent(slicesIn, nIn, k, (size_t)ks->elemSize);
+  SliceList merged;
+  mergeAdjacent(merged, slicesIn, nIn, k, (size_t)ks->elemSize, div);
   const int U = unrollFor(k);
-  std::vector<uint32_t> tiles;
+  SmallVec<uint32_t, kFewSlices> tiles;
   tiles.reserve(merged.size());
   size_t kept = 0;
   for (size_t i = 0; i < merged.size(); i++) {
@@ -287,7 +291,7 @@ int fx_reduce_triggers(const fxReduceTrigger *triggers, size_t n, void *stream) 
   if (n == 0) return flagcxSuccess;
   if (!triggers) return flagcxInvalidArgument;
   return guarded([&]() -> int {
-    std::vector<fxSliceDesc> run;
+    SliceList run;
     size_t i = 0;
     while (i < n) {
       int dtype, op;
@@ -322,9 +326,7 @@ int fx_copy_slices(const fxSliceDesc *slices, size_t n, void *stream) {
     if (slices[i].count && (!slices[i].in[0] || !slices[i].out)) return flagcxInvalidArgument;
   return guarded([&]() -> int {
     const int es = copyGranularity(slices, n);
-    std::vector<fxSliceDesc> el(slices, slices + n);
-    for (auto &d : el) d.count /= (uint64_t)es;
-    return launchSliceBatches(copySetFor(es), el.data(), n, 1, (hipStream_t)stream);
+    return launchSliceBatches(copySetFor(es), slices, n, 1, (hipStream_t)stream, (uint64_t)es);
   });
 }
 
@@ -360,7 +362,7 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
     const KernelSet *ks = copy ? copySetFor(es) : setFor(dtype, op);
     const int U = unrollFor(k);
     // merge slices that continue each other in every stream
-    std::vector<fxBcastDesc> merged;
+    SmallVec<fxBcastDesc, kFewSlices> merged;
     merged.reserve(n);
     for (size_t i = 0; i < n; i++) {
       fxBcastDesc d = slices[i];
@@ -379,9 +381,9 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
       }
       merged.push_back(d);
     }
-    std::vector<fxSliceDesc> plainReduce, plainCopy;  // slices whose outputs are not co-aligned
-    std::vector<BcastDescDev> dev;
-    std::vector<uint32_t> devTiles;
+    SliceList plainReduce, plainCopy;  // slices whose outputs are not co-aligned
+    SmallVec<BcastDescDev, kFewSlices> dev;
+    SmallVec<uint32_t, kFewSlices> devTiles;
     for (const fxBcastDesc &d : merged) {
       bool same = true;
       for (int o = 1; o < nout; o++) same = same && (((uintptr_t)d.out[o] & 15u) == ((uintptr_t)d.out[0] & 15u));
@@ -454,7 +456,8 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
         if (d.count && !d.in[p]) return flagcxInvalidArgument;
       d.count /= div;
     }
-    const std::vector<fxSliceDesc> merged = mergeAdjacent(scaled.data(), scaled.size(), k, (size_t)ks->elemSize);
+    SliceList merged;
+    mergeAdjacent(merged, scaled.data(), scaled.size(), k, (size_t)ks->elemSize);
     for (size_t i = 0; i < merged.size(); i++) {
       fxSliceDesc s = merged[i];
       uint64_t tiles;
@@ -593,7 +596,7 @@ static int packOrUnpack(bool pack, void *a, const void *b, const size_t *counts,
   if (npeers == 0) return flagcxSuccess;
   if (!counts || !displs) return flagcxInvalidArgument;
   return guarded([&]() -> int {
-    std::vector<fxSliceDesc> sl;
+    SliceList sl;
     size_t slot = 0;
     for (int i = 0; i < npeers; i++) {
       if (counts[i]) {

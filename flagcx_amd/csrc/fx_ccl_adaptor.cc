@@ -15,10 +15,13 @@
 #include "flagcx_amd/fx_kernels.h"
 #include "flagcx_amd/fx_sim.h"
 
+constexpr int kMaxOutgrown = 128;  // two directions, each at least doubling: never reached in practice
 struct flagcxInnerComm {
   flagcxComm_t base;           // simulated-rank communicator
   void *staged[2];             // send / recv staging buffers handed out by getStagedBuffer
   size_t stagedBytes[2];
+  void *outgrown[kMaxOutgrown];  // earlier, smaller staging buffers: the caller may still hold them
+  int noutgrown;
 };
 
 namespace {
@@ -50,16 +53,22 @@ const char *cclGetErrorString(flagcxResult_t r) { return flagcxGetErrorString(r)
 
 const char *cclGetLastError(flagcxInnerComm_t) { return ""; }
 
-// Device staging buffers cached per communicator and direction; grown on demand.
+// Device staging buffers cached per communicator and direction; grown on demand
+// (at least doubling).  A buffer handed out earlier stays valid until the
+// communicator is destroyed: the caller may still hold its address, and freeing
+// it would wait for the whole device.
 flagcxResult_t cclGetStagedBuffer(const flagcxInnerComm_t comm, void **buff, size_t size, int isRecv) {
   if (!comm || !buff) return flagcxInvalidArgument;
   const int i = isRecv ? 1 : 0;
   if (comm->stagedBytes[i] < size) {
-    if (comm->staged[i]) (void)hipFree(comm->staged[i]);
-    comm->staged[i] = nullptr;
-    comm->stagedBytes[i] = 0;
-    if (hipMalloc(&comm->staged[i], size) != hipSuccess) return flagcxUnhandledDeviceError;
-    comm->stagedBytes[i] = size;
+    if (comm->staged[i] && comm->noutgrown == kMaxOutgrown) return flagcxSystemError;
+    size_t want = comm->stagedBytes[i] * 2;
+    if (want < size) want = size;
+    void *blk = nullptr;
+    if (hipMalloc(&blk, want) != hipSuccess) return flagcxUnhandledDeviceError;
+    if (comm->staged[i]) comm->outgrown[comm->noutgrown++] = comm->staged[i];
+    comm->staged[i] = blk;
+    comm->stagedBytes[i] = want;
   }
   *buff = comm->staged[i];
   return flagcxSuccess;
@@ -88,6 +97,7 @@ flagcxResult_t cclCommDestroy(flagcxInnerComm_t comm) {
   if (!comm) return flagcxInvalidArgument;
   for (int i = 0; i < 2; i++)
     if (comm->staged[i]) (void)hipFree(comm->staged[i]);
+  for (int i = 0; i < comm->noutgrown; i++) (void)hipFree(comm->outgrown[i]);
   flagcxResult_t rc = comm->base ? fxSimCommDestroy(comm->base) : flagcxSuccess;
   free(comm);
   return rc;
@@ -182,8 +192,10 @@ flagcxResult_t cclRecv(void *r, size_t count, flagcxDataType_t dt, int peer, fla
                        flagcxStream_t stream) {
   return flagcxRecv(r, count, dt, peer, FX_BASE(comm), stream);
 }
-flagcxResult_t cclGroupStart(void) { return flagcxSuccess; }
-flagcxResult_t cclGroupEnd(void) { return flagcxSuccess; }
+// The brackets are per host thread in the simulated-rank layer, which is all
+// these two can name.
+flagcxResult_t cclGroupStart(void) { return flagcxGroupStart(nullptr); }
+flagcxResult_t cclGroupEnd(void) { return flagcxGroupEnd(nullptr); }
 
 }  // namespace
 

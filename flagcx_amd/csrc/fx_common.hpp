@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <stdlib.h>
+#include <string.h>
 #include <new>
 #include <tuple>
 #include <utility>
@@ -66,6 +68,55 @@ inline int guarded(F body) noexcept {
     return flagcxInternalError;
   }
 }
+
+// Array of trivially copyable T that lives on the stack up to N elements and
+// moves to the heap beyond: the descriptor lists of a call are almost always a
+// handful (one per rank or per peer), and a heap allocation per call is a
+// measurable part of a 3 us launch.
+template <class T, size_t N>
+class SmallVec {
+ public:
+  SmallVec() : p_(inl_), n_(0), cap_(N) {}
+  ~SmallVec() {
+    if (p_ != inl_) free(p_);
+  }
+  SmallVec(const SmallVec &) = delete;
+  SmallVec &operator=(const SmallVec &) = delete;
+  void push_back(const T &v) {
+    if (n_ == cap_) reserve(cap_ * 2);
+    p_[n_++] = v;
+  }
+  void reserve(size_t want) {
+    if (want <= cap_) return;
+    T *q = static_cast<T *>(malloc(want * sizeof(T)));
+    if (!q) throw std::bad_alloc();
+    memcpy(static_cast<void *>(q), static_cast<const void *>(p_), n_ * sizeof(T));
+    if (p_ != inl_) free(p_);
+    p_ = q;
+    cap_ = want;
+  }
+  void resize(size_t n) {   // new elements are left uninitialised
+    reserve(n);
+    n_ = n;
+  }
+  void clear() { n_ = 0; }
+  bool empty() const { return n_ == 0; }
+  size_t size() const { return n_; }
+  T *data() { return p_; }
+  const T *data() const { return p_; }
+  T &operator[](size_t i) { return p_[i]; }
+  const T &operator[](size_t i) const { return p_[i]; }
+  T &back() { return p_[n_ - 1]; }
+  T *begin() { return p_; }
+  T *end() { return p_ + n_; }
+  const T *begin() const { return p_; }
+  const T *end() const { return p_ + n_; }
+
+ private:
+  T inl_[N];
+  T *p_;
+  size_t n_, cap_;
+};
 
 // 128-bit streaming accesses: every byte is touched once, so keep it out of
 // the caches' way (nontemporal).  Loads may start at any byte: gfx950 under HSA

@@ -84,9 +84,12 @@ struct Group {
   long long sync = FX_SYNC_GROUP;
   long long algo = FX_ALGO_DIRECT, order = FX_ORDER_RANK;
   long long nslices = 1, nredslices = 0, redslicesize = 65536;
-  // scratch: ring reduce-scatter partials / alltoallv staging
+  // scratch: ring reduce-scatter partials / alltoallv staging.  Outgrown
+  // blocks stay allocated until the group is destroyed: kernels enqueued earlier
+  // may still use them, and freeing would wait for the whole device.
   void *scratch = nullptr;
   size_t scratchBytes = 0;
+  std::vector<void *> outgrown;
   std::vector<void *> windows;
   size_t windowBytes = 0;
 };
@@ -104,15 +107,34 @@ inline int mod(int a, int n) { return ((a % n) + n) % n; }
 inline const char *cadd(const void *p, size_t bytes) { return (const char *)p + bytes; }
 inline char *madd(void *p, size_t bytes) { return (char *)p + bytes; }
 
-flagcxResult_t ensureScratch(Group *g, size_t bytes) {
+// Scratch of at least `bytes`.  Growing allocates a new block (at least twice
+// the old size, so the blocks kept add up to less than the last one) and
+// enqueues nothing that waits for the device.  A stream that is being captured
+// cannot allocate: the caller reserves beforehand (FX_SIM_SCRATCH_BYTES) or
+// gets flagcxInvalidUsage.
+flagcxResult_t ensureScratch(Group *g, size_t bytes, hipStream_t s) {
   if (bytes <= g->scratchBytes) return flagcxSuccess;
-  if (g->scratch) (void)hipFree(g->scratch);  // waits for the device: earlier launches are done
-  g->scratch = nullptr;
-  g->scratchBytes = 0;
-  if (hipMalloc(&g->scratch, bytes) != hipSuccess) return flagcxUnhandledDeviceError;
-  g->scratchBytes = bytes;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (s && hipStreamIsCapturing(s, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) return flagcxInvalidUsage;
+  size_t want = g->scratchBytes * 2;
+  if (want < bytes) want = bytes;
+  void *blk = nullptr;
+  if (hipMalloc(&blk, want) != hipSuccess) {
+    (void)hipGetLastError();
+    if (want == bytes || hipMalloc(&blk, bytes) != hipSuccess) return flagcxUnhandledDeviceError;
+    want = bytes;
+  }
+  if (g->scratch) g->outgrown.push_back(g->scratch);
+  g->scratch = blk;
+  g->scratchBytes = want;
   return flagcxSuccess;
 }
+
+// Descriptor lists of one collective: a handful of entries in the common case
+// (one per rank), kept on the stack.
+typedef fx::SmallVec<fxSliceDesc, 16> SliceList;
+typedef fx::SmallVec<fxBcastDesc, 16> BcastList;
+typedef fx::SmallVec<const void *, 16> PtrList;
 
 fxSliceDesc copyDesc(const void *src, void *dst, size_t bytes) {
   fxSliceDesc d;
@@ -134,7 +156,7 @@ struct Ctx {
 
 // k-way reduce of element range [off, off+cnt) of every rank's sendbuff (+sendBase
 // elements) into out, in order first, first+1, ...
-flagcxResult_t kway(const Ctx &c, std::vector<fxSliceDesc> &descs, size_t sendOff, size_t cnt, void *out, int first) {
+flagcxResult_t kway(const Ctx &c, SliceList &descs, size_t sendOff, size_t cnt, void *out, int first) {
   if (cnt == 0) return flagcxSuccess;
   if (c.n <= FX_MAX_SLICE_INPUTS) {
     fxSliceDesc d;
@@ -145,12 +167,13 @@ flagcxResult_t kway(const Ctx &c, std::vector<fxSliceDesc> &descs, size_t sendOf
     descs.push_back(d);
     return flagcxSuccess;
   }
-  std::vector<const void *> in(c.n);
+  PtrList in;
+  in.resize((size_t)c.n);
   for (int j = 0; j < c.n; j++) in[j] = cadd(c.send(j), sendOff * c.ts);
   return R(fx_reduce_copy(out, in.data(), c.n, cnt, c.g->dtype, c.g->op, first, c.s));
 }
 
-flagcxResult_t flushKway(const Ctx &c, std::vector<fxSliceDesc> &descs) {
+flagcxResult_t flushKway(const Ctx &c, SliceList &descs) {
   if (descs.empty()) return flagcxSuccess;
   flagcxResult_t rc = R(fx_reduce_slices(descs.data(), descs.size(), c.n, c.g->dtype, c.g->op, c.s));
   descs.clear();
@@ -234,11 +257,11 @@ flagcxResult_t chainHostPieces(const Ctx &c, const std::vector<HostPiece> &piece
   }
   if (total == 0) return flagcxSuccess;
   if (n > 2) {
-    flagcxResult_t rc = ensureScratch(g, total);
+    flagcxResult_t rc = ensureScratch(g, total, c.s);
     if (rc != flagcxSuccess) return rc;
   }
-  std::vector<fxSliceDesc> plain, copies;
-  std::vector<fxBcastDesc> bcast;
+  SliceList plain, copies;
+  BcastList bcast;
   int nout = 1;
   for (int j = 1; j < n; j++) {
     plain.clear();
@@ -283,8 +306,8 @@ inline bool isFloating(int dtype) {
 flagcxResult_t reduceHostPieces(const Ctx &c, const std::vector<HostPiece> &pieces) {
   if ((c.g->op == flagcxMax || c.g->op == flagcxMin) && isFloating(c.g->dtype)) return chainHostPieces(c, pieces);
   std::vector<int> order;
-  std::vector<fxBcastDesc> bcast;
-  std::vector<fxSliceDesc> plain;
+  BcastList bcast;
+  SliceList plain;
   int nout = 0;
   for (const HostPiece &p : pieces) {
     if (p.cnt == 0) continue;
@@ -309,11 +332,12 @@ flagcxResult_t reduceHostPieces(const Ctx &c, const std::vector<HostPiece> &piec
       continue;
     }
     // more than eight ranks: one runtime-k launch per piece, then copies
-    std::vector<const void *> in(c.n);
+    PtrList in;
+    in.resize((size_t)c.n);
     for (int j = 0; j < c.n; j++) in[j] = cadd(c.send(order[j]), p.off * c.ts);
     flagcxResult_t rc = R(fx_reduce_copy(p.outs[0], in.data(), c.n, p.cnt, c.g->dtype, c.g->op, 0, c.s));
     if (rc != flagcxSuccess) return rc;
-    std::vector<fxSliceDesc> copies;
+    SliceList copies;
     for (int o = 1; o < nout; o++) copies.push_back(copyDesc(p.outs[0], p.outs[o], p.cnt * c.ts));
     rc = R(fx_copy_slices(copies.data(), copies.size(), c.s));
     if (rc != flagcxSuccess) return rc;
@@ -347,7 +371,7 @@ flagcxResult_t runAllReduce(const Ctx &c) {
     return reduceHostPieces(c, pieces);
   }
   const size_t nred = fx_nredslices(count, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
-  std::vector<fxSliceDesc> descs;
+  SliceList descs;
   if (g->algo == FX_ALGO_RING && g->op != flagcxAvg) {  // a mean is not a chain of two-input means
     // reduce-scatter: step i, rank r reduces chunk (r-i-1)%n: partial from the
     // previous rank (its sendbuff at step 0, its recvbuff afterwards) + own data.
@@ -392,7 +416,7 @@ flagcxResult_t runAllReduce(const Ctx &c) {
   // all n receive buffers by the same workgroup -- (k + n) * size bytes of
   // traffic instead of the (k + 1 + 2 (n - 1)) * size of reduce-then-copy.
   if (canBroadcast(c)) {
-    std::vector<fxBcastDesc> bd;
+    BcastList bd;
     for (int ch = 0; ch < n; ch++) {
       size_t ccnt, coff;
       fx_split(count, n, ch, &ccnt, &coff);
@@ -465,21 +489,22 @@ flagcxResult_t runReduce(const Ctx &c) {
     return reduceHostPieces(c, pieces);
   }
   if (g->order != FX_ORDER_TREE || n == 1 || g->op == flagcxAvg) {
-    std::vector<const void *> in(n);
+    PtrList in;
+    in.resize((size_t)n);
     for (int j = 0; j < n; j++) in[j] = c.send(j);
     return R(fx_reduce_copy(c.recv(root), in.data(), n, count, g->dtype, g->op, 0, c.s));
   }
   // Tree order: round i, every tree rank a with more than i receive steps
   // computes partial(a) = partial(a + 2^i) (op) partial(a).  Partials live in a
   // per-rank scratch row; the root's last round writes recvbuff.
-  flagcxResult_t rc = ensureScratch(g, (size_t)n * count * ts);
+  flagcxResult_t rc = ensureScratch(g, (size_t)n * count * ts, c.s);
   if (rc != flagcxSuccess) return rc;
   const int total = treeSteps(0, n);
   auto rankOf = [&](int a) { return mod(a + root, n); };
   auto partial = [&](int a, int round) -> const void * {   // where tree rank a's partial is before `round`
     return (round == 0 || treeSteps(a, n) == 0) ? c.send(rankOf(a)) : madd(g->scratch, (size_t)a * count * ts);
   };
-  std::vector<fxSliceDesc> descs;
+  SliceList descs;
   for (int i = 0; i < total; i++) {
     for (int a = 0; a < n; a++) {
       if (treeSteps(a, n) <= i) continue;
@@ -520,10 +545,10 @@ flagcxResult_t runReduceScatter(const Ctx &c) {
     return reduceHostPieces(c, pieces);
   }
   const size_t nred = fx_nredslices(rcount, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
-  std::vector<fxSliceDesc> descs;
+  SliceList descs;
   if (g->algo == FX_ALGO_RING && g->op != flagcxAvg) {  // a mean is not a chain of two-input means
     // Per-rank scratch of n*recvcount elements holds the travelling partials.
-    flagcxResult_t rc = ensureScratch(g, (size_t)n * n * rcount * ts);
+    flagcxResult_t rc = ensureScratch(g, (size_t)n * n * rcount * ts, c.s);
     if (rc != flagcxSuccess) return rc;
     auto scratch = [&](int r) { return madd(g->scratch, (size_t)r * n * rcount * ts); };
     for (int i = 0; i < n - 1; i++) {
@@ -563,7 +588,8 @@ flagcxResult_t runAllGather(const Ctx &c) {
   const size_t bytes = c.g->count * c.ts;
   if (bytes == 0) return flagcxSuccess;
   if (canBroadcast(c)) {  // each rank's block is read once and stored to every receive buffer
-    std::vector<fxBcastDesc> bd(c.n);
+    BcastList bd;
+    bd.resize((size_t)c.n);
     for (int r = 0; r < c.n; r++) {
       memset(&bd[r], 0, sizeof(fxBcastDesc));
       bd[r].in[0] = c.send(r);
@@ -572,7 +598,7 @@ flagcxResult_t runAllGather(const Ctx &c) {
     }
     return R(fx_reduce_bcast_slices(bd.data(), bd.size(), 1, c.n, 0, -1, c.s));
   }
-  std::vector<fxSliceDesc> descs;
+  SliceList descs;
   for (int r = 0; r < c.n; r++)
     for (int j = 0; j < c.n; j++) {
       void *dst = madd(c.recv(j), (size_t)r * bytes);
@@ -616,14 +642,14 @@ flagcxResult_t runAlltoAllv(const Ctx &c) {
     for (size_t b = 0; b < sendR.size() && !overlap; b++)
       overlap = recvR[a].lo < sendR[b].hi && sendR[b].lo < recvR[a].hi;
   if (!overlap) {
-    std::vector<fxSliceDesc> direct;
+    SliceList direct;
     for (size_t a = 0; a < recvR.size(); a++)
       direct.push_back(copyDesc((const void *)sendR[a].lo, (void *)recvR[a].lo, recvR[a].hi - recvR[a].lo));
     return R(fx_copy_slices(direct.data(), direct.size(), c.s));
   }
-  flagcxResult_t rc = ensureScratch(g, base[n]);
+  flagcxResult_t rc = ensureScratch(g, base[n], c.s);
   if (rc != flagcxSuccess) return rc;
-  std::vector<fxSliceDesc> pack, unpack;
+  SliceList pack, unpack;
   for (int r = 0; r < n; r++) {
     size_t slot = 0;
     for (int i = 0; i < n; i++) {
@@ -646,7 +672,7 @@ flagcxResult_t runAlltoAllv(const Ctx &c) {
 // flagcx/adaptor/ccl/rccl_adaptor.cc:126-184,222-246).
 flagcxResult_t runGather(const Ctx &c) {
   const size_t bytes = c.g->count * c.ts;
-  std::vector<fxSliceDesc> d;
+  SliceList d;
   for (int r = 0; r < c.n && bytes; r++) {
     void *dst = madd(c.recv(c.g->root), (size_t)r * bytes);
     if (dst != c.send(r)) d.push_back(copyDesc(c.send(r), dst, bytes));
@@ -656,7 +682,7 @@ flagcxResult_t runGather(const Ctx &c) {
 
 flagcxResult_t runScatter(const Ctx &c) {
   const size_t bytes = c.g->count * c.ts;
-  std::vector<fxSliceDesc> d;
+  SliceList d;
   for (int r = 0; r < c.n && bytes; r++) {
     const void *src = cadd(c.send(c.g->root), (size_t)r * bytes);
     if (src != c.recv(r)) d.push_back(copyDesc(src, c.recv(r), bytes));
@@ -674,7 +700,7 @@ flagcxResult_t runBroadcast(const Ctx &c) {
     b.count = bytes;
     return R(fx_reduce_bcast_slices(&b, 1, 1, c.n, 0, -1, c.s));
   }
-  std::vector<fxSliceDesc> d;
+  SliceList d;
   for (int r = 0; r < c.n && bytes; r++)
     if (c.recv(r) != c.send(c.g->root)) d.push_back(copyDesc(c.send(c.g->root), c.recv(r), bytes));
   return R(fx_copy_slices(d.data(), d.size(), c.s));
@@ -689,14 +715,14 @@ flagcxResult_t runAlltoAll(const Ctx &c) {
   if (bytes == 0) return flagcxSuccess;
   bool inplace = false;
   for (int r = 0; r < n; r++) inplace = inplace || (c.send(r) == c.recv(r));
-  std::vector<fxSliceDesc> d;
+  SliceList d;
   if (!inplace) {
     for (int r = 0; r < n; r++)
       for (int i = 0; i < n; i++)
         d.push_back(copyDesc(cadd(c.send(r), (size_t)i * bytes), madd(c.recv(i), (size_t)r * bytes), bytes));
     return R(fx_copy_slices(d.data(), d.size(), c.s));
   }
-  flagcxResult_t rc = ensureScratch(g, (size_t)n * n * bytes);
+  flagcxResult_t rc = ensureScratch(g, (size_t)n * n * bytes, c.s);
   if (rc != flagcxSuccess) return rc;
   for (int r = 0; r < n; r++)
     d.push_back(copyDesc(c.send(r), madd(g->scratch, (size_t)r * n * bytes), (size_t)n * bytes));
@@ -720,7 +746,7 @@ flagcxResult_t runCustomAllReduce(const Ctx &c) {
     b.count = g->count;
     return R(fx_reduce_bcast_slices(&b, 1, c.n, c.n, g->dtype, g->op, c.s));
   }
-  std::vector<fxSliceDesc> descs;
+  SliceList descs;
   for (int r = 0; r < c.n; r++) {
     if (c.n <= FX_MAX_SLICE_INPUTS) {
       fxSliceDesc d;
@@ -884,6 +910,16 @@ flagcxResult_t screenReduce(int dtype, int op) {
 std::mutex gRegistryMu;
 std::map<std::string, Group *> gRegistry;  // groups still waiting for ranks to join, by id
 
+void freeGroupResources(Group *g) {
+  for (auto e : g->ready)
+    if (e) (void)hipEventDestroy(e);
+  if (g->done) (void)hipEventDestroy(g->done);
+  for (auto &p : g->p2p) (void)hipEventDestroy(p.posted);
+  if (g->scratch) (void)hipFree(g->scratch);
+  for (void *b : g->outgrown) (void)hipFree(b);
+  delete g;
+}
+
 flagcxResult_t newGroup(int nranks, Group **out) {
   Group *g = new (std::nothrow) Group();
   if (!g) return flagcxSystemError;
@@ -918,17 +954,52 @@ flagcxResult_t newGroup(int nranks, Group **out) {
   if (sync && !strcmp(sync, "rendezvous")) g->sync = FX_SYNC_RENDEZVOUS;
   g->timeoutMs = envParam("FX_SIM_RENDEZVOUS_TIMEOUT_MS", 30000);
   if (g->timeoutMs < 1) g->timeoutMs = 1;
+  const long long reserve = envParam("FX_SIM_SCRATCH_BYTES", 0);
+  if (reserve > 0 && ensureScratch(g, (size_t)reserve, nullptr) != flagcxSuccess) {
+    freeGroupResources(g);
+    return flagcxUnhandledDeviceError;
+  }
   *out = g;
   return flagcxSuccess;
 }
 
 void freeGroup(Group *g) {
   (void)hipDeviceSynchronize();
-  for (auto e : g->ready) (void)hipEventDestroy(e);
-  (void)hipEventDestroy(g->done);
-  for (auto &p : g->p2p) (void)hipEventDestroy(p.posted);
-  if (g->scratch) (void)hipFree(g->scratch);
-  delete g;
+  freeGroupResources(g);
+}
+
+// Group brackets are per host thread (the CCL adaptor's groupStart / groupEnd
+// carry no communicator).  They matter in rendezvous mode only: a send or recv
+// posted inside a bracket does not sleep until its partner arrives -- every
+// rank's thread would sit in its first call and none would reach its second --
+// it is remembered here and waited for when the outermost bracket closes, which
+// is where the reference issues the grouped operations (flagcx/flagcx.cc group
+// semantics; rccl_adaptor.cc:322-332 forwards the bracket to the vendor library).
+struct DeferredP2p {
+  Group *g;
+  uint64_t id;
+};
+thread_local int tGroupDepth = 0;
+thread_local std::vector<DeferredP2p> tDeferred;
+
+// Wait until the partner of pending half `id` has made its call (it enqueues the
+// copy and makes our stream wait for it) and hand back its result; on time-out
+// the half is withdrawn.  Called with g->mu held.
+flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64_t id) {
+  const bool matched = g->cv.wait_for(lock, std::chrono::milliseconds(g->timeoutMs),
+                                      [&] { return g->p2pMatched.count(id) != 0; });
+  if (!matched) {  // the partner never came: withdraw this half
+    for (size_t i = 0; i < g->p2p.size(); i++)
+      if (g->p2p[i].id == id) {
+        (void)hipEventDestroy(g->p2p[i].posted);
+        g->p2p.erase(g->p2p.begin() + (long)i);
+        break;
+      }
+    return flagcxInternalError;
+  }
+  const flagcxResult_t res = g->p2pMatched[id];
+  g->p2pMatched.erase(id);
+  return res;
 }
 
 // send / recv between simulated ranks: the later of the two calls performs the
@@ -984,22 +1055,12 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
   }
   g->p2p.push_back(p);
   if (g->sync != FX_SYNC_RENDEZVOUS) return flagcxSuccess;
-  // Sleep until the partner has made its call and enqueued the copy.
-  const uint64_t id = p.id;
-  const bool matched = g->cv.wait_for(lock, std::chrono::milliseconds(g->timeoutMs),
-                                      [&] { return g->p2pMatched.count(id) != 0; });
-  if (!matched) {  // the partner never came: withdraw this half
-    for (size_t i = 0; i < g->p2p.size(); i++)
-      if (g->p2p[i].id == id) {
-        (void)hipEventDestroy(g->p2p[i].posted);
-        g->p2p.erase(g->p2p.begin() + (long)i);
-        break;
-      }
-    return flagcxInternalError;
+  if (tGroupDepth > 0) {  // inside a bracket: the wait happens when the bracket closes
+    tDeferred.push_back(DeferredP2p{g, p.id});
+    return flagcxSuccess;
   }
-  const flagcxResult_t res = g->p2pMatched[id];
-  g->p2pMatched.erase(id);
-  return res;
+  // Sleep until the partner has made its call and enqueued the copy.
+  return awaitPartner(g, lock, p.id);
 }
 
 }  // namespace
@@ -1168,6 +1229,9 @@ flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
       if (g->nposted) return flagcxInvalidUsage;  // not while a collective is half posted
       g->sync = value;
       break;
+    case FX_SIM_SCRATCH_BYTES:  // reserve now what the scratch users would otherwise allocate at their first call
+      if (value < 0) return flagcxInvalidArgument;
+      return ensureScratch(g, (size_t)value, nullptr);
     default: return flagcxInvalidArgument;
   }
   return flagcxSuccess;
@@ -1268,10 +1332,28 @@ flagcxResult_t flagcxRecv(void *recvbuff, size_t count, flagcxDataType_t datatyp
   return postP2p(comm, false, nullptr, recvbuff, count, datatype, peer, stream);
 }
 
-// Calls are asynchronous and matched across ranks as they arrive, so a group
-// bracket has nothing to defer.
-flagcxResult_t flagcxGroupStart(flagcxComm_t) { return flagcxSuccess; }
-flagcxResult_t flagcxGroupEnd(flagcxComm_t) { return flagcxSuccess; }
+// Calls are asynchronous and matched across ranks as they arrive, so in group
+// mode a bracket has nothing to defer.  In rendezvous mode the sends and recvs
+// posted inside the outermost bracket of this thread are waited for here.
+flagcxResult_t flagcxGroupStart(flagcxComm_t) {
+  tGroupDepth++;
+  return flagcxSuccess;
+}
+flagcxResult_t flagcxGroupEnd(flagcxComm_t) {
+  if (tGroupDepth == 0) return flagcxInvalidUsage;  // no bracket open on this thread
+  if (--tGroupDepth > 0) return flagcxSuccess;
+  return R(fx::guarded([&]() -> int {
+    flagcxResult_t first = flagcxSuccess;
+    std::vector<DeferredP2p> mine;
+    mine.swap(tDeferred);
+    for (const DeferredP2p &d : mine) {
+      std::unique_lock<std::mutex> lock(d.g->mu);
+      const flagcxResult_t rc = awaitPartner(d.g, lock, d.id);
+      if (first == flagcxSuccess) first = rc;
+    }
+    return first;
+  }));
+}
 
 flagcxResult_t fxSimCommDevice(const flagcxComm_t comm, int *device) {
   if (!comm || !comm->g || !device) return flagcxInvalidArgument;

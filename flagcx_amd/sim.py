@@ -6,7 +6,7 @@ from . import _native as N
 
 lib = N.lib
 
-ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE, SYNC = 0, 1, 2, 3, 4, 5
+ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE, SYNC, SCRATCH_BYTES = 0, 1, 2, 3, 4, 5, 6
 ALGO_DIRECT, ALGO_RING = 0, 1
 ORDER_RANK, ORDER_RING, ORDER_TREE, ORDER_HOST = 0, 1, 2, 3
 SYNC_GROUP, SYNC_RENDEZVOUS = 0, 1
@@ -23,9 +23,10 @@ class SimGroup:
         N.check(lib.fxSimCommInitAll(self.comms, nranks), "fxSimCommInitAll")
         self.configure(**config)
 
-    def configure(self, algo=None, order=None, nslices=None, nredslices=None, redslicesize=None, sync=None):
+    def configure(self, algo=None, order=None, nslices=None, nredslices=None, redslicesize=None, sync=None,
+                  scratch_bytes=None):
         for key, val in ((ALGO, algo), (ORDER, order), (NSLICES, nslices), (NREDSLICES, nredslices),
-                         (REDSLICESIZE, redslicesize), (SYNC, sync)):
+                         (REDSLICESIZE, redslicesize), (SYNC, sync), (SCRATCH_BYTES, scratch_bytes)):
             if val is not None:
                 N.check(lib.fxSimCommConfig(self.comms[0], key, val), f"fxSimCommConfig({key})")
 

@@ -29,6 +29,18 @@
  *     the rank enqueues after the call returns is ordered after the collective.
  *     A rank that never arrives makes the others return flagcxInternalError
  *     after FX_SIM_RENDEZVOUS_TIMEOUT_MS (environment, default 30000).
+ *     flagcxSend / flagcxRecv posted between flagcxGroupStart and
+ *     flagcxGroupEnd on a host thread do not block: the outermost
+ *     flagcxGroupEnd of that thread waits for their partners, so every rank's
+ *     thread can run GroupStart, Send(next), Recv(prev), GroupEnd.
+ *
+ * Scratch (partials of the tree reduce and of the ring reduce-scatter, the
+ * host order's floating max / min, staging of in-place all-to-all(v)) is grown
+ * by allocating a larger block and keeping the old ones until the group is
+ * destroyed: no call waits for the device.  A captured stream cannot
+ * allocate: reserve beforehand with fxSimCommConfig(comm, FX_SIM_SCRATCH_BYTES,
+ * n) or the environment variable of the same name, else such a call returns
+ * flagcxInvalidUsage while the stream is capturing.
  */
 #ifndef FLAGCX_AMD_FX_SIM_H_
 #define FLAGCX_AMD_FX_SIM_H_
@@ -84,7 +96,8 @@ enum {
   FX_SIM_NSLICES = 2,      /* FLAGCX_UNIRUNNER_NSLICES (default 1)        */
   FX_SIM_NREDSLICES = 3,   /* FLAGCX_UNIRUNNER_NREDSLICES (0 = automatic) */
   FX_SIM_REDSLICESIZE = 4, /* FLAGCX_UNIRUNNER_REDSLICESIZE (65536 elems) */
-  FX_SIM_SYNC = 5          /* FX_SYNC_*; environment FX_SIM_SYNC=group|rendezvous */
+  FX_SIM_SYNC = 5,         /* FX_SYNC_*; environment FX_SIM_SYNC=group|rendezvous */
+  FX_SIM_SCRATCH_BYTES = 6 /* reserve at least this much scratch now            */
 };
 enum {
   FX_SYNC_GROUP = 0,

@@ -425,6 +425,56 @@ def test_rendezvous_mode_orders_later_work_after_the_collective(dev):
         assert not errors, errors[:4]
 
 
+def test_rendezvous_ring_exchange_inside_a_group_bracket(dev, monkeypatch):
+    """The usual thread-per-rank pattern: every rank runs GroupStart, Send(next),
+    Recv(prev), GroupEnd -- all of them send FIRST.  Outside a bracket that would
+    leave every thread asleep in its send; inside one the posts are remembered
+    and the bracket's end waits for the partners.  It must finish by itself, well
+    inside the rendezvous time-out (set long enough here that a pass through the
+    time-out path would show in the elapsed time), with the right data."""
+    import threading
+    import time
+    monkeypatch.setenv("FX_SIM_RENDEZVOUS_TIMEOUT_MS", "15000")
+    n, count, rounds = 8, 40003, 10
+    errors = []
+    with DevBufs(dev) as b, S.SimGroup(n, sync=S.SYNC_RENDEZVOUS) as g:
+        dsend = [b.alloc(count * 4) for _ in range(n)]
+        drecv = [b.alloc(count * 4) for _ in range(n)]
+
+        def rank_main(r):
+            try:
+                dev.set_device()
+                s = dev.stream_create()
+                host = np.empty(count, np.float32)
+                for it in range(rounds):
+                    src = np.full(count, r * 100 + it, np.float32)
+                    dev.upload(dsend[r], src, s)
+                    N.check(N.lib.flagcxGroupStart(g.comms[r]))
+                    N.check(N.lib.flagcxSend(dsend[r], count, N.DT_FP32, (r + 1) % n, g.comms[r], s))
+                    N.check(N.lib.flagcxRecv(drecv[r], count, N.DT_FP32, (r - 1) % n, g.comms[r], s))
+                    N.check(N.lib.flagcxGroupEnd(g.comms[r]))
+                    dev.download(host, drecv[r], s)
+                    dev.stream_sync(s)
+                    if not (host == ((r - 1) % n) * 100 + it).all():
+                        errors.append((r, it, host[:4].tolist()))
+                    N.check(N.lib.flagcxBarrier(g.comms[r], s))     # nobody overwrites dsend while a neighbour reads it
+                    dev.stream_sync(s)
+                dev.stream_destroy(s)
+            except Exception as e:                      # noqa: BLE001 - reported below
+                errors.append((r, repr(e)))
+
+        t0 = time.time()
+        threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=100)
+        assert not any(t.is_alive() for t in threads)
+        assert not errors, errors[:4]
+        assert time.time() - t0 < 12, "the exchange went through the time-out path"
+    assert N.lib.flagcxGroupEnd(None) == N.INVALID_USAGE            # no bracket open on this thread
+
+
 def test_rendezvous_times_out_when_a_rank_never_arrives(dev, stream, monkeypatch):
     import threading
     monkeypatch.setenv("FX_SIM_RENDEZVOUS_TIMEOUT_MS", "200")

@@ -111,3 +111,74 @@ def test_simulated_rank_allreduce_replays_correctly_in_a_graph(dev):
         hip.hipGraphExecDestroy(gexec)
         hip.hipGraphDestroy(graph)
     dev.stream_destroy(stream)
+
+
+def test_scratch_users_capture_cold_after_a_reservation(dev):
+    """Tree-order reduce, ring reduce-scatter and in-place all-to-all need scratch.
+    With the scratch reserved at set-up (fxSimCommConfig FX_SIM_SCRATCH_BYTES) their
+    very first call may be inside a capture -- no eager call beforehand -- and the
+    graph replays correctly on new data; without a reservation the same call is
+    refused while the stream is capturing, and works eagerly afterwards."""
+    from flagcx_amd import sim as S
+    n, count = 5, 5 * 30011
+    dtype = N.DT_FP32
+    stream = dev.stream_create()
+    raw = dev.raw_stream(stream)
+    with DevBufs(dev) as b:
+        sends = seeded_inputs(dtype, n, count, seed=8)
+        ds = [b.put(a) for a in sends]
+        droot = b.alloc(count * 4)
+        dp = [b.alloc(count // n * 4) for _ in range(n)]
+        da = [b.put(a) for a in sends]                       # all-to-all runs in place on these
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        # no reservation: refused under capture (nothing is enqueued), fine eagerly
+        with S.SimGroup(n, order=S.ORDER_TREE) as g:
+            assert hip.hipStreamBeginCapture(raw, 0) == 0
+            try:
+                rc = g.reduce(ds, [droot] * n, count, dtype, N.OP_SUM, 2, stream)
+            finally:
+                assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
+            assert rc == N.INVALID_USAGE
+            hip.hipGraphDestroy(graph)
+            N.check(g.reduce(ds, [droot] * n, count, dtype, N.OP_SUM, 2, stream))
+            dev.stream_sync(stream)
+            assert_parity(dev.to_host(droot, count, np.float32), O.tree_reduce(sends, 2, dtype, N.OP_SUM), dtype,
+                          N.OP_SUM, "eager tree reduce")
+        # reserved: cold capture
+        with S.SimGroup(n, order=S.ORDER_TREE, algo=S.ALGO_RING, scratch_bytes=n * n * count * 4) as g:
+            assert hip.hipStreamBeginCapture(raw, 0) == 0
+            try:
+                N.check(g.reduce(ds, [droot] * n, count, dtype, N.OP_SUM, 2, stream))
+                N.check(g.reduce_scatter(ds, dp, count // n, dtype, N.OP_SUM, stream))
+                N.check(N.lib.flagcxAlltoAll(da[0], da[0], count // n, dtype, g.comms[0], stream))
+                for r in range(1, n):
+                    N.check(N.lib.flagcxAlltoAll(da[r], da[r], count // n, dtype, g.comms[r], stream))
+            finally:
+                assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
+            assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+            part = count // n
+            for rep in range(3):
+                if rep:
+                    sends = seeded_inputs(dtype, n, count, seed=8 + rep)
+                    for d, a in zip(ds, sends):
+                        dev.upload(d, a)
+                for d, a in zip(da, sends):
+                    dev.upload(d, a)
+                dev.memset(droot, 0xEE, count * 4)
+                dev.sync()
+                assert hip.hipGraphLaunch(gexec, raw) == 0
+                dev.stream_sync(stream)
+                assert_parity(dev.to_host(droot, count, np.float32), O.tree_reduce(sends, 2, dtype, N.OP_SUM), dtype,
+                              N.OP_SUM, f"replay {rep} tree reduce")
+                for r in (0, n - 1):
+                    # the ring leaves chunk r on rank r folded from rank r + 1 round to rank r
+                    want = O.reduce_copy([a[r * part:(r + 1) * part] for a in sends], dtype, N.OP_SUM, first=(r + 1) % n)
+                    assert_parity(dev.to_host(dp[r], part, np.float32), want, dtype, N.OP_SUM,
+                                  f"replay {rep} reduce-scatter rank {r}")
+                    a2a = dev.to_host(da[r], count, np.float32)
+                    for src in range(n):
+                        assert np.array_equal(a2a[src * part:(src + 1) * part].view(np.uint32),
+                                              sends[src][r * part:(r + 1) * part].view(np.uint32)), (rep, r, src)
+            hip.hipGraphExecDestroy(gexec)
+            hip.hipGraphDestroy(graph)
+    dev.stream_destroy(stream)

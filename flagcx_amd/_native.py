@@ -18,6 +18,8 @@ DT_FP16, DT_FP32, DT_FP64, DT_BF16 = 6, 7, 8, 9
 OP_SUM, OP_PROD, OP_MAX, OP_MIN, OP_AVG = 0, 1, 2, 3, 4
 MEMCPY_H2D, MEMCPY_D2H, MEMCPY_D2D = 0, 1, 2
 MEM_HOST, MEM_DEVICE, MEM_MANAGED = 0, 1, 2
+# TIMER_COLL_* slots of fxHostStagedAllReduce (include/flagcx_amd/fx_host_staged.h)
+TIMER_NAMES = ("total", "calc", "comm", "mem", "mem_d2h", "mem_h2d", "alloc", "free")
 STATIC_MAX_SLICES = 1024   # FX_STATIC_MAX_SLICES of include/flagcx_amd/fx_kernels.h
 
 DTYPE_SIZE = {DT_INT8: 1, DT_UINT8: 1, DT_INT32: 4, DT_UINT32: 4, DT_INT64: 8, DT_UINT64: 8,
@@ -132,6 +134,10 @@ _SIGS.update({
     "flagcxAllGather": (_i, [_vp, _vp, _sz, _i, _vp, _vp]),
     "flagcxAlltoAllv": (_i, [_vp, _szp, _szp, _vp, _szp, _szp, _i, _vp, _vp]),
     "flagcxCustomAllReduceImpl": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),
+    # include/flagcx_amd/fx_host_staged.h
+    "fxHostStagedCreate": (_i, [C.POINTER(_vp), _i, _vp]),
+    "fxHostStagedAllReduce": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _i, _i, C.POINTER(C.c_uint64)]),
+    "fxHostStagedDestroy": (_i, [_vp]),
     "fx_part_ring_ar": (_sz, [_sz, _i, _i, _sz, _sz, C.POINTER(RedNode)]),
     "fx_part_ring_rs": (_sz, [_sz, _i, _i, _sz, _sz, C.POINTER(RedNode)]),
     "fx_part_locred": (_sz, [_sz, _i, _i, _sz, C.POINTER(RedNode)]),

@@ -79,3 +79,34 @@ class SimGroup:
     def register_windows(self, windows, nbytes):
         arr = (C.c_void_p * self.n)(*windows) if windows else None
         return lib.fxSimRegisterWindows(self.comms[0], arr, nbytes)
+
+
+class HostStaged:
+    """The reference's host-staged all-reduce over n simulated ranks
+    (include/flagcx_amd/fx_host_staged.h): D2H, ring all-reduce on the host, H2D,
+    with the reference's per-phase timers."""
+
+    def __init__(self, nranks, device_memcpy=None):
+        self.n = nranks
+        self.h = C.c_void_p()
+        fn = C.cast(device_memcpy, C.c_void_p) if device_memcpy is not None else None
+        N.check(lib.fxHostStagedCreate(C.byref(self.h), nranks, fn), "fxHostStagedCreate")
+
+    def all_reduce(self, sends, recvs, count, dtype, op):
+        """Returns (result code, per-rank dicts of phase nanoseconds)."""
+        t = (C.c_uint64 * (self.n * len(N.TIMER_NAMES)))()
+        rc = lib.fxHostStagedAllReduce(self.h, (C.c_void_p * self.n)(*sends), (C.c_void_p * self.n)(*recvs), count,
+                                       dtype, op, t)
+        k = len(N.TIMER_NAMES)
+        return rc, [dict(zip(N.TIMER_NAMES, t[r * k:(r + 1) * k])) for r in range(self.n)]
+
+    def destroy(self):
+        if self.h:
+            lib.fxHostStagedDestroy(self.h)
+            self.h = C.c_void_p()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.destroy()

@@ -608,3 +608,52 @@ def test_single_rank_and_empty_collectives(dev, stream):
         assert g.reduce(p, p, 4, N.DT_FP32, N.OP_SUM, 4, stream) == N.INVALID_ARGUMENT          # root out of range
         assert N.lib.flagcxAllReduce(p[0], p[0], 4, N.DT_FP32, N.OP_SUM, g.comms[0], None) == N.INVALID_ARGUMENT
         assert N.lib.flagcxAllReduce(None, p[0], 4, N.DT_FP32, N.OP_SUM, g.comms[0], stream) == N.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("dname", ["fp32", "fp64", "int32", "uint8", "int64"])
+@pytest.mark.parametrize("n,count", [(8, 100003), (3, 10), (4, 2), (5, 77777), (2, 1 << 20)])
+def test_host_staged_allreduce_matches_host_order_and_oracle(dev, stream, dname, n, count):
+    """fxHostStagedAllReduce is the reference's CPU path end to end
+    (host_runner.cc:236-289 over bootstrap.cc:787-942): device to host through
+    the device adaptor's deviceMemcpy, ring all-reduce with the host loops, host
+    to device.  Its result must be the hop-by-hop oracle's and, bit for bit, what
+    the device computes under FX_ORDER_HOST; its timers must add up."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    npdt = N.NP_DTYPE[dtype]
+    sends = seeded_inputs(dtype, n, count, seed=3 * n + count)
+    if dname in ("fp32", "fp64"):
+        rng = np.random.default_rng(count)
+        sends = [(a * 10.0 ** rng.integers(-3, 9, count)).astype(npdt) for a in sends]
+        for r, a in enumerate(sends):
+            a[:min(count, 8)] = [(0.0, -0.0)[(r + i) % 2] for i in range(min(count, 8))]
+        for i in range(8, min(count, 8 + 3 * n)):
+            sends[i % n][i] = np.nan
+    with DevBufs(dev) as b, S.HostStaged(n, dev.t.deviceMemcpy) as hs, S.SimGroup(n, order=S.ORDER_HOST) as g:
+        ds = [b.put(a) for a in sends]
+        dr = [b.alloc(count * es) for _ in range(n)]
+        ddev = [b.alloc(count * es) for _ in range(n)]
+        for op in (N.OP_SUM, N.OP_MAX, N.OP_MIN):
+            want = O.bootstrap_allreduce(sends, dtype, op)
+            rc, timers = hs.all_reduce(ds, dr, count, dtype, op)
+            N.check(rc, "fxHostStagedAllReduce")
+            N.check(g.all_reduce(ds, ddev, count, dtype, op, stream))
+            dev.stream_sync(stream)
+            for r in range(n):
+                got = dev.to_host(dr[r], count, npdt)
+                assert np.array_equal(got.view(np.uint8), want[r].view(np.uint8)), f"rank {r} op {op} vs the oracle"
+                on_device = dev.to_host(ddev[r], count, npdt)
+                assert np.array_equal(got.view(np.uint8), on_device.view(np.uint8)), f"rank {r} op {op} vs FX_ORDER_HOST"
+                t = timers[r]
+                # (the ring's own buffer allocation is counted in both `alloc` and `comm`, as in the reference)
+                assert t["total"] >= t["mem_d2h"] + t["comm"] + t["mem_h2d"] and t["comm"] >= t["calc"] + t["mem"]
+                assert t["mem_d2h"] > 0 and t["mem_h2d"] > 0 and (n == 1 or count < n or t["calc"] > 0)
+        # in place on the device buffers
+        rc, _ = hs.all_reduce(ds, ds, count, dtype, N.OP_SUM)
+        N.check(rc)
+        want = O.bootstrap_allreduce(sends, dtype, N.OP_SUM)
+        for r in (0, n - 1):
+            assert np.array_equal(dev.to_host(ds[r], count, npdt).view(np.uint8), want[r].view(np.uint8))
+        # what the reference's host loops do not carry is refused, as there
+        assert hs.all_reduce(ds, dr, count, dtype, N.OP_PROD)[0] == N.INVALID_ARGUMENT
+        assert hs.all_reduce(ds, dr, count, N.DT_BF16, N.OP_SUM)[0] == N.INVALID_ARGUMENT

@@ -97,10 +97,9 @@ def test_cfg2_ring_share_slices_then_allgather(dev, stream):
 
 @pytest.mark.parametrize("dtype", list(W.CFG3["dists"]))
 def test_cfg3_size_and_op_sweep(dev, dtype):
-    """k = 4, 1 KiB .. 1 GiB per input, sum/max/min/prod, in place and out of
-    place.  Up to 16 MiB every case is compared with the committed digests; above,
-    sum runs at every size and the other ops at 64 MiB and 1 GiB, against the
-    oracle run live."""
+    """k = 4, 1 KiB .. 1 GiB per input at every power of two, sum/max/min/prod, in
+    place and out of place.  Up to 16 MiB every case is compared with the
+    committed digests; above, with the oracle run live on the same inputs."""
     es = N.DTYPE_SIZE[dtype]
     nmax = (1 << 30) // es
     ins = W.cfg3_inputs(dtype, nmax, THREADS)
@@ -112,20 +111,19 @@ def test_cfg3_size_and_op_sweep(dev, dtype):
         for lg in range(10, 31):
             n = (1 << lg) // es
             for oname, op in W.OPS.items():
-                if lg > 24 and op != N.OP_SUM and lg not in (26, 30):
-                    continue
                 if lg <= 24:
                     want_digest, want = GOLDEN["cfg3"][f"{name}_{oname}_{1 << lg}"]["out_sha256"], None
                 else:
-                    want = O.reduce_copy([a[:n] for a in ins], dtype, op)
-                    want_digest = W.digest(want)
+                    want_digest, want = None, O.reduce_copy([a[:n] for a in ins], dtype, op)
                 N.check(K.reduce_copy(dout, dins, n, dtype, op))
                 dev.copy(dscratch, dins[0], n * es)
                 N.check(K.reduce_copy(dscratch, [dscratch] + dins[1:], n, dtype, op))     # out = in[0]
                 dev.sync()
                 for label, ptr in (("out-of-place", dout), ("in-place", dscratch)):
                     got = dev.to_host(ptr, n, N.NP_DTYPE[dtype])
-                    if W.digest(got) != want_digest:      # fp16 sum/prod may differ by 1 ulp at most: show it
+                    same = (W.digest(got) == want_digest) if want is None else \
+                        np.array_equal(got.view(np.uint8), want.view(np.uint8))
+                    if not same:                          # fp16 sum/prod may differ by 1 ulp at most: show it
                         want = want if want is not None else O.reduce_copy([a[:n] for a in ins], dtype, op)
                         assert_parity(got, want, dtype, op, f"cfg3 {name} {oname} {1 << lg} B {label}")
                         if dtype != N.DT_FP16 or op in (N.OP_MAX, N.OP_MIN):

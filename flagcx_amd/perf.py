@@ -35,20 +35,25 @@ class Timer:
         self.raw = dev.raw_stream(self.stream)
 
     def ms(self, fn):
+        """Milliseconds per call: `iters` back-to-back calls between two events, the
+        median of three such rounds (one host hiccup of half a millisecond would
+        otherwise add tens of microseconds to a ten-microsecond figure)."""
         d = self.dev
         for _ in range(self.warmup):
             fn()
         d.stream_sync(self.stream)
-        e0, e1 = d.event_create(), d.event_create()
-        d.event_record(e0, self.stream)
-        for _ in range(self.iters):
-            fn()
-        d.event_record(e1, self.stream)
-        d.event_sync(e1)
-        t = d.event_ms(e0, e1) / self.iters
-        d.event_destroy(e0)
-        d.event_destroy(e1)
-        return t
+        rounds = []
+        for _ in range(3):
+            e0, e1 = d.event_create(), d.event_create()
+            d.event_record(e0, self.stream)
+            for _ in range(self.iters):
+                fn()
+            d.event_record(e1, self.stream)
+            d.event_sync(e1)
+            rounds.append(d.event_ms(e0, e1) / self.iters)
+            d.event_destroy(e0)
+            d.event_destroy(e1)
+        return sorted(rounds)[1]
 
 
 def row(label, nbytes, ms, algo_bytes):
@@ -60,10 +65,17 @@ def run_reduce(dev, a):
     dtype, op, k = DT[a.dtype], OP[a.op], a.k
     es = N.DTYPE_SIZE[dtype]
     emax = size(a.max)
-    ins = [dev.malloc(emax + a.misalign * es + a.in_shift * k) + a.in_shift * i for i in range(k)]
+    if a.stride:        # one arena: buffer i starts i * stride bytes in (the output is buffer k), plus the shifts
+        span = size(a.stride)
+        arena = dev.malloc((k + 1) * span + emax + a.misalign * es + a.in_shift * k)
+        ins = [arena + i * span + a.in_shift * i for i in range(k)]
+        spare = arena + k * span
+    else:
+        ins = [dev.malloc(emax + a.misalign * es + a.in_shift * k) + a.in_shift * i for i in range(k)]
+        spare = None
     for i, p in enumerate(ins):
         dev.memset(p, 0x3c + i, emax)
-    out = ins[0] if a.inplace else dev.malloc(emax + a.misalign * es)
+    out = ins[0] if a.inplace else (spare if spare is not None else dev.malloc(emax + a.misalign * es))
     nbytes = size(a.min)
     while nbytes <= emax:
         n = nbytes // es
@@ -292,6 +304,8 @@ def main(argv=None):
     ap.add_argument("--graph", action="store_true", help="allreduce: capture one call into a HIP graph and time replays")
     ap.add_argument("--misalign", type=int, default=0, help="shift buffers by this many elements")
     ap.add_argument("--mixed", action="store_true", help="shift only every other input (inputs not aligned like the output)")
+    ap.add_argument("--stride", default="",
+                    help="reduce: place the k inputs and the output in ONE allocation, STRIDE bytes apart (e.g. 512M, 16G)")
     ap.add_argument("--in-shift", type=int, default=0,
                     help="start input i at byte offset i*IN_SHIFT of its allocation (multiple of 16 keeps vector loads)")
     a = ap.parse_args(argv)

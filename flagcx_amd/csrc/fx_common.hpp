@@ -128,6 +128,21 @@ typedef u32x4 u32x4_anywhere __attribute__((aligned(1)));
 __device__ __forceinline__ u32x4 ldg_stream(const void *p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4_anywhere *>(p));
 }
+// A load without the streaming hint: the line stays in the die's L2 for a
+// neighbouring workgroup that needs its other half.  Issued as a buffer load
+// (descriptor based at the first active lane's address; lane addresses only
+// grow with the lane number in every tiling used here, so the 32-bit offsets
+// are small and non-negative) rather than as a plain global load: two code
+// paths that differ only in the hint of otherwise identical loads get merged by
+// the optimiser, which drops the hint from both.
+typedef int i32x4_raw __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4 ldg_keep(const void *p) {
+  const uint64_t a = (uint64_t)(uintptr_t)p;
+  const uint64_t base = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
+  __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)base, 0, 0x7fffffff, 0x00020000);
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(uint32_t)(a - base), 0, 0));
+}
 __device__ __forceinline__ void stg_stream(void *p, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
 }

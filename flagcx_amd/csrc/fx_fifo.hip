@@ -118,7 +118,8 @@ __device__ __forceinline__ void runShare(const void *in1, const void *in2, void 
   SegWT<2> sg;  // written through: see the count-in below
   const TilePlan tp = makeSeg<R::ES, kFifoU>(static_cast<Seg<2> &>(sg), in, out, count, 2);
   const uint64_t tiles = tp.tiles();
-  for (uint64_t t = sh.idx; t < tiles; t += sh.takers) reduceTile<R, 2, kFifoU>(sg, tp, (uint32_t)t);
+  // (tiles go to whichever workgroups the trigger's share names: no die grouping of columns here)
+  for (uint64_t t = sh.idx; t < tiles; t += sh.takers) reduceTile<R, 2, kFifoU>(sg, tp, (uint32_t)t, 0u);
 }
 
 template <int DT>
@@ -143,7 +144,7 @@ __device__ __forceinline__ Share shareOf(uint64_t seq, const void *in1, const vo
   if (es != 0 && count != 0 && op >= flagcxSum && op <= flagcxAvg) {
     const bool co = sameLinePhase((uint64_t)(uintptr_t)in1, (uint64_t)(uintptr_t)out) &&
                     sameLinePhase((uint64_t)(uintptr_t)in2, (uint64_t)(uintptr_t)out);
-    tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, co).tiles();
+    tiles = planTiles((uint64_t)(uintptr_t)out, count, es, kFifoU, handOutFor(co, 2)).tiles();
   }
   return shareFor(gridDim.x, blockIdx.x, seq, tiles, bulk);
 }

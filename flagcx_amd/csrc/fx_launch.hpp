@@ -32,7 +32,7 @@ struct KernelSet {
 inline uint64_t tilesFor(const void *out, const void *const *in, int k, uint64_t count, int es, int U,
                          void *const *more = nullptr, int nmore = 0) {
   if (count == 0) return 0;
-  return planTiles((uint64_t)(uintptr_t)out, count, es, U, coAlignedHost(out, in, k, more, nmore)).tiles();
+  return planTiles((uint64_t)(uintptr_t)out, count, es, U, handOutFor(coAlignedHost(out, in, k, more, nmore), k)).tiles();
 }
 
 template <class R, int K, int U>

@@ -389,13 +389,24 @@ struct CopyRed {
 // write stream mixed into reads is expensive (measured: 5.9 TB/s for 8 inputs).
 // The same bytes moved as 512-byte pieces 32 KiB apart reach 6.4-6.5 TB/s.  So
 // the part of a segment that consists of whole regions of kStripeTiles tiles,
-// aligned in ABSOLUTE address, is handed out striped when every input shares
-// the output's position within a 128-byte cache line (an input that does not
-// would have a line straddle every 512-byte piece, fetched by two workgroups:
-// counter-measured 1.22-1.25 x the bytes for an input 16 bytes off, and 5.5-6.0
-// against 6.1-6.5 TB/s contiguous): tile i of a region owns
-// piece i of every 32 KiB row of that region.  The rest (head before the first
-// region boundary, tail after the last) is handed out contiguously.
+// aligned in ABSOLUTE address of the output, is handed out striped: tile i of a
+// region owns one 512-byte column of every 32 KiB row of that region.  The rest
+// (head before the first region boundary, tail after the last) is handed out
+// contiguously.
+//
+// Two flavours.  When every stream sits at the output's offset within a
+// 128-byte cache line, a piece is four whole lines in every stream: tile i
+// takes column i and all loads are nontemporal.  When some stream does not, its
+// piece cuts five lines and the fifth is the first line of the next column's
+// piece: then tile i takes column 8 * (i % 8) + i / 8 -- workgroups are dealt
+// round-robin to the eight dies, so eight neighbouring columns land on one die
+// and share its L2 -- and the loads are ordinary (temporal) ones, so that the
+// shared line is still in that L2 when the neighbour asks for it.  Measured on
+// copies of 1-2 GiB whose source is 4-132 bytes off: contiguous tiles 5.6-5.9
+// TB/s; striped by column i with nontemporal loads 5.8 (1.25 x the bytes
+// fetched); grouped columns and temporal loads 6.3-6.4 (1.11 x).  Aligned
+// streams keep column i and nontemporal loads (grouped columns cost 1-2 % for
+// 8 inputs of 512 MiB, temporal loads 4 % for large aligned streams).
 constexpr uint32_t kPieceVecs = 32;                           // 512 bytes
 constexpr uint32_t kStripeTiles = 64;                         // tiles per region
 constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;      // 32 KiB
@@ -415,11 +426,28 @@ struct TilePlan {
   uint64_t firstFull, endFull; // vectors [firstFull, endFull) lie wholly inside the segment
   uint64_t zs, ze;             // striped zone [zs, ze) in vectors; empty when zs == ze
   uint32_t zoneTiles, headTiles, tailTiles;
+  bool grouped;                // striped zone of a segment with a stream off the output's line phase (see above)
   __host__ __device__ uint64_t tiles() const { return (uint64_t)zoneTiles + headTiles + tailTiles; }
 };
 
 // Same function on host (grid size, tile prefix tables) and device (mapping).
-__host__ __device__ inline TilePlan planTiles(uint64_t outAddr, uint64_t count, int es, int U, bool coAligned) {
+// How the whole regions of a segment are handed out.
+enum HandOut {
+  kContiguous = 0,  // not striped at all
+  kStriped = 1,     // tile i owns column i, nontemporal loads: every stream at the output's line phase
+  kGrouped = 2      // eight neighbouring columns per die, temporal loads: a copy whose source is off that phase
+};
+
+// Reductions of several inputs with one off the line phase stay contiguous:
+// measured with every other input off by one element, the grouped flavour
+// (temporal loads for the aligned inputs too) read 6.0-6.2 TB/s for 2 inputs and
+// 6.0 for 4 where contiguous tiles read 6.45-6.58 and 6.37; for 8 inputs the two
+// were equal (6.0).
+__host__ __device__ inline HandOut handOutFor(bool samePhase, int k) {
+  return samePhase ? kStriped : (k == 1 ? kGrouped : kContiguous);
+}
+
+__host__ __device__ inline TilePlan planTiles(uint64_t outAddr, uint64_t count, int es, int U, HandOut how) {
   TilePlan tp;
   const uint64_t V = (uint64_t)U * kBlock, RV = V * kStripeTiles, ve = 16u / (uint32_t)es;
   const uint64_t mis = outAddr & 15u, lead = mis / (uint32_t)es, end = lead + count;
@@ -428,7 +456,8 @@ __host__ __device__ inline TilePlan planTiles(uint64_t outAddr, uint64_t count, 
   tp.endFull = end / ve;
   const uint64_t a0 = (outAddr - mis) >> 4;  // absolute vector number of vector 0
   uint64_t zs = (a0 + tp.firstFull + RV - 1) / RV * RV, ze = (a0 + tp.endFull) / RV * RV;
-  if (!coAligned || ze <= zs || count * (uint64_t)es < kStripeMinBytes) {
+  tp.grouped = (how == kGrouped);
+  if (how == kContiguous || ze <= zs || count * (uint64_t)es < kStripeMinBytes) {
     tp.zs = tp.ze = 0;
   } else {
     tp.zs = zs - a0;
@@ -618,15 +647,23 @@ __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
 }
 
 // Branch-free body: lane handles U whole vectors at byte offsets off + u*ustride
-// of every stream, all K*U loads in flight before the first use.
-template <class R, int K, int U, class SG>
+// of every stream, all K*U loads in flight before the first use.  TEMPORAL picks
+// ordinary loads instead of nontemporal ones (the grouped flavour of the striped
+// zone); it is a template parameter so that the nontemporal body is compiled,
+// and scheduled, exactly as it is without it.
+template <bool TEMPORAL>
+__device__ __forceinline__ u32x4 ldg_as(const void *p) {
+  return TEMPORAL ? ldg_keep(p) : ldg_stream(p);
+}
+
+template <class R, int K, int U, bool TEMPORAL, class SG>
 __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, uint64_t ustride) {
   if (K > 0) {
     u32x4 v[U][K > 0 ? K : 1];
 #pragma unroll
     for (int u = 0; u < U; u++)
 #pragma unroll
-      for (int p = 0; p < K; p++) v[u][p] = ldg_stream(sg.inp(p) + off + u * ustride);
+      for (int p = 0; p < K; p++) v[u][p] = ldg_as<TEMPORAL>(sg.inp(p) + off + u * ustride);
 #pragma unroll
     for (int u = 0; u < U; u++) {
       typename R::Acc acc;
@@ -638,12 +675,12 @@ __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, ui
   } else {
     typename R::Acc acc[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) R::init(acc[u], ldg_stream(sg.inp(0) + off + u * ustride));
+    for (int u = 0; u < U; u++) R::init(acc[u], ldg_as<TEMPORAL>(sg.inp(0) + off + u * ustride));
     for (int p = 1; p < sg.inputs(); p++) {
       const char *ip = sg.inp(p);
       u32x4 v[U];
 #pragma unroll
-      for (int u = 0; u < U; u++) v[u] = ldg_stream(ip + off + u * ustride);
+      for (int u = 0; u < U; u++) v[u] = ldg_as<TEMPORAL>(ip + off + u * ustride);
 #pragma unroll
       for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
     }
@@ -662,13 +699,18 @@ struct TileLane {
   bool fast;
 };
 
-__host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile, uint32_t tid, int U) {
+// xcdShift = (number of the workgroup that executes the tile - tile) mod 8:
+// workgroups are dealt to the eight dies round-robin by their number, and the
+// grouped flavour wants eight neighbouring columns on one die.
+__host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile, uint32_t tid, int U,
+                                               uint32_t xcdShift = 0) {
   const uint64_t V = (uint64_t)U * kBlock;
   TileLane tl;
   if (tile < tp.zoneTiles) {
     // tile i of region r owns vectors zs + r*RV + row*kRowVecs + i*kPieceVecs + [0, kPieceVecs)
     // for row = 0 .. V/kPieceVecs-1; lane (u, tid) takes row u*(kBlock/kPieceVecs) + tid/kPieceVecs.
-    const uint32_t r = tile / kStripeTiles, i = tile % kStripeTiles;
+    const uint32_t r = tile / kStripeTiles, t = tile % kStripeTiles;
+    const uint32_t i = tp.grouped ? ((t + xcdShift) % 8) * (kStripeTiles / 8) + t / 8 : t;   // which column this tile owns
     tl.j = tp.zs + (uint64_t)r * (V * kStripeTiles) + (uint64_t)(tid / kPieceVecs) * kRowVecs + i * kPieceVecs +
            (tid % kPieceVecs);
     tl.stride = (uint64_t)(kBlock / kPieceVecs) * kRowVecs;
@@ -693,11 +735,19 @@ __host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile
 }
 
 // Tile `tile` of the segment: striped zone first, then head, then tail.
+// xcdShift must be the same for every tile of the segment (it decides which
+// column a tile owns in the grouped flavour): a launch whose workgroup b runs
+// tile b - first passes (b - tile) mod 8 = first mod 8, so that the grouping
+// follows the dies; a kernel that hands tiles out differently passes 0.
 template <class R, int K, int U, class SG>
-__device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uint32_t tile) {
-  const TileLane tl = laneOfTile(tp, tile, threadIdx.x, U);
+__device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uint32_t tile, uint32_t xcdShift) {
+  const TileLane tl = laneOfTile(tp, tile, threadIdx.x, U, xcdShift);
   if (tl.fast) {
-    reduceVectorsFast<R, K, U>(sg, tl.j * 16, tl.stride * 16);
+    // The grouped flavour only occurs for one-input segments (handOutFor).
+    if (K == 1 && tp.grouped && tile < tp.zoneTiles)
+      reduceVectorsFast<R, K, U, true>(sg, tl.j * 16, tl.stride * 16);
+    else
+      reduceVectorsFast<R, K, U, false>(sg, tl.j * 16, tl.stride * 16);
   } else {
 #pragma unroll 1
     for (int u = 0; u < U; u++) {
@@ -722,7 +772,7 @@ __device__ __forceinline__ TilePlan makeSeg(Seg<K> &sg, const void *const *in, v
     co = co && sameLinePhase((uint64_t)(uintptr_t)in[p], (uint64_t)(uintptr_t)out);
     sg.in[p] = asGlobal(in[p]) - mis;
   }
-  return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
+  return planTiles((uint64_t)(uintptr_t)out, count, ES, U, handOutFor(co, K));
 }
 
 template <int ES, int U>
@@ -736,7 +786,7 @@ __device__ __forceinline__ TilePlan makeSeg(Seg<0> &sg, const void *const *in, v
   sg.k = k;
   bool co = true;
   for (int p = 0; p < k; p++) co = co && sameLinePhase((uint64_t)(uintptr_t)in[p], (uint64_t)(uintptr_t)out);
-  return planTiles((uint64_t)(uintptr_t)out, count, ES, U, co);
+  return planTiles((uint64_t)(uintptr_t)out, count, ES, U, handOutFor(co, k));
 }
 
 // Host twin of the co-alignment test above; `more` are further outputs.
@@ -762,7 +812,7 @@ template <class R, int K, int U>
 __global__ void __launch_bounds__(kBlock) reduceCopyDirect(DirectArgs<K> a) {
   Seg<K> sg;
   const TilePlan tp = makeSeg<R::ES, U>(sg, a.in, a.out, a.count, a.k);
-  reduceTile<R, K, U>(sg, tp, blockIdx.x);
+  reduceTile<R, K, U>(sg, tp, blockIdx.x, 0u);
 }
 
 // Batched slices: a table of independent segments sharing dtype, op and k.
@@ -818,7 +868,7 @@ __device__ __forceinline__ void reduceSlicesBody(const D *d, const uint32_t *til
   const uint32_t i = findSlice(tileStart, n, b);
   Seg<K> sg;
   const TilePlan tp = makeSeg<R::ES, U>(sg, d[i].in, d[i].out, d[i].count, K);
-  reduceTile<R, K, U>(sg, tp, b - tileStart[i]);
+  reduceTile<R, K, U>(sg, tp, b - tileStart[i], tileStart[i] & 7u);
 }
 
 template <class R, int K, int U, int NS>
@@ -868,7 +918,7 @@ __global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable<NS>
     if (o < sg.nmore) co = co && sameLinePhase((uint64_t)(uintptr_t)d.out[o + 1], (uint64_t)(uintptr_t)d.out[0]);
   }
   const TilePlan tp = makeSeg<R::ES, U>(static_cast<Seg<K> &>(sg), d.in, d.out[0], d.count, K, co);
-  reduceTile<R, K, U>(sg, tp, b - t.tileStart[i]);
+  reduceTile<R, K, U>(sg, tp, b - t.tileStart[i], t.tileStart[i] & 7u);
 }
 
 }  // namespace fx

@@ -152,6 +152,7 @@ def run_pack(dev, a):
     big = [4_194_304] * 8
     bd = [i * 4_194_304 + 0 for i in range(8)]
     dbig, dpk = dev.malloc(8 * 4_194_304 * 4 + 64), dev.malloc(8 * 4_194_304 * 4)
+    dev.memset(dbig, 2, 8 * 4_194_304 * 4 + 64)
     row("pack, 8 x 4,194,304 el aligned", sum(big) * 4, t.ms(lambda: N.check(K.pack(dpk, dbig, big, bd, N.DT_FP32, t.raw))), 2 * sum(big) * 4)
     row("pack, 8 x 4,194,304 el, source off by 1 el", sum(big) * 4,
         t.ms(lambda: N.check(K.pack(dpk, dbig + 4, big, bd, N.DT_FP32, t.raw))), 2 * sum(big) * 4)

@@ -12,8 +12,11 @@
 
 using namespace fx;
 
-static long checkOne(uint64_t outAddr, uint64_t count, int es, int U, bool co) {
-  const TilePlan tp = planTiles(outAddr, count, es, U, co);
+// `shift` plays the part of (workgroup number - tile) mod 8 in a launch whose first workgroup is not tile 0.
+static long checkOne(uint64_t outAddr, uint64_t count, int es, int U, HandOut how, uint32_t shift = 0) {
+  const TilePlan tp = planTiles(outAddr, count, es, U, how);
+  if (tp.grouped != (how == kGrouped)) return 9;
+  if (how == kContiguous && tp.zoneTiles) return 3;          // no striped tiles when asked for none
   const uint64_t ve = 16u / (uint32_t)es, lead = (outAddr & 15u) / (uint32_t)es, end = lead + count;
   if (count == 0) return 0;  // empty segments never reach a kernel (the launchers return first)
   std::vector<unsigned char> seen(tp.nv, 0);
@@ -21,13 +24,12 @@ static long checkOne(uint64_t outAddr, uint64_t count, int es, int U, bool co) {
   for (uint64_t tile = 0; tile < tiles; tile++) {
     bool fast0 = false;
     for (uint32_t tid = 0; tid < (uint32_t)kBlock; tid++) {
-      const TileLane tl = laneOfTile(tp, (uint32_t)tile, tid, U);
+      const TileLane tl = laneOfTile(tp, (uint32_t)tile, tid, U, shift);
       if (tid == 0) fast0 = tl.fast;
       if (tl.fast != fast0) return 2;                       // the path must be uniform in a workgroup
       for (int u = 0; u < U; u++) {
         const uint64_t j = tl.j + (uint64_t)u * tl.stride;
         if (tl.fast) {
-          if (!co && tile < tp.zoneTiles) return 3;           // striped tiles only for co-aligned inputs
           if (j < tp.firstFull || j >= tp.endFull) return 4;  // whole vectors inside the segment only
           if (seen[j]++) return 5;
         } else {
@@ -45,6 +47,13 @@ static long checkOne(uint64_t outAddr, uint64_t count, int es, int U, bool co) {
     const bool overlaps = !(e0 >= end || e0 + ve <= lead);
     if (overlaps != (seen[j] == 1)) return 8;
   }
+  // Grouped flavour: within a region, the workgroups whose number is the same modulo 8 (one die) own eight
+  // neighbouring columns; plain flavour: tile i owns column i.
+  for (uint64_t tile = 0; tile < tp.zoneTiles; tile++) {
+    const uint64_t col = ((laneOfTile(tp, (uint32_t)tile, 0, U, shift).j - tp.zs) % kRowVecs) / kPieceVecs;
+    const uint64_t t = tile % kStripeTiles;
+    if (tp.grouped ? (col / 8 != (t + shift) % 8) : (col != t)) return 10;
+  }
   return 0;
 }
 
@@ -55,7 +64,7 @@ int main() {
                             0x7f0000000000ull + MiB - 16, 0x7f0000000000ull + 3 * MiB + 4096};
   for (int es : {1, 2, 4, 8})
     for (int U : {2, 4, 8})
-      for (bool co : {true, false})
+      for (HandOut co : {kStriped, kGrouped, kContiguous})
         for (uint64_t base : bases)
           for (uint64_t mis = 0; mis < 16; mis += (uint64_t)es * (es == 1 ? 5 : 1)) {
             const uint64_t V = (uint64_t)U * kBlock * 16 / es;   // elements per tile
@@ -70,7 +79,7 @@ int main() {
             }
             if (mis == 0 || mis == 8 || (es == 2 && mis == 2))
               for (uint64_t c : big) {
-                long rc = checkOne(base + mis, c, es, U, co);
+                long rc = checkOne(base + mis, c, es, U, co, (uint32_t)((c + mis + (uint64_t)U) % 8));
                 cases++;
                 if (rc) { printf("FAIL rc=%ld es=%d U=%d co=%d addr=%llx count=%llu\n", rc, es, U, (int)co, (unsigned long long)(base + mis), (unsigned long long)c); return 1; }
               }
@@ -90,9 +99,12 @@ int main() {
     }
     const uint64_t count = (16ull << 20) / 4;
     const void *in1[1] = {o + 16};
-    if (tilesFor(o, in1, 1, count, 4, 4) != (count * 4 + 16383) / 16384 ||          // contiguous: one tile per 16 KiB
-        planTiles((uint64_t)(uintptr_t)o, count, 4, 4, coAlignedHost(o, in1, 1)).zoneTiles != 0 ||
-        planTiles((uint64_t)(uintptr_t)o, count, 4, 4, coAlignedHost(o, same, 3)).zoneTiles == 0) {
+    const TilePlan off = planTiles((uint64_t)(uintptr_t)o, count, 4, 4, handOutFor(coAlignedHost(o, in1, 1), 1));
+    const TilePlan on = planTiles((uint64_t)(uintptr_t)o, count, 4, 4, handOutFor(coAlignedHost(o, same, 3), 3));
+    const TilePlan red = planTiles((uint64_t)(uintptr_t)o, count, 4, 4, handOutFor(coAlignedHost(o, off16, 3), 3));
+    if (tilesFor(o, in1, 1, count, 4, 4) != off.tiles() || off.zoneTiles == 0 || !off.grouped ||    // copy: striped, grouped columns
+        on.zoneTiles != off.zoneTiles || on.grouped ||                                             // same phase: striped, column i
+        red.zoneTiles != 0 || tilesFor(o, off16, 3, count, 4, 4) != (count * 4 + 16383) / 16384) { // reduction off phase: contiguous
       printf("FAIL striping decision\n");
       return 1;
     }

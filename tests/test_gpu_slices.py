@@ -130,6 +130,62 @@ def test_copy_slices_byte_granular(dev):
     assert np.array_equal(got, want)
 
 
+def test_long_copies_at_every_kind_of_line_phase(dev):
+    """Copies long enough for the striped hand-out (4 MiB and more) whose source sits
+    at the destination's offset within a 128-byte line, at another 16-byte multiple,
+    or at an odd byte: several to a launch, so that later ones start at a tile number
+    that is not a multiple of eight, through fx_copy_slices, fx_pack / fx_unpack and the
+    one-input fx_reduce_copy.  Bytes either side of every destination stay untouched."""
+    rng = np.random.default_rng(77)
+    mib = 1 << 20
+    src = rng.integers(0, 256, 40 * mib, dtype=np.uint8)
+    # (src offset, dst offset, bytes)
+    cases = [(0, 0, 5 * mib), (5 * mib + 16, 5 * mib + 64, 4 * mib + 4096), (10 * mib + 48, 10 * mib, 6 * mib + 17),
+             (17 * mib + 1, 17 * mib + 128, 4 * mib + 1), (22 * mib + 64, 22 * mib + 64, 4 * mib),
+             (27 * mib + 100, 27 * mib + 36, 7 * mib - 5), (35 * mib, 35 * mib + 2, 4 * mib + 300)]
+    with DevBufs(dev) as b:
+        dsrc = b.put(src)
+        ddst = b.alloc(src.size)
+        for order in (cases, cases[::-1], cases[3:4]):
+            dev.memset(ddst, 0xEE, src.size)
+            N.check(K.copy_slices([(dsrc + s, ddst + d, n) for s, d, n in order]), "fx_copy_slices")
+            dev.sync()
+            got = dev.to_host(ddst, src.size, np.uint8)
+            want = np.full(src.size, 0xEE, np.uint8)
+            for s, d, n in order:
+                want[d:d + n] = src[s:s + n]
+            assert np.array_equal(got, want)
+        # the same through the typed one-input reduce-copy (fp32: element offsets 0..31 cover every 16-byte phase and
+        # the element-misaligned ones) and through pack / unpack with element displacements
+        s32 = src.view(np.uint32)
+        for so, do, n in ((3, 0, 5 * mib // 4), (4, 8, 4 * mib // 4 + 1), (0, 17, 6 * mib // 4 + 3), (12, 28, 4 * mib // 4)):
+            dev.memset(ddst, 0xEE, src.size)
+            N.check(K.reduce_copy(ddst + 4 * do, [dsrc + 4 * so], n, N.DT_FP32, N.OP_SUM, 0), "fx_reduce_copy k=1")
+            dev.sync()
+            got = dev.to_host(ddst, n + do + 64, np.uint32)
+            assert np.array_equal(got[do:do + n], s32[so:so + n]), (so, do, n)
+            assert (got[:do] == 0xEEEEEEEE).all() and (got[do + n:] == 0xEEEEEEEE).all(), (so, do, n)
+        counts = [mib + 3, 0, 2 * mib, mib // 2, mib + 1, 3 * mib // 2]          # fp32 elements: 4-8 MiB segments and a short one
+        sdispls, pos = [], 5
+        for c in counts:
+            sdispls.append(pos)
+            pos += c + 3
+        total = sum(counts)
+        dpacked = b.alloc(total * 4 + 64)
+        dev.memset(dpacked, 0x77, total * 4 + 64)
+        N.check(K.pack(dpacked, dsrc, counts, sdispls, N.DT_FP32), "fx_pack")
+        dev.memset(ddst, 0xEE, src.size)
+        rdispls = [d + 7 for d in sdispls]
+        N.check(K.unpack(ddst, dpacked, counts, rdispls, N.DT_FP32), "fx_unpack")
+        dev.sync()
+        packed = dev.to_host(dpacked, total + 16, np.uint32)
+        back = dev.to_host(ddst, pos + 64, np.uint32)
+    assert np.array_equal(packed[:total], O.pack(s32, counts, sdispls))
+    assert (packed[total:] == 0x77777777).all()
+    want = O.unpack(np.full(pos + 64, 0xEEEEEEEE, np.uint32), packed[:total], counts, rdispls)
+    assert np.array_equal(back, want)
+
+
 def _random_layout(rng, counts, slack):
     """Random non-overlapping displacements for the given segment counts."""
     order = rng.permutation(len(counts))

@@ -44,13 +44,20 @@ const KernelSet *copySetFor(int es) { return &kernelSetsCopy()[es == 4 ? 2 : (es
 
 bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// Validate one slice and return the number of workgroups it needs.
-flagcxResult_t sliceTiles(const fxSliceDesc &s, int k, int es, int U, uint64_t *tiles) {
-  *tiles = 0;
+// Validate one slice: pointers present and aligned to the element size.
+flagcxResult_t sliceOk(const fxSliceDesc &s, int k, int es) {
   if (s.count == 0) return flagcxSuccess;
   if (!s.out || !aligned(s.out, es)) return flagcxInvalidArgument;
   for (int p = 0; p < k; p++)
     if (!s.in[p] || !aligned(s.in[p], es)) return flagcxInvalidArgument;
+  return flagcxSuccess;
+}
+
+// Validate one slice and return the number of workgroups it needs with U vectors per lane.
+flagcxResult_t sliceTiles(const fxSliceDesc &s, int k, int es, int U, uint64_t *tiles) {
+  *tiles = 0;
+  const flagcxResult_t rc = sliceOk(s, k, es);
+  if (rc != flagcxSuccess || s.count == 0) return rc;
   *tiles = tilesFor(s.out, s.in, k, s.count, es, U);
   return flagcxSuccess;
 }
@@ -92,25 +99,16 @@ flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slices
         if (!slicesIn[i].in[p]) return flagcxInvalidArgument;
     }
   SliceList merged;
-  mergeAdjacent(merged, slicesIn, nIn, k, (size_t)ks->elemSize, div);
-  const int U = unrollFor(k);
-  SmallVec<uint32_t, kFewSlices> tiles;
-  tiles.reserve(merged.size());
-  size_t kept = 0;
+  mergeAdjacent(merged, slicesIn, nIn, k, (size_t)ks->elemSize, div);   // drops empty slices
   for (size_t i = 0; i < merged.size(); i++) {
-    uint64_t t = 0;
-    flagcxResult_t rc = sliceTiles(merged[i], k, ks->elemSize, U, &t);
+    const flagcxResult_t rc = sliceOk(merged[i], k, ks->elemSize);
     if (rc != flagcxSuccess) return rc;
-    if (t == 0) continue;
-    if (t > 0x7ffffff0ull) return flagcxInvalidArgument;
-    merged[kept++] = merged[i];
-    tiles.push_back((uint32_t)t);
   }
-  if (kept == 0) return flagcxSuccess;
+  if (merged.empty()) return flagcxSuccess;
   // A single segment needs no table: the direct kernel's argument block is 100
-  // bytes instead of 4 KiB, which is 1.3 us of an 11 us launch.
-  if (kept == 1) return ks->direct[k](merged[0].out, merged[0].in, k, merged[0].count, s);
-  return ks->slicesInline[k](merged.data(), tiles.data(), kept, s);
+  // bytes instead of the eight-slot table's 700.
+  if (merged.size() == 1) return ks->direct[k](merged[0].out, merged[0].in, k, merged[0].count, s);
+  return ks->slicesInline[k](merged.data(), merged.size(), s);
 }
 
 // Largest power-of-two granularity (4, 2 or 1 bytes) shared by all copy slices.
@@ -360,7 +358,6 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
     const int es = copy ? ((bits & 1) ? 1 : ((bits & 2) ? 2 : 4)) : (int)dtypeSize(dtype);
     if (!copy && (bits & (uintptr_t)(es - 1))) return flagcxInvalidArgument;
     const KernelSet *ks = copy ? copySetFor(es) : setFor(dtype, op);
-    const int U = unrollFor(k);
     // merge slices that continue each other in every stream
     SmallVec<fxBcastDesc, kFewSlices> merged;
     merged.reserve(n);
@@ -383,7 +380,6 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
     }
     SliceList plainReduce, plainCopy;  // slices whose outputs are not co-aligned
     SmallVec<BcastDescDev, kFewSlices> dev;
-    SmallVec<uint32_t, kFewSlices> devTiles;
     for (const fxBcastDesc &d : merged) {
       bool same = true;
       for (int o = 1; o < nout; o++) same = same && (((uintptr_t)d.out[o] & 15u) == ((uintptr_t)d.out[0] & 15u));
@@ -404,17 +400,14 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
         }
         continue;
       }
-      const uint64_t tiles = tilesFor(d.out[0], d.in, k, d.count, es, U, d.out + 1, nout - 1);
-      if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
       BcastDescDev dd;
       for (int p = 0; p < kMaxFixedK; p++) dd.in[p] = (p < k) ? d.in[p] : nullptr;
       for (int o = 0; o < kMaxFixedK; o++) dd.out[o] = (o < nout) ? d.out[o] : nullptr;
       dd.count = d.count;
       dd.nout = (uint32_t)nout;
       dev.push_back(dd);
-      devTiles.push_back((uint32_t)tiles);
     }
-    flagcxResult_t rc = dev.empty() ? flagcxSuccess : ks->bcastInline[k](dev.data(), devTiles.data(), dev.size(), s);
+    flagcxResult_t rc = dev.empty() ? flagcxSuccess : ks->bcastInline[k](dev.data(), dev.size(), s);
     if (rc != flagcxSuccess) return rc;
     if (!plainReduce.empty()) {
       rc = launchSliceBatches(ks, plainReduce.data(), plainReduce.size(), k, s);

@@ -7,24 +7,36 @@
 
 namespace fx {
 
-// Vectors per lane per input.  Measured on MI355X at 512 MiB per stream, 4 is
-// the best or within 1 % of it for every k; 8 inputs gain 2 % more with 8
-// (256 VGPRs) once the launch is large enough not to miss the extra workgroups
-// and every input is aligned like the output (unaligned: 4 is 7-10 % faster).
-constexpr int unrollFor(int K) { return K == 0 ? 2 : 4; }
+// Vectors per lane per input, measured on MI355X.
+//  * Large launches: 4, or 2 for one and two inputs (a copy gains 1 %, a
+//    two-input sum 1.5-3.5 % from 64 MiB per input upwards); 8 inputs gain
+//    another 1-2 % with 8 (256 VGPRs) once the launch is large enough not to
+//    miss the extra workgroups and every input is aligned like the output
+//    (unaligned: 4 is 7-10 % faster).
+//  * Launches of less than 4 MiB of output: 1 for three inputs and more.
+//    With 4, such a launch has fewer workgroups than the device has compute
+//    units and each lane waits for 32 loads: an eight-input reduction of
+//    1 MiB per input takes 4.8 us against 2.9 us, the eight-rank all-reduce
+//    of 64 KiB per rank 6.2 against 4.3 us.  At large sizes 1 is 0.5-4 %
+//    slower than 4, so both exist.
+constexpr int unrollFor(int K) { return K <= 2 ? 2 : 4; }
+constexpr int smallUnrollFor(int K) { return K >= 3 ? 1 : unrollFor(K); }
 constexpr int bigUnrollFor(int K) { return K == 8 ? 8 : unrollFor(K); }
 constexpr uint64_t kBigLaunchTiles = 1024;  // use bigUnrollFor only above this many of its tiles (32 MiB per input)
+constexpr uint64_t kSmallLaunchVecs = 256 * 1024;  // fewer 16-byte vectors of output than this: smallUnrollFor
+
+inline uint64_t vectorsOf(uint64_t count, int es) { return (count * (uint64_t)es + 15) / 16; }
 
 struct KernelSet {
   // index = compile-time input count, 0 = runtime-k kernel
   flagcxResult_t (*direct[kMaxFixedK + 1])(void *out, const void *const *in, int k, uint64_t count, hipStream_t s);
-  // n slices with their tile counts (all non-zero), as many launches as their kernel-argument tables need
-  flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const fxSliceDesc *slices, const uint32_t *tiles, size_t n,
-                                                 hipStream_t s);
+  // n validated, non-empty slices; as many launches as their kernel-argument tables need
+  flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const fxSliceDesc *slices, size_t n, hipStream_t s);
+  // device-resident tables, tile counts made with unrollFor(k)
   flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
                                                 uint32_t grid, hipStream_t s);
-  // n multi-output slices with their tile counts (all non-zero)
-  flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const BcastDescDev *d, const uint32_t *tiles, size_t n, hipStream_t s);
+  // n validated, non-empty multi-output slices
+  flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const BcastDescDev *d, size_t n, hipStream_t s);
   int elemSize;
 };
 
@@ -51,22 +63,28 @@ flagcxResult_t launchDirectU(void *out, const void *const *in, int k, uint64_t c
 
 template <class R, int K>
 flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t count, hipStream_t s) {
-  constexpr int UB = bigUnrollFor(K);
-  if (UB != unrollFor(K) && coAlignedHost(out, in, (K > 0) ? K : k) &&
-      tilesFor(out, in, (K > 0) ? K : k, count, R::ES, UB) >= kBigLaunchTiles)
-    return launchDirectU<R, K, UB>(out, in, k, count, s);
-  return launchDirectU<R, K, unrollFor(K)>(out, in, k, count, s);
+  constexpr int US = smallUnrollFor(K), UD = unrollFor(K), UB = bigUnrollFor(K);
+  if constexpr (US != UD)
+    if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
+  if constexpr (UB != UD)
+    if (coAlignedHost(out, in, (K > 0) ? K : k) && tilesFor(out, in, (K > 0) ? K : k, count, R::ES, UB) >= kBigLaunchTiles)
+      return launchDirectU<R, K, UB>(out, in, k, count, s);
+  return launchDirectU<R, K, UD>(out, in, k, count, s);
 }
 
-template <class R, int K, int NS>
-flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, const uint32_t *tiles, size_t n, hipStream_t s) {
-  constexpr int U = unrollFor(K);
+template <class R, int K, int U, int NS>
+flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, size_t n, hipStream_t s) {
   InlineSliceTable<K, NS> t;
   t.n = 0;
   t.tileStart[0] = 0;
   for (size_t i = 0; i <= n; i++) {
+    uint64_t tiles = 0;
+    if (i < n) {
+      tiles = tilesFor(slices[i].out, slices[i].in, K, slices[i].count, R::ES, U);
+      if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+    }
     const bool full = t.n == (uint32_t)InlineSliceTable<K, NS>::kSlots ||
-                      (i < n && (uint64_t)t.tileStart[t.n] + tiles[i] > 0x7ffffff0ull);
+                      (i < n && (uint64_t)t.tileStart[t.n] + tiles > 0x7ffffff0ull);
     if ((i == n || full) && t.n > 0) {
       const flagcxResult_t rc = launchKernel(reduceSlicesInline<R, K, U, NS>, t.tileStart[t.n], s, t);
       if (rc != flagcxSuccess) return rc;
@@ -77,16 +95,22 @@ flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, const uint32_t
     for (int p = 0; p < K; p++) d.in[p] = slices[i].in[p];
     d.out = slices[i].out;
     d.count = slices[i].count;
-    t.tileStart[t.n + 1] = t.tileStart[t.n] + tiles[i];
+    t.tileStart[t.n + 1] = t.tileStart[t.n] + (uint32_t)tiles;
     t.n++;
   }
   return flagcxSuccess;
 }
 
 template <class R, int K>
-flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, const uint32_t *tiles, size_t n, hipStream_t s) {
-  if (n <= (size_t)kSmallSliceTable) return launchSlicesInlineSized<R, K, kSmallSliceTable>(slices, tiles, n, s);
-  return launchSlicesInlineSized<R, K, 0>(slices, tiles, n, s);
+flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, size_t n, hipStream_t s) {
+  constexpr int US = smallUnrollFor(K), UD = unrollFor(K);
+  if (n > (size_t)kSmallSliceTable) return launchSlicesInlineSized<R, K, UD, 0>(slices, n, s);
+  if constexpr (US != UD) {
+    uint64_t vecs = 0;
+    for (size_t i = 0; i < n; i++) vecs += vectorsOf(slices[i].count, R::ES);
+    if (vecs < kSmallLaunchVecs) return launchSlicesInlineSized<R, K, US, kSmallSliceTable>(slices, n, s);
+  }
+  return launchSlicesInlineSized<R, K, UD, kSmallSliceTable>(slices, n, s);
 }
 
 template <class R, int K>
@@ -97,30 +121,48 @@ flagcxResult_t launchSlicesTable(const SliceDescDev *d, const uint32_t *tileStar
   return launchKernel(reduceSlicesTable<R, K, U>, grid, s, d, tileStart, n);
 }
 
+inline uint64_t bcastTiles(const BcastDescDev &d, int k, int es, int U) {
+  return tilesFor(d.out[0], d.in, k, d.count, es, U, d.out + 1, (int)d.nout - 1);
+}
+
+template <class R, int K, int U>
+flagcxResult_t launchBcastOne(const BcastDescDev &d, hipStream_t s) {  // the one-slot table
+  const uint64_t tiles = bcastTiles(d, K, R::ES, U);
+  if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+  InlineBcastTable<1> t;
+  t.d[0] = d;
+  t.tileStart[0] = 0;
+  t.tileStart[1] = (uint32_t)tiles;
+  t.n = 1;
+  return launchKernel(reduceBcastInline<R, K, U, 1>, (uint32_t)tiles, s, t);
+}
+
 template <class R, int K>
-flagcxResult_t launchBcastInline(const BcastDescDev *d, const uint32_t *tiles, size_t n, hipStream_t s) {
-  constexpr int U = unrollFor(K);
-  if (n == 1) {  // the small table
-    InlineBcastTable<1> t;
-    t.d[0] = d[0];
-    t.tileStart[0] = 0;
-    t.tileStart[1] = tiles[0];
-    t.n = 1;
-    return launchKernel(reduceBcastInline<R, K, U, 1>, tiles[0], s, t);
+flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s) {
+  constexpr int US = smallUnrollFor(K), UD = unrollFor(K);
+  if (n == 1) {
+    if constexpr (US != UD)
+      if (vectorsOf(d[0].count, R::ES) < kSmallLaunchVecs) return launchBcastOne<R, K, US>(d[0], s);
+    return launchBcastOne<R, K, UD>(d[0], s);
   }
   InlineBcastTable<kInlineBcast> t;
   t.n = 0;
   t.tileStart[0] = 0;
   for (size_t i = 0; i <= n; i++) {
-    const bool full = t.n == (uint32_t)kInlineBcast || (i < n && (uint64_t)t.tileStart[t.n] + tiles[i] > 0x7ffffff0ull);
+    uint64_t tiles = 0;
+    if (i < n) {
+      tiles = bcastTiles(d[i], K, R::ES, UD);
+      if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+    }
+    const bool full = t.n == (uint32_t)kInlineBcast || (i < n && (uint64_t)t.tileStart[t.n] + tiles > 0x7ffffff0ull);
     if ((i == n || full) && t.n > 0) {
-      const flagcxResult_t rc = launchKernel(reduceBcastInline<R, K, U, kInlineBcast>, t.tileStart[t.n], s, t);
+      const flagcxResult_t rc = launchKernel(reduceBcastInline<R, K, UD, kInlineBcast>, t.tileStart[t.n], s, t);
       if (rc != flagcxSuccess) return rc;
       t.n = 0;
     }
     if (i == n) break;
     t.d[t.n] = d[i];
-    t.tileStart[t.n + 1] = t.tileStart[t.n] + tiles[i];
+    t.tileStart[t.n + 1] = t.tileStart[t.n] + (uint32_t)tiles;
     t.n++;
   }
   return flagcxSuccess;

@@ -63,7 +63,7 @@ int main() {
   const uint64_t bases[] = {0x7f0000000000ull, 0x7f0000000000ull + 512, 0x7f0000000000ull + 96 * 1024 + 16,
                             0x7f0000000000ull + MiB - 16, 0x7f0000000000ull + 3 * MiB + 4096};
   for (int es : {1, 2, 4, 8})
-    for (int U : {2, 4, 8})
+    for (int U : {1, 2, 4, 8})
       for (HandOut co : {kStriped, kGrouped, kContiguous})
         for (uint64_t base : bases)
           for (uint64_t mis = 0; mis < 16; mis += (uint64_t)es * (es == 1 ? 5 : 1)) {

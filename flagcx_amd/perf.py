@@ -249,8 +249,9 @@ def run_fifo(dev, a):
         lib.fx_fifo_consumer_destroy(cons)
 
 
-def _replay_of(t, post):
-    """Capture what `post` enqueues on the timer's stream into a HIP graph once; the returned function replays it."""
+def _replay_of(t, post, calls=1):
+    """Capture what `calls` calls of `post` enqueue on the timer's stream into a HIP graph once; the returned
+    function replays it."""
     import ctypes as C
     hip = C.CDLL("libamdhip64.so.7")          # the runtime the library is linked against (same mapping)
     hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
@@ -263,7 +264,8 @@ def _replay_of(t, post):
     if hip.hipStreamBeginCapture(t.raw, 0) != 0:
         raise RuntimeError("hipStreamBeginCapture failed")
     try:
-        post()
+        for _ in range(calls):
+            post()
     finally:
         rc = hip.hipStreamEndCapture(t.raw, C.byref(graph))
     if rc != 0 or hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) != 0:
@@ -288,7 +290,7 @@ def run_allreduce(dev, a):
             while nbytes <= emax:
                 cnt = nbytes // es
                 post = lambda: N.check(g.all_reduce(ds, dr, cnt, dtype, OP[a.op], t.stream))
-                ms = t.ms(_replay_of(t, post)) if a.graph else t.ms(post)
+                ms = t.ms(_replay_of(t, post, a.graph_calls)) / a.graph_calls if a.graph else t.ms(post)
                 alg = nbytes / ms / 1e6
                 # algBw = size / time, busBw = algBw * 2 (n - 1) / n, as test/perf/host_api/test_allreduce.cpp:11
                 print(f"{'allreduce n=%d %s %s' % (n, a.dtype, ('ring' if algo else 'direct') + (' graph' if a.graph else '')):<44s} size {nbytes:>12d} B   "
@@ -308,6 +310,7 @@ def main(argv=None):
     ap.add_argument("-f", "--factor", type=int, default=2)
     ap.add_argument("--inplace", action="store_true")
     ap.add_argument("--graph", action="store_true", help="allreduce: capture one call into a HIP graph and time replays")
+    ap.add_argument("--graph-calls", type=int, default=1, help="allreduce --graph: calls captured into the one graph")
     ap.add_argument("--misalign", type=int, default=0, help="shift buffers by this many elements")
     ap.add_argument("--mixed", action="store_true", help="shift only every other input (inputs not aligned like the output)")
     ap.add_argument("--stride", default="",

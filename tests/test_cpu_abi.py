@@ -393,3 +393,17 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode == 2 and "--gpus must be 1" in r.stderr and r.stdout == ""
+
+
+def test_torch_backend_module_loads_and_fails_loudly_without_a_gpu():
+    """The c10d backend module imports against the installed torch, exports its
+    factory, and a rank that cannot reach a GPU raises instead of falling back."""
+    torch = pytest.importorskip("torch")
+    import torch.distributed as dist
+    import flagcx_amd.torch_backend as fxb
+    ext = fxb.extension()
+    assert callable(ext.create_backend)
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is visible: the refusal cannot be shown")
+    with pytest.raises(RuntimeError, match="flagcxCommInitRank failed"):
+        fxb.new_backend(dist.HashStore(), 0, 2)

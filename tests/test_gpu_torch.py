@@ -22,3 +22,14 @@ def test_torch_tensors_and_streams(dev):
     r = subprocess.run([sys.executable, "-u", os.path.join(ROOT, "tests", "torch_client.py")], cwd=ROOT, env=env,
                        capture_output=True, text=True, timeout=420)
     assert r.returncode == 0 and "torch client ok" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]
+
+
+def test_torch_distributed_backend(dev):
+    """torch.distributed's collectives through the "flagcx" c10d backend module
+    (flagcx_amd/torch_backend): 4 and 8 simulated ranks, and a one-rank process group."""
+    if importlib.util.find_spec("torch") is None:
+        pytest.skip("torch is not installed")
+    env = dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    r = subprocess.run([sys.executable, "-u", os.path.join(ROOT, "tests", "torch_backend_client.py")], cwd=ROOT, env=env,
+                       capture_output=True, text=True, timeout=420)
+    assert r.returncode == 0 and "torch backend ok" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]

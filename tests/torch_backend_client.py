@@ -216,9 +216,19 @@ def one_rank(gen):
         dist.barrier()
         torch.cuda.synchronize()
         assert torch.equal(t, keep)
+        # DistributedDataParallel: parameter broadcast, shape check and gradient buckets all go through the backend
+        torch.manual_seed(0)
+        model = torch.nn.Sequential(torch.nn.Linear(64, 128), torch.nn.ReLU(), torch.nn.Linear(128, 8)).cuda()
+        ddp = torch.nn.parallel.DistributedDataParallel(model, device_ids=[0])
+        x = torch.randn(32, 64, device="cuda")
+        ddp(x).square().mean().backward()
+        grads = [p.grad.clone() for p in model.parameters()]
+        model.zero_grad()
+        model(x).square().mean().backward()
+        assert all(torch.equal(g, p.grad) for g, p in zip(grads, model.parameters())), "DDP gradients differ"
     finally:
         dist.destroy_process_group()
-    print("ok  init_process_group('flagcx'), world_size 1", flush=True)
+    print("ok  init_process_group('flagcx'), world_size 1, module API and DistributedDataParallel", flush=True)
 
 
 def main():

@@ -298,9 +298,51 @@ def run_allreduce(dev, a):
                 nbytes *= a.factor
 
 
+def run_torchref():
+    """PyTorch's own kernels on the same shapes, as a reference point on the same box: torch.add(out=) for the
+    two-input sum, Tensor.copy_ for the copy, and the 8-input bf16 sum done the torch way.  Uses torch only."""
+    import torch
+    torch.cuda.set_device(0)
+
+    def ms_of(fn, iters):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            e1.synchronize()
+            best = min(best, e0.elapsed_time(e1) / iters)
+        return best
+
+    for dt, es in ((torch.float32, 4), (torch.bfloat16, 2)):
+        for mib in (64, 256, 512):
+            n = (mib << 20) // es
+            a, b = torch.randn(n, device="cuda").to(dt), torch.randn(n, device="cuda").to(dt)
+            c = torch.empty_like(a)
+            row(f"torch.add(a, b, out=c) {str(dt)[6:]}", mib << 20, ms_of(lambda: torch.add(a, b, out=c), 50), 3 * (mib << 20))
+            row(f"c.copy_(a) {str(dt)[6:]}", mib << 20, ms_of(lambda: c.copy_(a), 50), 2 * (mib << 20))
+            del a, b, c
+    n = (512 << 20) // 2
+    xs = [torch.randn(n, device="cuda").to(torch.bfloat16) for _ in range(8)]
+    out = torch.empty_like(xs[0])
+
+    def chain():
+        torch.add(xs[0], xs[1], out=out)
+        for x in xs[2:]:
+            out.add_(x)
+    row("8 x bf16 as 7 torch adds (one-pass bytes)", 512 << 20, ms_of(chain, 10), 9 * (512 << 20))
+    st = torch.stack(xs)
+    row("torch.sum(stacked [8, n] bf16, 0, out=)", 512 << 20, ms_of(lambda: torch.sum(st, 0, out=out), 10), 9 * (512 << 20))
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo"])
+    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo", "torchref"])
     ap.add_argument("-k", type=int, default=4)
     ap.add_argument("-n", "--nranks", type=int, default=8)
     ap.add_argument("-d", "--dtype", default="fp32", choices=list(DT))
@@ -318,6 +360,8 @@ def main(argv=None):
     ap.add_argument("--in-shift", type=int, default=0,
                     help="start input i at byte offset i*IN_SHIFT of its allocation (multiple of 16 keeps vector loads)")
     a = ap.parse_args(argv)
+    if a.what == "torchref":         # torch brings its own HIP runtime: nothing of this library is loaded beside it
+        return run_torchref()
     dev = Device(0)
     {"reduce": run_reduce, "slices": run_slices, "pack": run_pack, "allreduce": run_allreduce,
      "fifo": run_fifo}[a.what](dev, a)

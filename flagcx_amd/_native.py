@@ -137,6 +137,8 @@ _SIGS.update({
     # include/flagcx_amd/fx_host_staged.h
     "fxHostStagedCreate": (_i, [C.POINTER(_vp), _i, _vp]),
     "fxHostStagedAllReduce": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _i, _i, C.POINTER(C.c_uint64)]),
+    "fxHostStagedReduce": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _i, _i, _i, C.POINTER(C.c_uint64)]),
+    "fxHostStagedReduceScatter": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _i, _i, C.POINTER(C.c_uint64)]),
     "fxHostStagedDestroy": (_i, [_vp]),
     "fx_part_ring_ar": (_sz, [_sz, _i, _i, _sz, _sz, C.POINTER(RedNode)]),
     "fx_part_ring_rs": (_sz, [_sz, _i, _i, _sz, _sz, C.POINTER(RedNode)]),

@@ -1,6 +1,8 @@
-// Host-staged all-reduce over simulated ranks, with per-phase timers: the
-// reference's CPU path end to end (flagcx/runner/host_runner.cc:236-289 on top
-// of flagcx/service/bootstrap.cc:787-942), one host thread per rank.
+// Host-staged reducing collectives over simulated ranks, with per-phase timers:
+// the reference's CPU path end to end -- hostRunnerAllReduce, hostRunnerReduce and
+// hostRunnerReduceScatter (flagcx/runner/host_runner.cc:236-289, 12-67, 291-346)
+// on top of the bootstrap ring (flagcx/service/bootstrap.cc:787-1066) -- one host
+// thread per rank.
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -134,21 +136,27 @@ flagcxResult_t moveBytes(const fxHostStaged *h, void *dst, const void *src, size
   return hipMemcpy(dst, src, bytes, kind) == hipSuccess ? flagcxSuccess : flagcxUnhandledDeviceError;
 }
 
+enum Kind { kAllReduce, kReduce, kReduceScatter };
+
 // One rank's whole call.  Every rank runs the same number of meetings whatever
-// its chunk lengths are, so nobody is left waiting.
-void rankMain(fxHostStaged *h, Meeting *meet, int rank, const void *sendDev, void *recvDev, size_t count, int dtype,
-              int op, uint64_t *t, std::atomic<int> *failed) {
+// its chunk lengths are, so nobody is left waiting.  `count` is the element
+// count of the call: per rank for all-reduce and reduce, the receive count for
+// reduce-scatter (the send side then holds n times as much).
+void rankMain(fxHostStaged *h, Meeting *meet, Kind kind, int root, int rank, const void *sendDev, void *recvDev,
+              size_t count, int dtype, int op, uint64_t *t, std::atomic<int> *failed) {
   const int n = h->n;
   RankState &me = h->ranks[(size_t)rank];
   const RankState &prev = h->ranks[(size_t)((rank + n - 1) % n)];
-  const size_t ts = fx::dtypeSize(dtype), size = count * ts;
+  const size_t ts = fx::dtypeSize(dtype);
+  const size_t outSize = count * ts;                                         // what this rank receives
+  const size_t size = (kind == kReduceScatter) ? outSize * (size_t)n : outSize;   // what it sends
   auto fail = [&](flagcxResult_t rc) { int zero = 0; failed->compare_exchange_strong(zero, (int)rc); };
   (void)hipSetDevice(h->device);
   t[FX_TIMER_COLL_TOTAL] = nowNs();
 
   // step 1: staged buffers
   uint64_t t0 = nowNs();
-  bool ok = growTo(&me.in, &me.inBytes, size) && growTo(&me.out, &me.outBytes, size);
+  bool ok = growTo(&me.in, &me.inBytes, size) && growTo(&me.out, &me.outBytes, size);   // the ring works in `out`
   t[FX_TIMER_COLL_ALLOC] = nowNs() - t0;
   if (!ok) fail(flagcxSystemError);
 
@@ -160,15 +168,19 @@ void rankMain(fxHostStaged *h, Meeting *meet, int rank, const void *sendDev, voi
   }
   t[FX_TIMER_COLL_MEM_D2H] = nowNs() - t0;
 
-  // step 3: the ring all-reduce on the host
+  // step 3: the ring collective on the host
   t0 = nowNs();
-  // chunk i: ceil(size / n) bytes rounded up to whole elements, the last non-empty one short, later ones empty
+  // all-reduce, reduce: chunk i is ceil(size / n) bytes rounded up to whole elements, the last non-empty one short,
+  // later ones empty (bootstrap.cc:900-922, 951-971); reduce-scatter: chunk i is rank i's recvcount elements (:1058-1061)
   size_t chunkBytes = (size + (size_t)n - 1) / (size_t)n;
   chunkBytes = (chunkBytes + ts - 1) / ts * ts;
   std::vector<size_t> offset((size_t)n, 0), length((size_t)n, 0);
   size_t longest = 0;
   for (size_t i = 0; i < (size_t)n; i++) {
-    if (chunkBytes * i >= size) {
+    if (kind == kReduceScatter) {
+      offset[i] = i * outSize;
+      length[i] = outSize;
+    } else if (chunkBytes * i >= size) {
       offset[i] = size;
       length[i] = 0;
     } else {
@@ -186,37 +198,51 @@ void rankMain(fxHostStaged *h, Meeting *meet, int rank, const void *sendDev, voi
   const bool run = failed->load() == 0;
   const char *sendbuff = me.in;
   char *recvbuff = me.out;
-  // reduce-scatter: n-1 steps; the partial of chunk c travels c+1 -> c+2 -> .. -> c
-  for (int iter = 0; iter < n - 1; iter++) {
-    const size_t sendNo = (size_t)((rank + 2 * n - iter - 1) % n), recvNo = (size_t)((rank + 2 * n - iter - 2) % n);
-    if (run && length[sendNo]) {
-      const uint64_t m0 = nowNs();
-      if (iter == 0) memcpy(me.forSend, sendbuff + offset[sendNo], length[sendNo]);
-      else std::swap(me.forSend, me.forRecv);
-      t[FX_TIMER_COLL_MEM] += nowNs() - m0;
+  if (n == 1) {   // one rank: the collective is a copy (bootstrap.cc:1006-1011, 1027-1032, 1049-1054)
+    if (run) memcpy(recvbuff, sendbuff, outSize);
+  } else {
+    // reduce-scatter: n-1 steps; the partial of chunk c travels c+1 -> c+2 -> .. -> c
+    for (int iter = 0; iter < n - 1; iter++) {
+      const size_t sendNo = (size_t)((rank + 2 * n - iter - 1) % n), recvNo = (size_t)((rank + 2 * n - iter - 2) % n);
+      if (run && length[sendNo]) {
+        const uint64_t m0 = nowNs();
+        if (iter == 0) memcpy(me.forSend, sendbuff + offset[sendNo], length[sendNo]);
+        else std::swap(me.forSend, me.forRecv);
+        t[FX_TIMER_COLL_MEM] += nowNs() - m0;
+      }
+      me.sending.store(me.forSend, std::memory_order_release);
+      meet->arrive();                             // the neighbours' send buffers are ready
+      if (run && length[recvNo]) {                // "receive": the chunk the previous rank sends is the one we expect
+        memcpy(me.forRecv, prev.sending.load(std::memory_order_acquire), length[recvNo]);
+      }
+      meet->arrive();                             // everybody has taken its chunk: send buffers may be reused
+      if (run && length[recvNo]) {
+        const uint64_t c0 = nowNs();
+        hostReduce(dtype, op, me.forRecv, sendbuff + offset[recvNo], me.forRecv, length[recvNo] / ts);
+        t[FX_TIMER_COLL_CALC] += nowNs() - c0;
+      }
     }
-    me.sending.store(me.forSend, std::memory_order_release);
-    meet->arrive();                             // the neighbours' send buffers are ready
-    if (run && length[recvNo]) {                // "receive": the chunk the previous rank sends is the one we expect
-      memcpy(me.forRecv, prev.sending.load(std::memory_order_acquire), length[recvNo]);
+    if (run) memcpy(recvbuff, me.forRecv, length[(size_t)rank]);   // this rank's reduced chunk, at the front
+    if (kind != kReduceScatter) {
+      if (run) memmove(recvbuff + offset[(size_t)rank], recvbuff, length[(size_t)rank]);   // to its place
+      if (kind == kAllReduce) {
+        // all-gather: step i, this rank takes chunk (rank - i - 1) from the previous rank's receive buffer
+        for (int i = 0; i < n - 1; i++) {
+          meet->arrive();
+          const size_t rslice = (size_t)((rank - i - 1 + 2 * n) % n);
+          if (run && length[rslice]) memcpy(recvbuff + offset[rslice], prev.out + offset[rslice], length[rslice]);
+          meet->arrive();
+        }
+      } else {
+        // gather to the root: every other rank hands over its chunk (bootstrap.cc:980-993)
+        meet->arrive();
+        if (run && rank == root)
+          for (int i = 0; i < n; i++)
+            if (i != rank && length[(size_t)i])
+              memcpy(recvbuff + offset[(size_t)i], h->ranks[(size_t)i].out + offset[(size_t)i], length[(size_t)i]);
+        meet->arrive();
+      }
     }
-    meet->arrive();                             // everybody has taken its chunk: send buffers may be reused
-    if (run && length[recvNo]) {
-      const uint64_t c0 = nowNs();
-      hostReduce(dtype, op, me.forRecv, sendbuff + offset[recvNo], me.forRecv, length[recvNo] / ts);
-      t[FX_TIMER_COLL_CALC] += nowNs() - c0;
-    }
-  }
-  if (run) {
-    memcpy(recvbuff, me.forRecv, length[(size_t)rank]);
-    memmove(recvbuff + offset[(size_t)rank], recvbuff, length[(size_t)rank]);
-  }
-  // all-gather: step i, this rank takes chunk (rank - i - 1) from the previous rank's receive buffer
-  for (int i = 0; i < n - 1; i++) {
-    meet->arrive();
-    const size_t rslice = (size_t)((rank - i - 1 + 2 * n) % n);
-    if (run && length[rslice]) memcpy(recvbuff + offset[rslice], prev.out + offset[rslice], length[rslice]);
-    meet->arrive();
   }
   free(me.forSend);
   free(me.forRecv);
@@ -225,8 +251,8 @@ void rankMain(fxHostStaged *h, Meeting *meet, int rank, const void *sendDev, voi
 
   // step 4: host to device
   t0 = nowNs();
-  if (run) {
-    const flagcxResult_t rc = moveBytes(h, recvDev, me.out, size, flagcxMemcpyHostToDevice);
+  if (run && (kind != kReduce || rank == root)) {   // a reduce lands on the root only (host_runner.cc:46-49)
+    const flagcxResult_t rc = moveBytes(h, recvDev, me.out, outSize, flagcxMemcpyHostToDevice);
     if (rc != flagcxSuccess) fail(rc);
   }
   t[FX_TIMER_COLL_MEM_H2D] = nowNs() - t0;
@@ -256,12 +282,16 @@ int fxHostStagedCreate(fxHostStaged_t *h, int nranks, fxDeviceMemcpyFn memcpyFn)
   });
 }
 
-int fxHostStagedAllReduce(fxHostStaged_t h, const void *const *sendbuffs, void *const *recvbuffs, size_t count,
-                          int dtype, int op, uint64_t *timers) {
+namespace {
+int runStaged(fxHostStaged_t h, Kind kind, int root, const void *const *sendbuffs, void *const *recvbuffs, size_t count,
+              int dtype, int op, uint64_t *timers) {
   if (!h || !sendbuffs || !recvbuffs) return flagcxInvalidArgument;
   if (!carried(dtype, op)) return flagcxInvalidArgument;   // as the reference's host loops
-  for (int r = 0; r < h->n; r++)
-    if (count && (!sendbuffs[r] || !recvbuffs[r])) return flagcxInvalidArgument;
+  if (kind == kReduce && (root < 0 || root >= h->n)) return flagcxInvalidArgument;
+  for (int r = 0; r < h->n; r++) {
+    const bool receives = kind != kReduce || r == root;
+    if (count && (!sendbuffs[r] || (receives && !recvbuffs[r]))) return flagcxInvalidArgument;
+  }
   return fx::guarded([&]() -> int {
     const int n = h->n;
     std::vector<uint64_t> local((size_t)n * FX_TIMERS_COLL_COUNT, 0);
@@ -272,11 +302,27 @@ int fxHostStagedAllReduce(fxHostStaged_t h, const void *const *sendbuffs, void *
     std::vector<std::thread> threads;
     threads.reserve((size_t)n);
     for (int r = 0; r < n; r++)
-      threads.emplace_back(rankMain, h, &meet, r, sendbuffs[r], recvbuffs[r], count, dtype, op,
+      threads.emplace_back(rankMain, h, &meet, kind, root, r, sendbuffs[r], recvbuffs[r], count, dtype, op,
                            t + (size_t)r * FX_TIMERS_COLL_COUNT, &failed);
     for (auto &th : threads) th.join();
     return failed.load();
   });
+}
+}  // namespace
+
+int fxHostStagedAllReduce(fxHostStaged_t h, const void *const *sendbuffs, void *const *recvbuffs, size_t count,
+                          int dtype, int op, uint64_t *timers) {
+  return runStaged(h, kAllReduce, 0, sendbuffs, recvbuffs, count, dtype, op, timers);
+}
+
+int fxHostStagedReduce(fxHostStaged_t h, const void *const *sendbuffs, void *const *recvbuffs, size_t count, int dtype,
+                       int op, int root, uint64_t *timers) {
+  return runStaged(h, kReduce, root, sendbuffs, recvbuffs, count, dtype, op, timers);
+}
+
+int fxHostStagedReduceScatter(fxHostStaged_t h, const void *const *sendbuffs, void *const *recvbuffs, size_t recvcount,
+                              int dtype, int op, uint64_t *timers) {
+  return runStaged(h, kReduceScatter, 0, sendbuffs, recvbuffs, recvcount, dtype, op, timers);
 }
 
 int fxHostStagedDestroy(fxHostStaged_t h) {

@@ -82,8 +82,8 @@ class SimGroup:
 
 
 class HostStaged:
-    """The reference's host-staged all-reduce over n simulated ranks
-    (include/flagcx_amd/fx_host_staged.h): D2H, ring all-reduce on the host, H2D,
+    """The reference's host-staged reducing collectives over n simulated ranks
+    (include/flagcx_amd/fx_host_staged.h): D2H, the bootstrap ring on the host, H2D,
     with the reference's per-phase timers."""
 
     def __init__(self, nranks, device_memcpy=None):
@@ -92,13 +92,28 @@ class HostStaged:
         fn = C.cast(device_memcpy, C.c_void_p) if device_memcpy is not None else None
         N.check(lib.fxHostStagedCreate(C.byref(self.h), nranks, fn), "fxHostStagedCreate")
 
-    def all_reduce(self, sends, recvs, count, dtype, op):
-        """Returns (result code, per-rank dicts of phase nanoseconds)."""
+    def _run(self, call):
         t = (C.c_uint64 * (self.n * len(N.TIMER_NAMES)))()
-        rc = lib.fxHostStagedAllReduce(self.h, (C.c_void_p * self.n)(*sends), (C.c_void_p * self.n)(*recvs), count,
-                                       dtype, op, t)
+        rc = call(t)
         k = len(N.TIMER_NAMES)
         return rc, [dict(zip(N.TIMER_NAMES, t[r * k:(r + 1) * k])) for r in range(self.n)]
+
+    def _ptrs(self, v):
+        return (C.c_void_p * self.n)(*v)
+
+    def all_reduce(self, sends, recvs, count, dtype, op):
+        """Returns (result code, per-rank dicts of phase nanoseconds)."""
+        return self._run(lambda t: lib.fxHostStagedAllReduce(self.h, self._ptrs(sends), self._ptrs(recvs), count,
+                                                             dtype, op, t))
+
+    def reduce(self, sends, recvs, count, dtype, op, root):
+        """recvs[r] is used for r == root only."""
+        return self._run(lambda t: lib.fxHostStagedReduce(self.h, self._ptrs(sends), self._ptrs(recvs), count,
+                                                          dtype, op, root, t))
+
+    def reduce_scatter(self, sends, recvs, recvcount, dtype, op):
+        return self._run(lambda t: lib.fxHostStagedReduceScatter(self.h, self._ptrs(sends), self._ptrs(recvs),
+                                                                 recvcount, dtype, op, t))
 
     def destroy(self):
         if self.h:

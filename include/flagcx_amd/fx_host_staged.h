@@ -1,11 +1,14 @@
 /*
- * The reference's host-staged all-reduce as a timed baseline: what
+ * The reference's host-staged reducing collectives as a timed baseline: what
  * FLAGCX_USE_HOST_COMM=1 does for every rank (hostRunnerAllReduce,
- * flagcx/runner/host_runner.cc:236-289) -- staged host buffers, a synchronous
+ * hostRunnerReduce, hostRunnerReduceScatter, flagcx/runner/host_runner.cc:236-289,
+ * 12-67, 291-346) -- staged host buffers, a synchronous
  * device-to-host copy, the bootstrap ring all-reduce on the host
  * (flagcx/service/bootstrap.cc:787-942: ceil(size/n) chunks, n-1 reduce steps
  * res = local (op) received with the loops of
- * flagcx/service/include/utils.h:697-725, then a ring all-gather), a
+ * flagcx/service/include/utils.h:697-725, then a ring all-gather; a reduce
+ * gathers the chunks on the root instead, :944-996; a reduce-scatter's chunk i is
+ * rank i's recvcount elements and stays on rank i, :1039-1066), a
  * host-to-device copy -- with that code's own per-phase timers.  The ranks are
  * simulated ranks of this process, one host thread each; where the reference
  * sends a chunk through a socket, the receiving rank's thread copies it from
@@ -14,7 +17,7 @@
  * It exists to be measured beside the device path and to be compared with it:
  * for the types and ops the reference's host loops carry (int8, uint8, int32,
  * uint32, int64, uint64, fp32, fp64; sum, max, min) the result is bit-identical
- * to flagcxAllReduce with FX_ORDER_HOST.  Other types and ops return
+ * to flagcxAllReduce / flagcxReduce / flagcxReduceScatter with FX_ORDER_HOST.  Other types and ops return
  * flagcxInvalidArgument, as the reference does (utils.h:690-694,
  * bootstrap.cc:872-874).
  */
@@ -63,6 +66,15 @@ int fxHostStagedCreate(fxHostStaged_t *h, int nranks, fxDeviceMemcpyFn memcpyFn)
 int fxHostStagedAllReduce(fxHostStaged_t h, const void *const *sendbuffs,
                           void *const *recvbuffs, size_t count, int dtype,
                           int op, uint64_t *timers);
+/* The same for a reduce (recvbuffs[r] is used for r == root only and may be
+ * NULL elsewhere) and a reduce-scatter (sendbuffs[r] holds nranks * recvcount
+ * elements, recvbuffs[r] receives chunk r). */
+int fxHostStagedReduce(fxHostStaged_t h, const void *const *sendbuffs,
+                       void *const *recvbuffs, size_t count, int dtype, int op,
+                       int root, uint64_t *timers);
+int fxHostStagedReduceScatter(fxHostStaged_t h, const void *const *sendbuffs,
+                              void *const *recvbuffs, size_t recvcount,
+                              int dtype, int op, uint64_t *timers);
 int fxHostStagedDestroy(fxHostStaged_t h);
 
 #ifdef __cplusplus

@@ -657,3 +657,67 @@ def test_host_staged_allreduce_matches_host_order_and_oracle(dev, stream, dname,
         # what the reference's host loops do not carry is refused, as there
         assert hs.all_reduce(ds, dr, count, dtype, N.OP_PROD)[0] == N.INVALID_ARGUMENT
         assert hs.all_reduce(ds, dr, count, N.DT_BF16, N.OP_SUM)[0] == N.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("dname", ["fp32", "int32", "uint8", "fp64"])
+@pytest.mark.parametrize("n,count", [(8, 100003), (3, 10), (4, 2), (5, 77777), (1, 1000)])
+def test_host_staged_reduce_and_reduce_scatter_match_host_order_and_oracle(dev, stream, dname, n, count):
+    """hostRunnerReduce and hostRunnerReduceScatter end to end (host_runner.cc:12-67,
+    291-346 over bootstrap.cc:944-996, 1039-1066): the root's result is the host
+    ring's all-reduce result and no other rank's buffer is written; chunk r of a
+    reduce-scatter ends on rank r.  Bit for bit the oracle's and what the device
+    computes under FX_ORDER_HOST."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    npdt = N.NP_DTYPE[dtype]
+    sends = seeded_inputs(dtype, n, count, seed=7 * n + count)
+    if dname in ("fp32", "fp64"):
+        rng = np.random.default_rng(count + 1)
+        sends = [(a * 10.0 ** rng.integers(-3, 9, count)).astype(npdt) for a in sends]
+        for i in range(min(count, 3 * n)):
+            sends[i % n][i] = (np.nan, 0.0, -0.0)[i % 3]
+    with DevBufs(dev) as b, S.HostStaged(n, dev.t.deviceMemcpy) as hs, S.SimGroup(n, order=S.ORDER_HOST) as g:
+        ds = [b.put(a) for a in sends]
+        dr = [b.alloc(count * es + 16) for _ in range(n)]
+        ddev = b.alloc(count * es)
+        for op, root in ((N.OP_SUM, n - 1), (N.OP_MAX, 0), (N.OP_MIN, n // 2)):
+            want = O.bootstrap_allreduce(sends, dtype, op)[0] if n > 1 else sends[0]
+            for q in dr:
+                dev.memset(q, 0x5A, count * es + 16)
+            rc, _ = hs.reduce(ds, [dr[r] if r == root else None for r in range(n)], count, dtype, op, root)
+            N.check(rc, "fxHostStagedReduce")
+            N.check(g.reduce(ds, [ddev if r == root else None for r in range(n)], count, dtype, op, root, stream))
+            dev.stream_sync(stream)
+            got = dev.to_host(dr[root], count, npdt)
+            assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(want).view(np.uint8)), f"op {op} vs the oracle"
+            assert np.array_equal(got.view(np.uint8), dev.to_host(ddev, count, npdt).view(np.uint8)), f"op {op} vs FX_ORDER_HOST"
+            assert (dev.to_host(dr[root] + count * es, 16, np.uint8) == 0x5A).all()
+            for r in range(n):
+                if r != root:
+                    assert (dev.to_host(dr[r], count * es, np.uint8) == 0x5A).all(), "a non-root buffer was written"
+        assert hs.reduce(ds, dr, count, dtype, N.OP_SUM, n)[0] == N.INVALID_ARGUMENT
+        # reduce-scatter: rank r sends n * rc elements and receives chunk r
+        rc_el = max(count // n, 1)
+        part = [a[:n * rc_el] if a.size >= n * rc_el else np.resize(a, n * rc_el) for a in sends]
+        dp = [b.put(a) for a in part]
+        off = (C.c_size_t * n)(*[r * rc_el * es for r in range(n)])
+        ln = (C.c_size_t * n)(*[rc_el * es] * n)
+        outs = [np.empty(rc_el, npdt) for _ in range(n)]
+        vp = lambda arrs: (C.c_void_p * n)(*[a.ctypes.data for a in arrs])
+        dd = [b.alloc(rc_el * es) for _ in range(n)]
+        for op in (N.OP_SUM, N.OP_MIN):
+            if n > 1:
+                assert O.lib.oracle_bootstrap_reduce_scatter(vp(outs), vp(part), n, off, ln, dtype, op) == 0
+            else:
+                outs = [part[0][:rc_el]]
+            for q in dr:
+                dev.memset(q, 0x5A, count * es + 16)
+            rc, _ = hs.reduce_scatter(dp, dr, rc_el, dtype, op)
+            N.check(rc, "fxHostStagedReduceScatter")
+            N.check(g.reduce_scatter(dp, dd, rc_el, dtype, op, stream))
+            dev.stream_sync(stream)
+            for r in range(n):
+                got = dev.to_host(dr[r], rc_el, npdt)
+                assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(outs[r]).view(np.uint8)), f"rank {r} op {op} vs the oracle"
+                assert np.array_equal(got.view(np.uint8), dev.to_host(dd[r], rc_el, npdt).view(np.uint8)), f"rank {r} vs FX_ORDER_HOST"
+                assert (dev.to_host(dr[r] + rc_el * es, 16, np.uint8) == 0x5A).all(), "wrote past the received chunk"

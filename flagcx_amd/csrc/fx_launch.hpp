@@ -19,11 +19,18 @@ namespace fx {
 //    1 MiB per input takes 4.8 us against 2.9 us, the eight-rank all-reduce
 //    of 64 KiB per rank 6.2 against 4.3 us.  At large sizes 1 is 0.5-4 %
 //    slower than 4, so both exist.
+//  * Three to seven inputs, all aligned like the output, through the direct
+//    kernel: 1 below 64 MiB of output and 2 above (bf16 sum, 4 -> 2 -> 1 vectors
+//    per lane: at 32 MiB per input 6.44 / 6.54 / 6.68 TB/s for 4 inputs, 6.18 /
+//    6.37 / 6.50 for 7; at 512 MiB 6.53 / 6.57 / 6.51 and 6.48 / 6.47 / 6.50).
+//    With an input off the output's alignment 4 stays 2-4 % ahead of both.
 constexpr int unrollFor(int K) { return K <= 2 ? 2 : 4; }
 constexpr int smallUnrollFor(int K) { return K >= 3 ? 1 : unrollFor(K); }
 constexpr int bigUnrollFor(int K) { return K == 8 ? 8 : unrollFor(K); }
+constexpr int alignedUnrollFor(int K) { return (K >= 3 && K <= 7) ? 2 : unrollFor(K); }
 constexpr uint64_t kBigLaunchTiles = 1024;  // use bigUnrollFor only above this many of its tiles (32 MiB per input)
 constexpr uint64_t kSmallLaunchVecs = 256 * 1024;  // fewer 16-byte vectors of output than this: smallUnrollFor
+constexpr uint64_t kMidLaunchVecs = 4096 * 1024;   // aligned, 3-7 inputs: smallUnrollFor below this, alignedUnrollFor above
 
 // The multi-output kernels (one read, up to eight stores per vector) run with one
 // vector per lane at every size: a broadcast to 8 buffers of 256 MiB takes 379 us
@@ -69,12 +76,21 @@ flagcxResult_t launchDirectU(void *out, const void *const *in, int k, uint64_t c
 
 template <class R, int K>
 flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t count, hipStream_t s) {
-  constexpr int US = smallUnrollFor(K), UD = unrollFor(K), UB = bigUnrollFor(K);
+  constexpr int US = smallUnrollFor(K), UD = unrollFor(K), UB = bigUnrollFor(K), UA = alignedUnrollFor(K);
+  const uint64_t vecs = vectorsOf(count, R::ES);
   if constexpr (US != UD)
-    if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
-  if constexpr (UB != UD)
-    if (coAlignedHost(out, in, (K > 0) ? K : k) && tilesFor(out, in, (K > 0) ? K : k, count, R::ES, UB) >= kBigLaunchTiles)
-      return launchDirectU<R, K, UB>(out, in, k, count, s);
+    if (vecs < kSmallLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
+  if constexpr (UA != UD || UB != UD) {
+    if (coAlignedHost(out, in, (K > 0) ? K : k)) {
+      if constexpr (UA != UD) {
+        if (vecs < kMidLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
+        return launchDirectU<R, K, UA>(out, in, k, count, s);
+      }
+      if constexpr (UB != UD)
+        if (tilesFor(out, in, (K > 0) ? K : k, count, R::ES, UB) >= kBigLaunchTiles)
+          return launchDirectU<R, K, UB>(out, in, k, count, s);
+    }
+  }
   return launchDirectU<R, K, UD>(out, in, k, count, s);
 }
 

@@ -13,6 +13,7 @@
 #include <dlfcn.h>
 #include <hip/hip_runtime.h>
 
+#include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/csrc/distributed/c10d/Backend.hpp>
 #include <torch/csrc/distributed/c10d/Store.hpp>
@@ -112,6 +113,9 @@ void checkOne(const Tensors &v, const char *what) {
 
 void checkDense(const at::Tensor &t, const char *what) {
   TORCH_CHECK(t.is_cuda(), what, ": tensor must live on the GPU");
+  // the call goes to the current device's current stream
+  TORCH_CHECK(t.get_device() == c10::hip::current_device(), what, ": tensor is on GPU ", t.get_device(),
+              " but the current device is ", (int)c10::hip::current_device());
   TORCH_CHECK(t.is_contiguous(), what, ": tensor must be contiguous");
   TORCH_CHECK(!t.is_sparse(), what, ": sparse tensors are not supported");
 }

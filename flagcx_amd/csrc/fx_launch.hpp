@@ -8,35 +8,25 @@
 namespace fx {
 
 // Vectors per lane per input, measured on MI355X.
-//  * Large launches: 4, or 2 for one and two inputs (a copy gains 1 %, a
-//    two-input sum 1.5-3.5 % from 64 MiB per input upwards); 8 inputs gain
-//    another 1-2 % with 8 (256 VGPRs) once the launch is large enough not to
-//    miss the extra workgroups and every input is aligned like the output
-//    (unaligned: 4 is 7-10 % faster).
-//  * Launches of less than 4 MiB of output: 1 for three inputs and more.
-//    With 4, such a launch has fewer workgroups than the device has compute
-//    units and each lane waits for 32 loads: an eight-input reduction of
-//    1 MiB per input takes 4.8 us against 2.9 us, the eight-rank all-reduce
-//    of 64 KiB per rank 6.2 against 4.3 us.  At large sizes 1 is 0.5-4 %
-//    slower than 4, so both exist.
-//  * Three to seven inputs, all aligned like the output, through the direct
-//    kernel: 1 below 64 MiB of output and 2 above (bf16 sum, 4 -> 2 -> 1 vectors
-//    per lane: at 32 MiB per input 6.44 / 6.54 / 6.68 TB/s for 4 inputs, 6.18 /
-//    6.37 / 6.50 for 7; at 512 MiB 6.53 / 6.57 / 6.51 and 6.48 / 6.47 / 6.50).
-//    With an input off the output's alignment 4 stays 2-4 % ahead of both.
+//  * Launches that write less than 4 MiB (per output buffer): 1 for three inputs
+//    and more, and for the multi-output kernels.  With 4, such a launch has fewer
+//    workgroups than the device has compute units and each lane waits for 32
+//    loads: an eight-input reduction of 1 MiB per input takes 4.8 us against
+//    2.9 us, the eight-rank all-reduce of 64 KiB per rank 6.2 against 4.3 us.
+//  * Larger launches: 4 (2 for one and two inputs); 8 for 8 inputs once the
+//    launch is large enough not to miss the extra workgroups and every input is
+//    aligned like the output (256 VGPRs; unaligned: 4 is 7-10 % faster).  Between
+//    1, 2 and 4 the difference at these sizes is within 1 % and changes sign with
+//    where the buffers sit: builds that differ only in this number, run
+//    alternately on one box, gave the same figures for two-input sums, copies,
+//    pack / unpack and four-input sums from 8 MiB to 1 GiB, and 0.5-1 % in favour
+//    of 4 over 1 for the eight-rank all-reduce from 64 MiB per rank.
 constexpr int unrollFor(int K) { return K <= 2 ? 2 : 4; }
 constexpr int smallUnrollFor(int K) { return K >= 3 ? 1 : unrollFor(K); }
 constexpr int bigUnrollFor(int K) { return K == 8 ? 8 : unrollFor(K); }
-constexpr int alignedUnrollFor(int K) { return (K >= 3 && K <= 7) ? 2 : unrollFor(K); }
 constexpr uint64_t kBigLaunchTiles = 1024;  // use bigUnrollFor only above this many of its tiles (32 MiB per input)
-constexpr uint64_t kSmallLaunchVecs = 256 * 1024;  // fewer 16-byte vectors of output than this: smallUnrollFor
-constexpr uint64_t kMidLaunchVecs = 4096 * 1024;   // aligned, 3-7 inputs: smallUnrollFor below this, alignedUnrollFor above
-
-// The multi-output kernels (one read, up to eight stores per vector) run with one
-// vector per lane at every size: a broadcast to 8 buffers of 256 MiB takes 379 us
-// against 399 us with four, a two-rank all-reduce 160 against 165 us, the
-// eight-rank one is 1.5-2 % faster up to 64 MiB per rank and 0.5 % slower at 512 MiB.
-constexpr int kBcastUnroll = 1;
+constexpr uint64_t kSmallLaunchVecs = 256 * 1024;  // fewer 16-byte vectors of output than this: one vector per lane
+constexpr int kBcastUnroll = 4, kSmallBcastUnroll = 1;   // the multi-output kernels, any number of inputs
 
 inline uint64_t vectorsOf(uint64_t count, int es) { return (count * (uint64_t)es + 15) / 16; }
 
@@ -76,21 +66,12 @@ flagcxResult_t launchDirectU(void *out, const void *const *in, int k, uint64_t c
 
 template <class R, int K>
 flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t count, hipStream_t s) {
-  constexpr int US = smallUnrollFor(K), UD = unrollFor(K), UB = bigUnrollFor(K), UA = alignedUnrollFor(K);
-  const uint64_t vecs = vectorsOf(count, R::ES);
+  constexpr int US = smallUnrollFor(K), UD = unrollFor(K), UB = bigUnrollFor(K);
   if constexpr (US != UD)
-    if (vecs < kSmallLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
-  if constexpr (UA != UD || UB != UD) {
-    if (coAlignedHost(out, in, (K > 0) ? K : k)) {
-      if constexpr (UA != UD) {
-        if (vecs < kMidLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
-        return launchDirectU<R, K, UA>(out, in, k, count, s);
-      }
-      if constexpr (UB != UD)
-        if (tilesFor(out, in, (K > 0) ? K : k, count, R::ES, UB) >= kBigLaunchTiles)
-          return launchDirectU<R, K, UB>(out, in, k, count, s);
-    }
-  }
+    if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
+  if constexpr (UB != UD)
+    if (coAlignedHost(out, in, (K > 0) ? K : k) && tilesFor(out, in, (K > 0) ? K : k, count, R::ES, UB) >= kBigLaunchTiles)
+      return launchDirectU<R, K, UB>(out, in, k, count, s);
   return launchDirectU<R, K, UD>(out, in, k, count, s);
 }
 
@@ -162,7 +143,10 @@ flagcxResult_t launchBcastOne(const BcastDescDev &d, hipStream_t s) {  // the on
 template <class R, int K>
 flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s) {
   constexpr int U = kBcastUnroll;
-  if (n == 1) return launchBcastOne<R, K, U>(d[0], s);
+  if (n == 1) {
+    if (vectorsOf(d[0].count, R::ES) < kSmallLaunchVecs) return launchBcastOne<R, K, kSmallBcastUnroll>(d[0], s);
+    return launchBcastOne<R, K, U>(d[0], s);
+  }
   InlineBcastTable<kInlineBcast> t;
   t.n = 0;
   t.tileStart[0] = 0;

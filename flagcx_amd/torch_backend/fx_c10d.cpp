@@ -277,7 +277,7 @@ class FxBackend : public c10d::Backend {
     for (int r = 0; r < getSize(); r++) displs[r] = (size_t)r * (size_t)in.numel();
     return run(OpType::ALLGATHER, outs[0], [&](flagcxStream_t s) {
       return flagcxAllGather(in.data_ptr(), flat.data_ptr(), (size_t)in.numel(), dtypeOf(in), comm_, s);
-    }, unpacker(flat, outs[0], displs, counts));
+    }, unpacker(flat, outs[0], displs, counts), {flat});
   }
 
   c10::intrusive_ptr<Work> allgather_into_tensor_coalesced(Tensors &outs, Tensors &ins, const c10d::AllgatherOptions &opts) override {
@@ -307,7 +307,7 @@ class FxBackend : public c10d::Backend {
     return run(OpType::REDUCE_SCATTER, outs, [&](flagcxStream_t s) {
       return flagcxReduceScatter(flat.data_ptr(), outs[0].data_ptr(), (size_t)outs[0].numel(), dtypeOf(flat),
                                  opOf(opts.reduceOp, flat), comm_, s);
-    }, keepAlive(flat));
+    }, nullptr, {flat});
   }
 
   c10::intrusive_ptr<Work> reduce_scatter_tensor_coalesced(Tensors &outs, Tensors &ins, const c10d::ReduceScatterOptions &opts) override {
@@ -373,7 +373,7 @@ class FxBackend : public c10d::Backend {
     checkDense(in, "all_to_all");
     return run(OpType::ALLTOALL, outs, [&](flagcxStream_t s) {
       return flagcxAlltoAllv(in.data_ptr(), sc.data(), sd.data(), out.data_ptr(), rc.data(), rd.data(), dtypeOf(in), comm_, s);
-    }, unpacker(out, outs, rd, rc, in));
+    }, unpacker(out, outs, rd, rc), {in, out});
   }
 
   c10::intrusive_ptr<Work> gather(std::vector<Tensors> &outs, Tensors &ins, const c10d::GatherOptions &opts) override {
@@ -396,7 +396,7 @@ class FxBackend : public c10d::Backend {
     }
     return run(OpType::GATHER, getRank() == root ? outs[0] : Tensors{}, [&](flagcxStream_t s) {
       return flagcxGather(in.data_ptr(), flat.defined() ? flat.data_ptr() : nullptr, (size_t)in.numel(), dtypeOf(in), root, comm_, s);
-    }, std::move(finish));
+    }, std::move(finish), flat.defined() ? Tensors{flat} : Tensors{});
   }
 
   c10::intrusive_ptr<Work> scatter(Tensors &outs, std::vector<Tensors> &ins, const c10d::ScatterOptions &opts) override {
@@ -416,7 +416,7 @@ class FxBackend : public c10d::Backend {
     }
     return run(OpType::SCATTER, outs, [&](flagcxStream_t s) {
       return flagcxScatter(flat.defined() ? flat.data_ptr() : nullptr, out.data_ptr(), (size_t)out.numel(), dtypeOf(out), root, comm_, s);
-    }, keepAlive(flat));
+    }, nullptr, {flat});
   }
 
   c10::intrusive_ptr<Work> send(Tensors &tensors, int dst, int /*tag*/) override {
@@ -442,32 +442,34 @@ class FxBackend : public c10d::Backend {
   }
 
  private:
-  // Staging tensors must outlive the launch, which with simulated ranks may come
-  // from a later rank's call: the Work holds them until its first wait.
-  static std::function<void()> keepAlive(at::Tensor t) {
-    return [t]() {};
-  }
   // Copy pieces of a staging tensor into a list of output tensors, on the
   // collective's stream, after the launch.
-  static std::function<void()> unpacker(at::Tensor flat, Tensors outs, std::vector<size_t> displs, std::vector<size_t> counts,
-                                        at::Tensor alsoKeep = at::Tensor()) {
-    return [flat, outs, displs, counts, alsoKeep]() mutable {
+  static std::function<void()> unpacker(at::Tensor flat, Tensors outs, std::vector<size_t> displs, std::vector<size_t> counts) {
+    return [flat, outs, displs, counts]() mutable {
       for (size_t r = 0; r < outs.size(); r++)
         if (counts[r]) outs[r].copy_(flat.narrow(0, (int64_t)displs[r], (int64_t)counts[r]).view_as(outs[r]), true);
     };
   }
 
+  // `staging`: tensors of this call that the kernels read or write and the
+  // caller never sees.  With simulated ranks the launch may come from a later
+  // rank's call, so they are held here, not by the Work the caller may drop,
+  // until this rank's next collective has been accepted -- which the rank layer
+  // only does once the previous one has been launched.
   template <class F>
-  c10::intrusive_ptr<Work> run(OpType op, Tensors outputs, F call, std::function<void()> finish = nullptr) {
+  c10::intrusive_ptr<Work> run(OpType op, Tensors outputs, F call, std::function<void()> finish = nullptr,
+                               Tensors staging = {}) {
     const hipStream_t raw = c10::hip::getCurrentHIPStream().stream();
     BorrowedStream s(raw);
     ok(call(s.get()), c10d::opTypeToString(op).c_str());
+    held_ = std::move(staging);
     auto work = c10::make_intrusive<FxWork>(getRank(), op, raw, std::move(outputs), std::move(finish));
     if (getSize() == 1) (void)work->wait();   // one rank: the launch has happened, finish now
     return work;
   }
 
   flagcxComm_t comm_ = nullptr;
+  Tensors held_;
 };
 
 c10::intrusive_ptr<c10d::Backend> createBackend(const c10::intrusive_ptr<c10d::Store> &store, int rank, int size) {

@@ -407,8 +407,14 @@ struct CopyRed {
 // fetched); grouped columns and temporal loads 6.3-6.4 (1.11 x).  Aligned
 // streams keep column i and nontemporal loads (grouped columns cost 1-2 % for
 // 8 inputs of 512 MiB, temporal loads 4 % for large aligned streams).
-constexpr uint32_t kPieceVecs = 32;                           // 512 bytes
-constexpr uint32_t kStripeTiles = 64;                         // tiles per region
+#ifndef FX_PIECE_VECS
+#define FX_PIECE_VECS 32      // 512 bytes; other values are for experiments (a divisor of the workgroup size)
+#endif
+#ifndef FX_STRIPE_TILES
+#define FX_STRIPE_TILES 64    // tiles per region; other values are for experiments (a multiple of 8)
+#endif
+constexpr uint32_t kPieceVecs = FX_PIECE_VECS;
+constexpr uint32_t kStripeTiles = FX_STRIPE_TILES;
 constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;      // 32 KiB
 #ifndef FX_STRIPE_MIN_BYTES
 #define FX_STRIPE_MIN_BYTES (4ull << 20)

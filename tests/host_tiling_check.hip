@@ -52,7 +52,7 @@ static long checkOne(uint64_t outAddr, uint64_t count, int es, int U, HandOut ho
   for (uint64_t tile = 0; tile < tp.zoneTiles; tile++) {
     const uint64_t col = ((laneOfTile(tp, (uint32_t)tile, 0, U, shift).j - tp.zs) % kRowVecs) / kPieceVecs;
     const uint64_t t = tile % kStripeTiles;
-    if (tp.grouped ? (col / 8 != (t + shift) % 8) : (col != t)) return 10;
+    if (tp.grouped ? (col / (kStripeTiles / 8) != (t + shift) % 8) : (col != t)) return 10;
   }
   return 0;
 }

@@ -140,13 +140,8 @@ flagcxResult_t launchBcastOne(const BcastDescDev &d, hipStream_t s) {  // the on
   return launchKernel(reduceBcastInline<R, K, U, 1>, (uint32_t)tiles, s, t);
 }
 
-template <class R, int K>
-flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s) {
-  constexpr int U = kBcastUnroll;
-  if (n == 1) {
-    if (vectorsOf(d[0].count, R::ES) < kSmallLaunchVecs) return launchBcastOne<R, K, kSmallBcastUnroll>(d[0], s);
-    return launchBcastOne<R, K, U>(d[0], s);
-  }
+template <class R, int K, int U>
+flagcxResult_t launchBcastMany(const BcastDescDev *d, size_t n, hipStream_t s) {  // the sixteen-slot table
   InlineBcastTable<kInlineBcast> t;
   t.n = 0;
   t.tileStart[0] = 0;
@@ -168,6 +163,15 @@ flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s)
     t.n++;
   }
   return flagcxSuccess;
+}
+
+template <class R, int K>
+flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s) {
+  uint64_t vecs = 0;   // per output buffer, all descriptors together
+  for (size_t i = 0; i < n; i++) vecs += vectorsOf(d[i].count, R::ES);
+  const bool small = vecs < kSmallLaunchVecs;
+  if (n == 1) return small ? launchBcastOne<R, K, kSmallBcastUnroll>(d[0], s) : launchBcastOne<R, K, kBcastUnroll>(d[0], s);
+  return small ? launchBcastMany<R, K, kSmallBcastUnroll>(d, n, s) : launchBcastMany<R, K, kBcastUnroll>(d, n, s);
 }
 
 template <class R, int K, bool BCAST = true>

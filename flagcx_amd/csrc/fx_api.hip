@@ -418,6 +418,54 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
   });
 }
 
+int fx_reduce_bcast(void *const *outs, int nout, const void *const *ins, int k, size_t count, int dtype, int op,
+                    int first, void *stream) {
+  const bool copy = (op == -1);
+  if (copy) {
+    if (k != 1) return flagcxInvalidArgument;
+  } else {
+    flagcxResult_t rc = screen(dtype, op);
+    if (rc != flagcxSuccess) return rc;
+  }
+  if (!outs || !ins || k < 1 || k > FX_MAX_INPUTS || nout < 1 || nout > FX_MAX_INPUTS || first < 0 || first >= k)
+    return flagcxInvalidArgument;
+  if (count == 0) return flagcxSuccess;
+  return guarded([&]() -> int {
+    hipStream_t s = (hipStream_t)stream;
+    uintptr_t bits = copy ? (uintptr_t)count : 0;
+    const void *rot[FX_MAX_INPUTS];
+    for (int j = 0; j < k; j++) {
+      rot[j] = ins[(first + j) % k];
+      if (!rot[j]) return flagcxInvalidArgument;
+      bits |= (uintptr_t)rot[j];
+    }
+    bool alike = true;
+    for (int o = 0; o < nout; o++) {
+      if (!outs[o]) return flagcxInvalidArgument;
+      bits |= (uintptr_t)outs[o];
+      alike = alike && (((uintptr_t)outs[o] & 15u) == ((uintptr_t)outs[0] & 15u));
+    }
+    const int es = copy ? ((bits & 1) ? 1 : ((bits & 2) ? 2 : 4)) : (int)dtypeSize(dtype);
+    if (!copy && (bits & (uintptr_t)(es - 1))) return flagcxInvalidArgument;
+    const KernelSet *ks = copy ? copySetFor(es) : setFor(dtype, op);
+    const uint64_t n = copy ? (uint64_t)count / (uint64_t)es : (uint64_t)count;
+    if (alike) return ks->bcastRuntime(outs, nout, rot, k, n, s);
+    // outputs at different offsets within 16 bytes: one reduce, then copies of its result
+    flagcxResult_t rc = ks->direct[k <= kMaxFixedK ? k : 0](outs[0], rot, k, n, s);
+    if (rc != flagcxSuccess) return rc;
+    SliceList copies;
+    for (int o = 1; o < nout; o++) {
+      fxSliceDesc c;
+      memset(&c, 0, sizeof(c));
+      c.in[0] = outs[0];
+      c.out = outs[o];
+      c.count = n * (uint64_t)es;
+      copies.push_back(c);
+    }
+    return copies.empty() ? flagcxSuccess : fx_copy_slices(copies.data(), copies.size(), stream);
+  });
+}
+
 int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, int dtype, int op) {
   if (!plan) return flagcxInvalidArgument;
   *plan = nullptr;

@@ -40,6 +40,9 @@ struct KernelSet {
                                                 uint32_t grid, hipStream_t s);
   // n validated, non-empty multi-output slices
   flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const BcastDescDev *d, size_t n, hipStream_t s);
+  // one segment, up to kMaxK inputs and kMaxK outputs (outputs aligned alike within 16 bytes)
+  flagcxResult_t (*bcastRuntime)(void *const *out, int nout, const void *const *in, int k, uint64_t count,
+                                 hipStream_t s);
   int elemSize;
 };
 
@@ -174,6 +177,22 @@ flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s)
   return small ? launchBcastMany<R, K, kSmallBcastUnroll>(d, n, s) : launchBcastMany<R, K, kBcastUnroll>(d, n, s);
 }
 
+template <class R>
+flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const *in, int k, uint64_t count,
+                                  hipStream_t s) {
+  constexpr int U = unrollFor(0);
+  ManyArgs a = {};
+  for (int p = 0; p < k; p++) a.in[p] = in[p];
+  for (int o = 0; o < nout; o++) a.out[o] = out[o];
+  a.count = count;
+  a.k = k;
+  a.nout = nout;
+  const uint64_t ntiles = tilesFor(out[0], in, k, count, R::ES, U, out + 1, nout - 1);
+  if (ntiles == 0) return flagcxSuccess;
+  if (ntiles > 0x7ffffff0ull) return flagcxInvalidArgument;
+  return launchKernel(reduceBcastRuntime<R, U>, (uint32_t)ntiles, s, a);
+}
+
 template <class R, int K, bool BCAST = true>
 void fillSet(KernelSet &ks) {
   ks.direct[K] = &launchDirect<R, K>;
@@ -201,6 +220,7 @@ KernelSet makeSet() {
   fillSet<R, 6>(ks);
   fillSet<R, 7>(ks);
   fillSet<R, 8>(ks);
+  ks.bcastRuntime = &launchBcastRuntime<R>;
   ks.elemSize = R::ES;
   return ks;
 }
@@ -210,6 +230,7 @@ template <int ES>
 KernelSet makeCopySet() {
   KernelSet ks = {};
   fillSet<CopyRed<ES>, 1, true>(ks);
+  ks.bcastRuntime = &launchBcastRuntime<CopyRed<ES>>;
   ks.elemSize = ES;
   return ks;
 }

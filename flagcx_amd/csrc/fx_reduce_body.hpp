@@ -628,6 +628,24 @@ __device__ __forceinline__ void storeElems(const SegB<K> &sg, uint64_t e0, int l
     if (o < sg.nmore) scatterElems<ES>(sg.more[o], e0, lo, hi, v);
 }
 
+// Runtime number of inputs AND of outputs (more ranks than a descriptor has
+// slots): both pointer tables stay in the kernel argument block and are read
+// through scalar loads.  All outputs share out's misalignment within 16 bytes.
+struct SegMany : Seg<0> {
+  void *const *rawOut;   // the outputs after the first
+  int nmore;
+  __device__ __forceinline__ char *outp(int o) const { return asGlobal(rawOut[o]) - mis; }
+};
+__device__ __forceinline__ void storeVector(const SegMany &sg, uint64_t byteOff, u32x4 v) {
+  stg_stream(sg.out + byteOff, v);
+  for (int o = 0; o < sg.nmore; o++) stg_stream(sg.outp(o) + byteOff, v);
+}
+template <int ES>
+__device__ __forceinline__ void storeElems(const SegMany &sg, uint64_t e0, int lo, int hi, u32x4 v) {
+  scatterElems<ES>(sg.out, e0, lo, hi, v);
+  for (int o = 0; o < sg.nmore; o++) scatterElems<ES>(sg.outp(o), e0, lo, hi, v);
+}
+
 // Reduce vector j of the segment with full bounds / alignment handling.
 template <class R, int K, class SG>
 __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
@@ -813,6 +831,33 @@ struct DirectArgs {
   uint64_t count;
   int k;
 };
+
+struct ManyArgs {
+  const void *in[kMaxK];
+  void *out[kMaxK];
+  uint64_t count;
+  int k, nout;
+};
+
+// k inputs (rotated by the host) folded once and stored to nout buffers.
+template <class R, int U>
+__global__ void __launch_bounds__(kBlock) reduceBcastRuntime(ManyArgs a) {
+  SegMany sg;
+  const uint64_t mis = (uint64_t)(uintptr_t)a.out[0] & 15u;
+  sg.raw = a.in;
+  sg.mis = mis;
+  sg.out = asGlobal(a.out[0]) - mis;
+  sg.lead = mis / R::ES;
+  sg.end = sg.lead + a.count;
+  sg.k = a.k;
+  sg.rawOut = a.out + 1;
+  sg.nmore = a.nout - 1;
+  bool co = true;
+  for (int p = 0; p < a.k; p++) co = co && sameLinePhase((uint64_t)(uintptr_t)a.in[p], (uint64_t)(uintptr_t)a.out[0]);
+  for (int o = 1; o < a.nout; o++) co = co && sameLinePhase((uint64_t)(uintptr_t)a.out[o], (uint64_t)(uintptr_t)a.out[0]);
+  const TilePlan tp = planTiles((uint64_t)(uintptr_t)a.out[0], a.count, R::ES, U, handOutFor(co, a.k));
+  reduceTile<R, 0, U>(sg, tp, blockIdx.x, 0u);
+}
 
 template <class R, int K, int U>
 __global__ void __launch_bounds__(kBlock) reduceCopyDirect(DirectArgs<K> a) {

@@ -154,9 +154,30 @@ struct Ctx {
   void *recv(int r) const { return g->posts[r].recv; }
 };
 
+// More inputs than a slice descriptor carries: such pieces go through the
+// runtime-k kernel, one launch each, so pieces that continue each other in the
+// send buffers and in the output are gathered into one run first (the
+// red-slice split alone cuts a 64 MiB all-reduce over 16 ranks into 512 pieces
+// of 128 KiB).
+struct KwayRun {
+  size_t sendOff = 0, cnt = 0;
+  void *out = nullptr;
+  int first = 0;
+};
+
+flagcxResult_t launchRun(const Ctx &c, KwayRun &run) {
+  if (run.cnt == 0) return flagcxSuccess;
+  PtrList in;
+  in.resize((size_t)c.n);
+  for (int j = 0; j < c.n; j++) in[j] = cadd(c.send(j), run.sendOff * c.ts);
+  const flagcxResult_t rc = R(fx_reduce_copy(run.out, in.data(), c.n, run.cnt, c.g->dtype, c.g->op, run.first, c.s));
+  run = KwayRun();
+  return rc;
+}
+
 // k-way reduce of element range [off, off+cnt) of every rank's sendbuff (+sendBase
 // elements) into out, in order first, first+1, ...
-flagcxResult_t kway(const Ctx &c, SliceList &descs, size_t sendOff, size_t cnt, void *out, int first) {
+flagcxResult_t kway(const Ctx &c, SliceList &descs, KwayRun &run, size_t sendOff, size_t cnt, void *out, int first) {
   if (cnt == 0) return flagcxSuccess;
   if (c.n <= FX_MAX_SLICE_INPUTS) {
     fxSliceDesc d;
@@ -167,15 +188,22 @@ flagcxResult_t kway(const Ctx &c, SliceList &descs, size_t sendOff, size_t cnt, 
     descs.push_back(d);
     return flagcxSuccess;
   }
-  PtrList in;
-  in.resize((size_t)c.n);
-  for (int j = 0; j < c.n; j++) in[j] = cadd(c.send(j), sendOff * c.ts);
-  return R(fx_reduce_copy(out, in.data(), c.n, cnt, c.g->dtype, c.g->op, first, c.s));
+  if (run.cnt && first == run.first && sendOff == run.sendOff + run.cnt && out == madd(run.out, run.cnt * c.ts)) {
+    run.cnt += cnt;
+    return flagcxSuccess;
+  }
+  const flagcxResult_t rc = launchRun(c, run);
+  run.sendOff = sendOff;
+  run.cnt = cnt;
+  run.out = out;
+  run.first = first;
+  return rc;
 }
 
-flagcxResult_t flushKway(const Ctx &c, SliceList &descs) {
-  if (descs.empty()) return flagcxSuccess;
-  flagcxResult_t rc = R(fx_reduce_slices(descs.data(), descs.size(), c.n, c.g->dtype, c.g->op, c.s));
+flagcxResult_t flushKway(const Ctx &c, SliceList &descs, KwayRun &run) {
+  flagcxResult_t rc = launchRun(c, run);
+  if (rc != flagcxSuccess || descs.empty()) return rc;
+  rc = R(fx_reduce_slices(descs.data(), descs.size(), c.n, c.g->dtype, c.g->op, c.s));
   descs.clear();
   return rc;
 }
@@ -435,29 +463,27 @@ flagcxResult_t runAllReduce(const Ctx &c) {
     }
     return R(fx_reduce_bcast_slices(bd.data(), bd.size(), n, n, g->dtype, g->op, c.s));
   }
-  // more ranks: chunk ch is reduced k-way into the rank the ring would leave it
-  // on, (ch-1)%n, then copied to everyone else.
+  // more ranks than a descriptor has slots: the runtime-k, runtime-n form of the
+  // same one-read-n-stores launch.  Rank order is one launch over the whole
+  // buffer; ring order starts chunk ch's fold at rank ch, one launch per chunk.
+  PtrList ins;
+  fx::SmallVec<void *, 16> outs;
+  ins.resize((size_t)n);
+  outs.resize((size_t)n);
+  auto bcast = [&](size_t off, size_t cnt, int first) {
+    for (int j = 0; j < n; j++) ins[j] = cadd(c.send(j), off * ts);
+    for (int r = 0; r < n; r++) outs[r] = madd(c.recv(r), off * ts);
+    return R(fx_reduce_bcast(outs.data(), n, ins.data(), n, cnt, g->dtype, g->op, first, c.s));
+  };
+  if (g->order != FX_ORDER_RING) return bcast(0, count, 0);
   for (int ch = 0; ch < n; ch++) {
     size_t ccnt, coff;
     fx_split(count, n, ch, &ccnt, &coff);
-    const int owner = mod(ch - 1, n);
-    const int first = (g->order == FX_ORDER_RING) ? ch : 0;
-    flagcxResult_t rc = forPieces(g, ccnt, coff, nred, [&](size_t off, size_t, size_t cnt) {
-      return kway(c, descs, off, cnt, madd(c.recv(owner), off * ts), first);
-    });
+    if (ccnt == 0) continue;
+    const flagcxResult_t rc = bcast(coff, ccnt, ch);
     if (rc != flagcxSuccess) return rc;
   }
-  flagcxResult_t rc = flushKway(c, descs);
-  if (rc != flagcxSuccess) return rc;
-  for (int ch = 0; ch < n; ch++) {
-    size_t ccnt, coff;
-    fx_split(count, n, ch, &ccnt, &coff);
-    const int owner = mod(ch - 1, n);
-    for (int r = 0; r < n; r++)
-      if (r != owner && ccnt)
-        descs.push_back(copyDesc(cadd(c.recv(owner), coff * ts), madd(c.recv(r), coff * ts), ccnt * ts));
-  }
-  return R(fx_copy_slices(descs.data(), descs.size(), c.s));
+  return flagcxSuccess;
 }
 
 // Receive steps of tree rank a (uni_runner_impl.cc:1314-1326): the root takes
@@ -546,6 +572,7 @@ flagcxResult_t runReduceScatter(const Ctx &c) {
   }
   const size_t nred = fx_nredslices(rcount, n, (size_t)g->nslices, (size_t)g->nredslices, (size_t)g->redslicesize);
   SliceList descs;
+  KwayRun run;
   if (g->algo == FX_ALGO_RING && g->op != flagcxAvg) {  // a mean is not a chain of two-input means
     // Per-rank scratch of n*recvcount elements holds the travelling partials.
     flagcxResult_t rc = ensureScratch(g, (size_t)n * n * rcount * ts, c.s);
@@ -577,11 +604,11 @@ flagcxResult_t runReduceScatter(const Ctx &c) {
   for (int r = 0; r < n; r++) {
     const int first = (g->order == FX_ORDER_RING) ? mod(r + 1, n) : 0;
     flagcxResult_t rc = forPieces(g, rcount, (size_t)r * rcount, nred, [&](size_t off, size_t inSlice, size_t cnt) {
-      return kway(c, descs, off, cnt, madd(c.recv(r), inSlice * ts), first);
+      return kway(c, descs, run, off, cnt, madd(c.recv(r), inSlice * ts), first);
     });
     if (rc != flagcxSuccess) return rc;
   }
-  return flushKway(c, descs);
+  return flushKway(c, descs, run);
 }
 
 flagcxResult_t runAllGather(const Ctx &c) {
@@ -746,22 +773,11 @@ flagcxResult_t runCustomAllReduce(const Ctx &c) {
     b.count = g->count;
     return R(fx_reduce_bcast_slices(&b, 1, c.n, c.n, g->dtype, g->op, c.s));
   }
-  SliceList descs;
-  for (int r = 0; r < c.n; r++) {
-    if (c.n <= FX_MAX_SLICE_INPUTS) {
-      fxSliceDesc d;
-      memset(&d, 0, sizeof(d));
-      for (int j = 0; j < c.n; j++) d.in[j] = g->windows[j];
-      d.out = c.recv(r);
-      d.count = g->count;
-      descs.push_back(d);
-    } else {
-      flagcxResult_t rc = R(fx_reduce_copy(c.recv(r), (const void *const *)g->windows.data(), c.n, g->count,
-                                           g->dtype, g->op, 0, c.s));
-      if (rc != flagcxSuccess) return rc;
-    }
-  }
-  return flushKway(c, descs);
+  fx::SmallVec<void *, 16> outs;
+  outs.resize((size_t)c.n);
+  for (int r = 0; r < c.n; r++) outs[r] = c.recv(r);
+  return R(fx_reduce_bcast(outs.data(), c.n, (const void *const *)g->windows.data(), c.n, g->count, g->dtype, g->op, 0,
+                           c.s));
 }
 
 void resetPending(Group *g) {

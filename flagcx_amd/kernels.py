@@ -50,6 +50,11 @@ def reduce_bcast_slices(descs, k, nout, dtype, op, stream=None):
     return lib.fx_reduce_bcast_slices(arr, len(descs), k, nout, dtype, op, stream)
 
 
+def reduce_bcast(outs, ins, count, dtype, op, first=0, stream=None):
+    """One segment, up to 64 inputs folded once into up to 64 outputs; op = -1 copies ins[0] (count in bytes)."""
+    return lib.fx_reduce_bcast(_ptr_array(outs), len(outs), _ptr_array(ins), len(ins), count, dtype, op, first, stream)
+
+
 def copy_slices(descs, stream=None):
     """descs: iterable of (src, dst, nbytes)."""
     arr, n = make_slices(([s], d, b) for s, d, b in descs)

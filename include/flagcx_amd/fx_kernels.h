@@ -189,6 +189,19 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
                            int dtype, int op, void *stream);
 
 /*
+ * The same for ONE segment with up to FX_MAX_INPUTS inputs and FX_MAX_INPUTS
+ * outputs: outs[0..nout) all receive the fold of ins[first], ins[first+1], ...
+ * (wrapping), in one launch and with (k + nout) * size bytes of traffic.  This
+ * is the all-reduce of more simulated ranks than a descriptor has slots
+ * (the reference's LSA kernel reads every peer and stores the result once per
+ * rank, custom_allreduce.cu:370-394, for any nRanks).  op = -1 copies ins[0]
+ * (k = 1, count in bytes).  Outputs that do not share outs[0]'s alignment
+ * within 16 bytes are served by a reduce into outs[0] plus copies.
+ */
+int fx_reduce_bcast(void *const *outs, int nout, const void *const *ins, int k,
+                    size_t count, int dtype, int op, int first, void *stream);
+
+/*
  * Copy n independent byte ranges (in[0] -> out, `count` = BYTES): the Cpy node
  * and the all-gather landing copies (uni_runner_impl.cc:322-344,1649-1662;
  * flagcx/core/p2p.cc:257-283) as one launch.

@@ -186,6 +186,63 @@ def test_long_copies_at_every_kind_of_line_phase(dev):
     assert np.array_equal(back, want)
 
 
+@pytest.mark.parametrize("dname", ["bf16", "fp32", "int32", "uint8", "fp64"])
+def test_reduce_bcast_many_inputs_many_outputs(dev, dname):
+    """fx_reduce_bcast: one segment, up to 64 inputs folded once (starting at
+    `first`) and stored to up to 64 outputs -- more ranks than a slice descriptor
+    has slots.  Odd lengths, buffers off 16-byte alignment (alike, and one output
+    at its own offset: the reduce-plus-copies route), a segment long enough for the
+    striped hand-out, in place; nothing written outside any output."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    npdt = N.NP_DTYPE[dtype]
+    rng = np.random.default_rng(es)
+    ve = 16 // es
+    cases = [(9, 9, 40001, 0, 0), (17, 3, 1, 2, 0), (12, 16, 65536 + 5, 5, 3), (1, 12, 300007, 0, 1), (33, 33, 2048, 7, 0),
+             (64, 64, 1500, 63, 2), (10, 2, (5 << 20) // es + 3, 4, 0)]
+    for k, nout, n, first, mis in cases:
+        for op in (N.OP_SUM, N.OP_MAX) if k < 30 else (N.OP_SUM,):
+            ins = seeded_inputs(dtype, k, n, seed=k * 100 + nout)
+            want = O.reduce_copy(ins, dtype, op, first=first)
+            for odd_one in (False, True):
+                with DevBufs(dev) as b:
+                    dins = [b.put(a, pad_before=mis * es) for a in ins]
+                    outs = []
+                    for o in range(nout):
+                        lead = (mis + (1 if odd_one and o == nout - 1 and ve > 1 else 0)) * es
+                        base = b.alloc(lead + n * es + 64)
+                        dev.memset(base, 0xA5, lead + n * es + 64)
+                        outs.append(base + lead)
+                    N.check(K.reduce_bcast(outs, dins, n, dtype, op, first), f"fx_reduce_bcast k={k} nout={nout}")
+                    dev.sync()
+                    for o, d in enumerate(outs):
+                        assert_parity(dev.to_host(d, n, npdt), want, dtype, op, f"{dname} k={k} nout={nout} n={n} out {o}")
+                        assert (dev.to_host(d + n * es, 32, np.uint8) == 0xA5).all(), "wrote past an output"
+                        lead = d % 16
+                        if lead:
+                            assert (dev.to_host(d - lead, lead, np.uint8) == 0xA5).all(), "wrote before an output"
+    # in place on every rank's buffer (the all-reduce shape), and a broadcast copy
+    k = 11
+    ins = seeded_inputs(dtype, k, 77777, seed=3)
+    want = O.reduce_copy(ins, dtype, N.OP_SUM)
+    with DevBufs(dev) as b:
+        dins = [b.put(a) for a in ins]
+        N.check(K.reduce_bcast(dins, dins, 77777, dtype, N.OP_SUM), "in place")
+        dev.sync()
+        for d in dins:
+            assert_parity(dev.to_host(d, 77777, npdt), want, dtype, N.OP_SUM, f"{dname} in place")
+        outs = [b.alloc(77777 * es + 8) + (o % 2) for o in range(13)]          # odd byte offsets: the copy granularity adapts
+        N.check(K.reduce_bcast(outs, [dins[0] + es], (77777 - 1) * es, dtype, -1), "broadcast copy")
+        dev.sync()
+        src = dev.to_host(dins[0] + es, (77777 - 1) * es, np.uint8)
+        for d in outs:
+            assert np.array_equal(dev.to_host(d, (77777 - 1) * es, np.uint8), src)
+    assert K.reduce_bcast([1], [], 4, dtype, N.OP_SUM) == N.INVALID_ARGUMENT
+    assert K.reduce_bcast([16] * 65, [16], 4, dtype, N.OP_SUM) == N.INVALID_ARGUMENT
+    assert K.reduce_bcast([16], [16, 16], 4, dtype, N.OP_SUM, first=2) == N.INVALID_ARGUMENT
+    assert K.reduce_bcast([16], [16, 16], 4, dtype, -1) == N.INVALID_ARGUMENT
+
+
 def _random_layout(rng, counts, slack):
     """Random non-overlapping displacements for the given segment counts."""
     order = rng.permutation(len(counts))

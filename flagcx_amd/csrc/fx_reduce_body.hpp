@@ -700,7 +700,24 @@ __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, ui
     typename R::Acc acc[U];
 #pragma unroll
     for (int u = 0; u < U; u++) R::init(acc[u], ldg_as<TEMPORAL>(sg.inp(0) + off + u * ustride));
-    for (int p = 1; p < sg.inputs(); p++) {
+    // four inputs in flight at a time (folded in their order): a lane that waits for
+    // every input in turn is what a small launch of many inputs spends its time on
+    const int k = sg.inputs();
+    int p = 1;
+    for (; p + 4 <= k; p += 4) {
+      u32x4 v[4][U];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const char *ip = sg.inp(p + q);
+#pragma unroll
+        for (int u = 0; u < U; u++) v[q][u] = ldg_as<TEMPORAL>(ip + off + u * ustride);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int u = 0; u < U; u++) R::fold(acc[u], v[q][u]);
+    }
+    for (; p < k; p++) {
       const char *ip = sg.inp(p);
       u32x4 v[U];
 #pragma unroll

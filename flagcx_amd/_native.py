@@ -49,6 +49,11 @@ class BcastDesc(C.Structure):
     _fields_ = [("inp", C.c_void_p * 8), ("out", C.c_void_p * 8), ("count", C.c_uint64)]
 
 
+class Chunk(C.Structure):
+    _fields_ = [("in_off", C.c_uint64), ("out_off", C.c_uint64), ("count", C.c_uint64),
+                ("first", C.c_int), ("in_sel", C.c_int), ("out_sel", C.c_int)]
+
+
 class SliceDesc(C.Structure):
     _fields_ = [("in_", C.c_void_p * 8), ("out", C.c_void_p), ("count", C.c_uint64)]
 
@@ -74,6 +79,7 @@ _SIGS = {
     "fx_reduce_bcast_slices": (_i, [C.POINTER(BcastDesc), _sz, _i, _i, _i, _i, _vp]),
     "fx_copy_slices": (_i, [C.POINTER(SliceDesc), _sz, _vp]),
     "fx_reduce_bcast": (_i, [C.POINTER(_vp), _i, C.POINTER(_vp), _i, _sz, _i, _i, _i, _vp]),
+    "fx_reduce_chunks": (_i, [C.POINTER(_vp), _i, C.POINTER(_vp), _i, C.POINTER(Chunk), _i, _i, _i, _vp]),
     "fx_plan_create": (_i, [C.POINTER(_vp), C.POINTER(SliceDesc), _sz, _i, _i, _i]),
     "fx_plan_launch": (_i, [_vp, _vp]),
     "fx_plan_destroy": (_i, [_vp]),

@@ -466,6 +466,64 @@ int fx_reduce_bcast(void *const *outs, int nout, const void *const *ins, int k, 
   });
 }
 
+int fx_reduce_chunks(void *const *outs, int nout, const void *const *ins, int k, const fxChunk *chunks, int nchunks,
+                     int dtype, int op, void *stream) {
+  const bool copy = (op == -1);
+  if (!copy) {
+    flagcxResult_t rc = screen(dtype, op);
+    if (rc != flagcxSuccess) return rc;
+  }
+  if (!outs || !ins || k < 1 || k > FX_MAX_INPUTS || nout < 1 || nout > FX_MAX_INPUTS || nchunks < 0) return flagcxInvalidArgument;
+  if (nchunks == 0) return flagcxSuccess;
+  if (!chunks) return flagcxInvalidArgument;
+  return guarded([&]() -> int {
+    uintptr_t bits = 0;
+    for (int j = 0; j < k; j++) {
+      if (!ins[j]) return flagcxInvalidArgument;
+      bits |= (uintptr_t)ins[j];
+    }
+    for (int o = 0; o < nout; o++) {
+      if (!outs[o]) return flagcxInvalidArgument;
+      bits |= (uintptr_t)outs[o];
+    }
+    for (int c = 0; c < nchunks; c++) {
+      const fxChunk &ch = chunks[c];
+      if (ch.in_sel >= k || ch.out_sel >= nout || (ch.in_sel < 0 && (ch.first < 0 || ch.first >= k))) return flagcxInvalidArgument;
+      if (copy && ch.in_sel < 0) return flagcxInvalidArgument;
+      if (copy) bits |= (uintptr_t)ch.in_off | (uintptr_t)ch.out_off | (uintptr_t)ch.count;
+      if (ch.out_sel < 0 && ch.count)   // the outputs of one chunk share their byte offset, so their bases must agree within 16
+        for (int o = 1; o < nout; o++)
+          if ((((uintptr_t)outs[o] ^ (uintptr_t)outs[0]) & 15u) != 0) return flagcxInvalidArgument;
+    }
+    const int es = copy ? ((bits & 1) ? 1 : ((bits & 2) ? 2 : 4)) : (int)dtypeSize(dtype);
+    if (!copy && (bits & (uintptr_t)(es - 1))) return flagcxInvalidArgument;
+    const KernelSet *ks = copy ? copySetFor(es) : setFor(dtype, op);
+    const uint64_t scale = copy ? 1 : (uint64_t)es;        // offsets to bytes
+    const uint64_t unit = copy ? (uint64_t)es : 1;         // counts to elements of the kernel's type
+    for (int base = 0; base < nchunks; base += kMaxK) {
+      ChunkedArgs a;
+      memset(&a, 0, sizeof(a));
+      for (int j = 0; j < k; j++) a.in[j] = ins[j];
+      for (int o = 0; o < nout; o++) a.out[o] = outs[o];
+      a.k = k;
+      a.nout = nout;
+      a.nchunks = (nchunks - base < kMaxK) ? nchunks - base : kMaxK;
+      for (int c = 0; c < a.nchunks; c++) {
+        const fxChunk &ch = chunks[base + c];
+        a.inOff[c] = ch.in_off * scale;
+        a.outOff[c] = ch.out_off * scale;
+        a.cnt[c] = ch.count / unit;
+        a.first[c] = (int8_t)(ch.in_sel < 0 ? ch.first : 0);
+        a.only[c] = (int8_t)(ch.in_sel < 0 ? -1 : ch.in_sel);
+        a.outSel[c] = (int8_t)(ch.out_sel < 0 ? -1 : ch.out_sel);
+      }
+      const flagcxResult_t rc = ks->chunksRuntime(&a, (hipStream_t)stream);
+      if (rc != flagcxSuccess) return rc;
+    }
+    return flagcxSuccess;
+  });
+}
+
 int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, int dtype, int op) {
   if (!plan) return flagcxInvalidArgument;
   *plan = nullptr;

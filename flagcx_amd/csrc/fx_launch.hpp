@@ -43,6 +43,8 @@ struct KernelSet {
   // one segment, up to kMaxK inputs and kMaxK outputs (outputs aligned alike within 16 bytes)
   flagcxResult_t (*bcastRuntime)(void *const *out, int nout, const void *const *in, int k, uint64_t count,
                                  hipStream_t s);
+  // chunks of a collective over up to kMaxK ranks; tileStart is filled here
+  flagcxResult_t (*chunksRuntime)(ChunkedArgs *a, hipStream_t s);
   int elemSize;
 };
 
@@ -193,6 +195,20 @@ flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const 
   return launchKernel(reduceBcastRuntime<R, U>, (uint32_t)ntiles, s, a);
 }
 
+template <class R>
+flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
+  constexpr int U = unrollFor(0);
+  uint64_t total = 0;
+  a->tileStart[0] = 0;
+  for (int c = 0; c < a->nchunks; c++) {
+    total += a->cnt[c] ? chunkPlan<R::ES, U>(*a, c).tiles() : 0;
+    if (total > 0x7ffffff0ull) return flagcxInvalidArgument;
+    a->tileStart[c + 1] = (uint32_t)total;
+  }
+  if (total == 0) return flagcxSuccess;
+  return launchKernel(reduceChunksRuntime<R, U>, (uint32_t)total, s, *a);
+}
+
 template <class R, int K, bool BCAST = true>
 void fillSet(KernelSet &ks) {
   ks.direct[K] = &launchDirect<R, K>;
@@ -221,6 +237,7 @@ KernelSet makeSet() {
   fillSet<R, 7>(ks);
   fillSet<R, 8>(ks);
   ks.bcastRuntime = &launchBcastRuntime<R>;
+  ks.chunksRuntime = &launchChunksRuntime<R>;
   ks.elemSize = R::ES;
   return ks;
 }
@@ -231,6 +248,7 @@ KernelSet makeCopySet() {
   KernelSet ks = {};
   fillSet<CopyRed<ES>, 1, true>(ks);
   ks.bcastRuntime = &launchBcastRuntime<CopyRed<ES>>;
+  ks.chunksRuntime = &launchChunksRuntime<CopyRed<ES>>;
   ks.elemSize = ES;
   return ks;
 }

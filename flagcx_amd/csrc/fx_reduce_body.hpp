@@ -646,6 +646,38 @@ __device__ __forceinline__ void storeElems(const SegMany &sg, uint64_t e0, int l
   for (int o = 0; o < sg.nmore; o++) scatterElems<ES>(sg.outp(o), e0, lo, hi, v);
 }
 
+// One chunk of a chunked collective over many ranks: the fold starts at input
+// `first` and wraps, or reads the single input `only`; the result goes to one
+// output or to all of them.  Pointer tables stay in the kernel argument block.
+struct SegChunk {
+  const void *const *rawIn;
+  void *const *rawOut;   // outputs after the primary one (nmore of them)
+  uint64_t inAdj;        // byte offset of the chunk in every input, minus the output's misalignment
+  uint64_t outAdj;       // the same for the extra outputs
+  char *out;
+  uint64_t lead, end;
+  int k, first, only, nmore;
+  __device__ __forceinline__ int inputs() const { return only >= 0 ? 1 : k; }
+  __device__ __forceinline__ const char *inp(int p) const {
+    int idx = only;
+    if (idx < 0) {
+      idx = first + p;
+      if (idx >= k) idx -= k;
+    }
+    return asGlobal(rawIn[idx]) + inAdj;
+  }
+  __device__ __forceinline__ char *outp(int o) const { return asGlobal(rawOut[o]) + outAdj; }
+};
+__device__ __forceinline__ void storeVector(const SegChunk &sg, uint64_t byteOff, u32x4 v) {
+  stg_stream(sg.out + byteOff, v);
+  for (int o = 0; o < sg.nmore; o++) stg_stream(sg.outp(o) + byteOff, v);
+}
+template <int ES>
+__device__ __forceinline__ void storeElems(const SegChunk &sg, uint64_t e0, int lo, int hi, u32x4 v) {
+  scatterElems<ES>(sg.out, e0, lo, hi, v);
+  for (int o = 0; o < sg.nmore; o++) scatterElems<ES>(sg.outp(o), e0, lo, hi, v);
+}
+
 // Reduce vector j of the segment with full bounds / alignment handling.
 template <class R, int K, class SG>
 __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
@@ -874,6 +906,66 @@ __global__ void __launch_bounds__(kBlock) reduceBcastRuntime(ManyArgs a) {
   for (int o = 1; o < a.nout; o++) co = co && sameLinePhase((uint64_t)(uintptr_t)a.out[o], (uint64_t)(uintptr_t)a.out[0]);
   const TilePlan tp = planTiles((uint64_t)(uintptr_t)a.out[0], a.count, R::ES, U, handOutFor(co, a.k));
   reduceTile<R, 0, U>(sg, tp, blockIdx.x, 0u);
+}
+
+__device__ __forceinline__ uint32_t findSlice(const uint32_t *tileStart, uint32_t n, uint32_t b);
+
+// Up to kMaxK chunks over up to kMaxK inputs and outputs in one launch.
+struct ChunkedArgs {
+  const void *in[kMaxK];
+  void *out[kMaxK];
+  uint64_t inOff[kMaxK], outOff[kMaxK];   // bytes
+  uint64_t cnt[kMaxK];                    // elements
+  uint32_t tileStart[kMaxK + 1];
+  int8_t first[kMaxK];                    // fold order starts at this input
+  int8_t only[kMaxK];                     // >= 0: this input alone
+  int8_t outSel[kMaxK];                   // >= 0: this output alone; -1: all nout
+  int k, nout, nchunks;
+};
+
+// Whether every stream of a chunk sits at the primary output's offset within a
+// cache line; shared by the kernel and by the host's tile count.
+__host__ __device__ inline bool chunkCoAligned(const ChunkedArgs &a, int c) {
+  const int primary = a.outSel[c] >= 0 ? a.outSel[c] : 0;
+  const uint64_t o = (uint64_t)(uintptr_t)a.out[primary] + a.outOff[c];
+  bool co = true;
+  if (a.only[c] >= 0) {
+    co = sameLinePhase((uint64_t)(uintptr_t)a.in[a.only[c]] + a.inOff[c], o);
+  } else {
+    for (int p = 0; p < a.k; p++) co = co && sameLinePhase((uint64_t)(uintptr_t)a.in[p] + a.inOff[c], o);
+  }
+  if (a.outSel[c] < 0)
+    for (int r = 1; r < a.nout; r++) co = co && sameLinePhase((uint64_t)(uintptr_t)a.out[r] + a.outOff[c], o);
+  return co;
+}
+template <int ES, int U>
+__host__ __device__ inline TilePlan chunkPlan(const ChunkedArgs &a, int c) {
+  const int primary = a.outSel[c] >= 0 ? a.outSel[c] : 0;
+  return planTiles((uint64_t)(uintptr_t)a.out[primary] + a.outOff[c], a.cnt[c], ES, U,
+                   handOutFor(chunkCoAligned(a, c), a.only[c] >= 0 ? 1 : a.k));
+}
+
+template <class R, int U>
+__global__ void __launch_bounds__(kBlock) reduceChunksRuntime(ChunkedArgs a) {
+  const uint32_t b = blockIdx.x;
+  const uint32_t c = findSlice(a.tileStart, (uint32_t)a.nchunks, b);
+  const int primary = a.outSel[c] >= 0 ? a.outSel[c] : 0;
+  const uint64_t o = (uint64_t)(uintptr_t)a.out[primary] + a.outOff[c];
+  const uint64_t mis = o & 15u;
+  SegChunk sg;
+  sg.rawIn = a.in;
+  sg.rawOut = a.out + 1;
+  sg.inAdj = a.inOff[c] - mis;
+  sg.outAdj = a.outOff[c] - mis;
+  sg.out = asGlobal((void *)(uintptr_t)o) - mis;
+  sg.lead = mis / R::ES;
+  sg.end = sg.lead + a.cnt[c];
+  sg.k = a.k;
+  sg.first = a.first[c];
+  sg.only = a.only[c];
+  sg.nmore = a.outSel[c] >= 0 ? 0 : a.nout - 1;
+  const TilePlan tp = chunkPlan<R::ES, U>(a, (int)c);
+  reduceTile<R, 0, U>(sg, tp, b - a.tileStart[c], a.tileStart[c] & 7u);
 }
 
 template <class R, int K, int U>

@@ -208,6 +208,14 @@ flagcxResult_t flushKway(const Ctx &c, SliceList &descs, KwayRun &run) {
   return rc;
 }
 
+// The many-rank kernels store one result to several buffers with shared byte
+// offsets: the receive buffers must agree in their low four address bits.
+inline bool recvsAlignedAlike(const Ctx &c) {
+  for (int r = 1; r < c.n; r++)
+    if ((((uintptr_t)c.recv(r) ^ (uintptr_t)c.recv(0)) & 15u) != 0) return false;
+  return true;
+}
+
 // One read, n stores: usable when both the inputs and the outputs of a
 // descriptor fit its eight slots.
 inline bool canBroadcast(const Ctx &c) { return c.n <= FX_MAX_SLICE_INPUTS; }
@@ -476,6 +484,17 @@ flagcxResult_t runAllReduce(const Ctx &c) {
     return R(fx_reduce_bcast(outs.data(), n, ins.data(), n, cnt, g->dtype, g->op, first, c.s));
   };
   if (g->order != FX_ORDER_RING) return bcast(0, count, 0);
+  if (n <= FX_MAX_INPUTS && recvsAlignedAlike(c)) {   // every chunk in one launch
+    fx::SmallVec<fxChunk, 16> chunks;
+    for (int ch = 0; ch < n; ch++) {
+      size_t ccnt, coff;
+      fx_split(count, n, ch, &ccnt, &coff);
+      chunks.push_back(fxChunk{coff, coff, ccnt, ch, -1, -1});
+    }
+    for (int j = 0; j < n; j++) ins[j] = c.send(j);
+    for (int r = 0; r < n; r++) outs[r] = c.recv(r);
+    return R(fx_reduce_chunks(outs.data(), n, ins.data(), n, chunks.data(), n, g->dtype, g->op, c.s));
+  }
   for (int ch = 0; ch < n; ch++) {
     size_t ccnt, coff;
     fx_split(count, n, ch, &ccnt, &coff);
@@ -601,6 +620,17 @@ flagcxResult_t runReduceScatter(const Ctx &c) {
     }
     return flagcxSuccess;
   }
+  if (n > FX_MAX_SLICE_INPUTS && n <= FX_MAX_INPUTS) {   // chunk r of every send buffer onto rank r, all in one launch
+    fx::SmallVec<fxChunk, 16> chunks;
+    PtrList ins;
+    fx::SmallVec<void *, 16> outs;
+    for (int r = 0; r < n; r++) {
+      chunks.push_back(fxChunk{(size_t)r * rcount, 0, rcount, (g->order == FX_ORDER_RING) ? mod(r + 1, n) : 0, -1, r});
+      ins.push_back(c.send(r));
+      outs.push_back(c.recv(r));
+    }
+    return R(fx_reduce_chunks(outs.data(), n, ins.data(), n, chunks.data(), n, g->dtype, g->op, c.s));
+  }
   for (int r = 0; r < n; r++) {
     const int first = (g->order == FX_ORDER_RING) ? mod(r + 1, n) : 0;
     flagcxResult_t rc = forPieces(g, rcount, (size_t)r * rcount, nred, [&](size_t off, size_t inSlice, size_t cnt) {
@@ -624,6 +654,17 @@ flagcxResult_t runAllGather(const Ctx &c) {
       bd[r].count = bytes;
     }
     return R(fx_reduce_bcast_slices(bd.data(), bd.size(), 1, c.n, 0, -1, c.s));
+  }
+  if (c.n <= FX_MAX_INPUTS && recvsAlignedAlike(c)) {   // rank q's block into slot q of every rank, all in one launch
+    fx::SmallVec<fxChunk, 16> chunks;
+    PtrList ins;
+    fx::SmallVec<void *, 16> outs;
+    for (int q = 0; q < c.n; q++) {
+      chunks.push_back(fxChunk{0, (size_t)q * bytes, bytes, 0, q, -1});
+      ins.push_back(c.send(q));
+      outs.push_back(c.recv(q));
+    }
+    return R(fx_reduce_chunks(outs.data(), c.n, ins.data(), c.n, chunks.data(), c.n, 0, -1, c.s));
   }
   SliceList descs;
   for (int r = 0; r < c.n; r++)

@@ -55,6 +55,13 @@ def reduce_bcast(outs, ins, count, dtype, op, first=0, stream=None):
     return lib.fx_reduce_bcast(_ptr_array(outs), len(outs), _ptr_array(ins), len(ins), count, dtype, op, first, stream)
 
 
+def reduce_chunks(outs, ins, chunks, dtype, op, stream=None):
+    """chunks: iterable of (in_off, out_off, count, first, in_sel, out_sel); op = -1 copies (bytes)."""
+    chunks = list(chunks)
+    arr = (N.Chunk * max(len(chunks), 1))(*[N.Chunk(*c) for c in chunks])
+    return lib.fx_reduce_chunks(_ptr_array(outs), len(outs), _ptr_array(ins), len(ins), arr, len(chunks), dtype, op, stream)
+
+
 def copy_slices(descs, stream=None):
     """descs: iterable of (src, dst, nbytes)."""
     arr, n = make_slices(([s], d, b) for s, d, b in descs)

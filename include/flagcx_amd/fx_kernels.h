@@ -202,6 +202,25 @@ int fx_reduce_bcast(void *const *outs, int nout, const void *const *ins, int k,
                     size_t count, int dtype, int op, int first, void *stream);
 
 /*
+ * Several chunks of one collective over up to FX_MAX_INPUTS ranks in ONE
+ * launch -- what a reduce-scatter, an all-gather or a ring-order all-reduce
+ * over more ranks than a slice descriptor has slots is made of.  Chunk c takes
+ * `count` elements at element offset in_off of the inputs: all k of them, folded
+ * in the order first, first + 1, ... (wrapping), or the single input in_sel
+ * (in_sel >= 0).  The result goes to element offset out_off of every output
+ * (out_sel = -1) or of output out_sel alone.  op = -1 copies (every chunk
+ * names its in_sel; offsets and counts in bytes).  Outputs of one chunk that do
+ * not share an offset within 16 bytes are refused (flagcxInvalidArgument).
+ */
+typedef struct fxChunk {
+  uint64_t in_off, out_off, count;
+  int first, in_sel, out_sel;
+} fxChunk;
+int fx_reduce_chunks(void *const *outs, int nout, const void *const *ins, int k,
+                     const fxChunk *chunks, int nchunks, int dtype, int op,
+                     void *stream);
+
+/*
  * Copy n independent byte ranges (in[0] -> out, `count` = BYTES): the Cpy node
  * and the all-gather landing copies (uni_runner_impl.cc:322-344,1649-1662;
  * flagcx/core/p2p.cc:257-283) as one launch.

@@ -243,6 +243,73 @@ def test_reduce_bcast_many_inputs_many_outputs(dev, dname):
     assert K.reduce_bcast([16], [16, 16], 4, dtype, -1) == N.INVALID_ARGUMENT
 
 
+@pytest.mark.parametrize("dname", ["bf16", "fp32", "int64", "uint8"])
+def test_reduce_chunks_is_a_collective_over_many_ranks_in_one_launch(dev, dname):
+    """fx_reduce_chunks with the three shapes it exists for, 12 and 17 ranks:
+    a ring-order all-reduce (chunk c folded from rank c on, stored to every rank),
+    a reduce-scatter (chunk r of every send buffer folded onto rank r alone) and an
+    all-gather (rank q's block copied into slot q of every rank), each in one call,
+    with ragged chunk sizes, an empty chunk and buffers off 16-byte alignment."""
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    npdt = N.NP_DTYPE[dtype]
+    for n, count, mis in ((12, 100003, 0), (17, 40000, 3), (9, 5, 1), (64, 6400, 0)):
+        sends = seeded_inputs(dtype, n, count, seed=n)
+        base, rem = divmod(count, n)
+        cnt = [base + (c < rem) for c in range(n)]
+        off = [c * base + min(c, rem) for c in range(n)]
+        with DevBufs(dev) as b:
+            ds = [b.put(a, pad_before=mis * es) for a in sends]
+            lead = mis * es
+            raw = [b.alloc(lead + count * es + 64) for _ in range(n)]
+            for q in raw:
+                dev.memset(q, 0xA5, lead + count * es + 64)
+            dr = [q + lead for q in raw]
+            # ring-order all-reduce
+            ch = [(off[c], off[c], cnt[c], c, -1, -1) for c in range(n)]
+            N.check(K.reduce_chunks(dr, ds, ch, dtype, N.OP_SUM), "all-reduce chunks")
+            dev.sync()
+            want = np.empty(count, npdt)
+            for c in range(n):
+                want[off[c]:off[c] + cnt[c]] = O.reduce_copy([a[off[c]:off[c] + cnt[c]] for a in sends], dtype, N.OP_SUM,
+                                                             first=c) if cnt[c] else []
+            for r in range(n):
+                assert_parity(dev.to_host(dr[r], count, npdt), want, dtype, N.OP_SUM, f"{dname} n={n} all-reduce rank {r}")
+                assert (dev.to_host(dr[r] + count * es, 32, np.uint8) == 0xA5).all()
+                if lead:
+                    assert (dev.to_host(raw[r], lead, np.uint8) == 0xA5).all()
+            # reduce-scatter: chunk r -> rank r, at the start of its buffer
+            for q in raw:
+                dev.memset(q, 0xA5, lead + count * es + 64)
+            ch = [(off[r], 0, cnt[r], (r + 1) % n, -1, r) for r in range(n)]
+            N.check(K.reduce_chunks(dr, ds, ch, dtype, N.OP_MAX), "reduce-scatter chunks")
+            dev.sync()
+            for r in range(n):
+                if cnt[r]:
+                    w = O.reduce_copy([a[off[r]:off[r] + cnt[r]] for a in sends], dtype, N.OP_MAX, first=(r + 1) % n)
+                    assert_parity(dev.to_host(dr[r], cnt[r], npdt), w, dtype, N.OP_MAX, f"{dname} n={n} reduce-scatter rank {r}")
+                assert (dev.to_host(dr[r] + cnt[r] * es, 32, np.uint8) == 0xA5).all(), "wrote past a reduce-scatter chunk"
+            # all-gather as a copy: block q of `blk` bytes from rank q into slot q of every rank
+            blk = (count // n) * es
+            if blk:
+                for q in raw:
+                    dev.memset(q, 0xA5, lead + count * es + 64)
+                ch = [(0, q * blk, blk, 0, q, -1) for q in range(n)]
+                N.check(K.reduce_chunks(dr, ds, ch, dtype, -1), "all-gather chunks")
+                dev.sync()
+                want8 = np.concatenate([a.view(np.uint8)[:blk] for a in sends])
+                for r in range(n):
+                    assert np.array_equal(dev.to_host(dr[r], n * blk, np.uint8), want8), f"all-gather rank {r}"
+                    assert (dev.to_host(dr[r] + n * blk, 16, np.uint8) == 0xA5).all()
+    with DevBufs(dev) as b:
+        p = b.alloc(64)
+        assert K.reduce_chunks([p], [p], [(0, 0, 4, 1, -1, -1)], dtype, N.OP_SUM) == N.INVALID_ARGUMENT     # first >= k
+        assert K.reduce_chunks([p], [p], [(0, 0, 4, 0, -1, 1)], dtype, N.OP_SUM) == N.INVALID_ARGUMENT      # out_sel >= nout
+        assert K.reduce_chunks([p], [p], [(0, 0, 4, 0, -1, -1)], dtype, -1) == N.INVALID_ARGUMENT           # a copy names its input
+        assert K.reduce_chunks([p, p + 4], [p], [(0, 0, 1, 0, -1, -1)], N.DT_UINT8, N.OP_SUM) == N.INVALID_ARGUMENT
+        assert K.reduce_chunks([p], [p], [], dtype, N.OP_SUM) == N.SUCCESS
+
+
 def _random_layout(rng, counts, slack):
     """Random non-overlapping displacements for the given segment counts."""
     order = rng.permutation(len(counts))

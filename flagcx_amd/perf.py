@@ -298,6 +298,38 @@ def run_allreduce(dev, a):
                 nbytes *= a.factor
 
 
+def run_collectives(dev, a):
+    """Every reducing / gathering collective over n simulated ranks, per order and algorithm, at one size per rank:
+    time per collective and TB/s of the least traffic the collective can do on one GPU."""
+    t = Timer(dev, warmup=2, iters=5)
+    per_rank = size(a.min)
+    dtype = DT[a.dtype]
+    es = N.DTYPE_SIZE[dtype]
+    orders = {S.ORDER_RANK: "rank", S.ORDER_RING: "ring", S.ORDER_TREE: "tree", S.ORDER_HOST: "host"}
+    print(f"{a.dtype}, {per_rank} B per rank; TB/s of: all-reduce (k+n) x size, reduce (n+1) x size, reduce-scatter (n+1) x size, "
+          f"all-gather (1+n) x size  [size = bytes per rank]")
+    for n in (2, 4, 8, 12, 16):
+        count = per_rank // es
+        ds = [dev.malloc(per_rank) for _ in range(n)]
+        dr = [dev.malloc(per_rank) for _ in range(n)]
+        for p in ds:
+            dev.memset(p, 1, per_rank)
+        for algo in (S.ALGO_DIRECT, S.ALGO_RING):
+            for order, oname in orders.items():
+                with S.SimGroup(n, algo=algo, order=order) as g:
+                    rc = count // n
+                    ms = [t.ms(lambda: N.check(g.all_reduce(ds, dr, count, dtype, OP[a.op], t.stream))),
+                          t.ms(lambda: N.check(g.reduce(ds, [dr[0]] + [None] * (n - 1), count, dtype, OP[a.op], 0, t.stream))),
+                          t.ms(lambda: N.check(g.reduce_scatter(ds, dr, rc, dtype, OP[a.op], t.stream))),
+                          t.ms(lambda: N.check(g.all_gather(ds, dr, rc, dtype, t.stream)))]
+                units = [2 * n, n + 1, n + 1, 1 + n]
+                cells = "  ".join(f"{m * 1e3:8.1f} us {u * per_rank / m / 1e9:5.2f}" for m, u in zip(ms, units))
+                print(f"n={n:2d} {'ring  ' if algo else 'direct'} {oname:4s} | all-reduce, reduce, reduce-scatter, all-gather: {cells}",
+                      flush=True)
+        for p in ds + dr:
+            dev.free(p)
+
+
 def run_torchref():
     """PyTorch's own kernels on the same shapes, as a reference point on the same box: torch.add(out=) for the
     two-input sum, Tensor.copy_ for the copy, and the 8-input bf16 sum done the torch way.  Uses torch only."""
@@ -342,7 +374,7 @@ def run_torchref():
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo", "torchref"])
+    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo", "collectives", "torchref"])
     ap.add_argument("-k", type=int, default=4)
     ap.add_argument("-n", "--nranks", type=int, default=8)
     ap.add_argument("-d", "--dtype", default="fp32", choices=list(DT))
@@ -364,7 +396,7 @@ def main(argv=None):
         return run_torchref()
     dev = Device(0)
     {"reduce": run_reduce, "slices": run_slices, "pack": run_pack, "allreduce": run_allreduce,
-     "fifo": run_fifo}[a.what](dev, a)
+     "fifo": run_fifo, "collectives": run_collectives}[a.what](dev, a)
 
 
 if __name__ == "__main__":

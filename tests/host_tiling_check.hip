@@ -70,8 +70,8 @@ int main() {
             const uint64_t V = (uint64_t)U * kBlock * 16 / es;   // elements per tile
             const uint64_t small[] = {0, 1, 2, 16 / (uint64_t)es - 1, 16 / (uint64_t)es, 16 / (uint64_t)es + 1, V - 1, V,
                                       V + 1, 3 * V + 7};
-            const uint64_t zone = 4 * MiB / es;
-            const uint64_t big[] = {zone - 1, zone, zone + 1, zone + V * 64 - 3, 2 * zone + 12345, 9 * MiB / es + 1};
+            const uint64_t zone = kStripeMinBytes / es;   // lengths around the striping threshold, and well above it
+            const uint64_t big[] = {zone - 1, zone, zone + 1, zone + V * 64 - 3, 2 * zone + 12345, 4 * MiB / es + 1, 9 * MiB / es + 1};
             for (uint64_t c : small) {
               long rc = checkOne(base + mis, c, es, U, co);
               cases++;

@@ -347,7 +347,7 @@ int main(void) {
 
 def test_kernel_index_arithmetic_on_the_host(tmp_path):
     """tests/host_tiling_check.hip drives fx::planTiles and fx::laneOfTile -- the
-    functions the kernels themselves call -- over 13,688 (address, length, element
+    functions the kernels themselves call -- over 14,168 (address, length, element
     size, unroll, hand-out, die shift) cases and checks that every vector of a segment
     is handled exactly once, the unchecked path only ever sees whole in-segment
     vectors, and nothing outside the segment is touched."""

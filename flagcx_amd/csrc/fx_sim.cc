@@ -768,6 +768,12 @@ flagcxResult_t runBroadcast(const Ctx &c) {
     b.count = bytes;
     return R(fx_reduce_bcast_slices(&b, 1, 1, c.n, 0, -1, c.s));
   }
+  if (bytes && c.n <= FX_MAX_INPUTS) {   // more ranks: the run-time form of the same one-read-n-stores copy
+    fx::SmallVec<void *, 16> outs;
+    for (int r = 0; r < c.n; r++) outs.push_back(c.recv(r));
+    const void *src = c.send(c.g->root);
+    return R(fx_reduce_bcast(outs.data(), c.n, &src, 1, bytes, 0, -1, 0, c.s));
+  }
   SliceList d;
   for (int r = 0; r < c.n && bytes; r++)
     if (c.recv(r) != c.send(c.g->root)) d.push_back(copyDesc(c.send(c.g->root), c.recv(r), bytes));

@@ -721,3 +721,71 @@ def test_host_staged_reduce_and_reduce_scatter_match_host_order_and_oracle(dev, 
                 assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(outs[r]).view(np.uint8)), f"rank {r} op {op} vs the oracle"
                 assert np.array_equal(got.view(np.uint8), dev.to_host(dd[r], rc_el, npdt).view(np.uint8)), f"rank {r} vs FX_ORDER_HOST"
                 assert (dev.to_host(dr[r] + rc_el * es, 16, np.uint8) == 0x5A).all(), "wrote past the received chunk"
+
+
+@pytest.mark.parametrize("n,count,phase", [(9, 1001, 0), (12, 70001, 4), (16, 3, 0), (17, 262147, 8), (33, 4099, 0)])
+def test_byte_moving_collectives_over_many_ranks(dev, stream, n, count, phase):
+    """Broadcast, gather, scatter and alltoall past eight ranks: every receive
+    buffer holds exactly the bytes the definition names, the bytes on either
+    side of it stay as they were, and the root may run in place
+    (flagcx/adaptor/ccl/rccl_adaptor.cc:126-184,222-246 builds them from
+    grouped send/recv pairs)."""
+    rng = np.random.default_rng(n * 1000 + count)
+    root = (2 * n) // 3
+    guard = 64
+    fill = np.full(guard, 0xA5, np.uint8)
+
+    def framed(b, nelem, init=None):
+        """A device buffer of nelem int32 at `phase` bytes past a guard, with guards on both sides."""
+        body = init if init is not None else np.full(nelem, -1, np.int32)
+        host = np.concatenate([fill, np.zeros(phase, np.uint8), body.view(np.uint8), fill])
+        return b.put(host) + guard + phase
+
+    def check(b, p, want, what):
+        got = dev.to_host(p - guard - phase, 2 * guard + phase + want.nbytes, np.uint8)
+        assert (got[:guard] == 0xA5).all() and (got[-guard:] == 0xA5).all(), f"{what}: guard bytes written"
+        assert np.array_equal(got[guard + phase:-guard].view(np.int32), want), what
+
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        def each(fn, name):
+            for r in range(n):
+                N.check(fn(r), name)
+            dev.stream_sync(stream)
+
+        # broadcast: out of place everywhere, then in place on the root
+        src = [rng.integers(-2**31, 2**31 - 1, count, dtype=np.int32) for _ in range(n)]
+        ds = [framed(b, count, src[r]) for r in range(n)]
+        dr = [framed(b, count) for _ in range(n)]
+        each(lambda r: N.lib.flagcxBroadcast(ds[r], dr[r], count, N.DT_INT32, root, g.comms[r], stream), "flagcxBroadcast")
+        for r in range(n):
+            check(b, dr[r], src[root], f"broadcast to rank {r}")
+            check(b, ds[r], src[r], f"broadcast left rank {r}'s send buffer alone")
+        dr2 = [ds[r] if r == root else framed(b, count) for r in range(n)]
+        each(lambda r: N.lib.flagcxBroadcast(ds[r], dr2[r], count, N.DT_INT32, root, g.comms[r], stream), "flagcxBroadcast")
+        for r in range(n):
+            check(b, dr2[r], src[root], f"in-place broadcast to rank {r}")
+
+        # gather to the root, root's own block already in place
+        gat = framed(b, n * count)
+        gs = [gat + root * count * 4 if r == root else ds[r] for r in range(n)]
+        dev.upload(gat + root * count * 4, src[root])
+        each(lambda r: N.lib.flagcxGather(gs[r], gat if r == root else None, count, N.DT_INT32, root, g.comms[r], stream),
+             "flagcxGather")
+        check(b, gat, np.concatenate(src), "gather")
+
+        # scatter the gathered buffer back out
+        sc = [framed(b, count) for _ in range(n)]
+        each(lambda r: N.lib.flagcxScatter(gat if r == root else None, sc[r], count, N.DT_INT32, root, g.comms[r], stream),
+             "flagcxScatter")
+        for r in range(n):
+            check(b, sc[r], src[r], f"scatter to rank {r}")
+
+        # alltoall: block i of rank r becomes block r of rank i
+        blk = max(count // n, 1)
+        a2a = [rng.integers(-2**31, 2**31 - 1, n * blk, dtype=np.int32) for _ in range(n)]
+        da = [framed(b, n * blk, a2a[r]) for r in range(n)]
+        db = [framed(b, n * blk) for _ in range(n)]
+        each(lambda r: N.lib.flagcxAlltoAll(da[r], db[r], blk, N.DT_INT32, g.comms[r], stream), "flagcxAlltoAll")
+        for i in range(n):
+            want = np.concatenate([a2a[r][i * blk:(i + 1) * blk] for r in range(n)])
+            check(b, db[i], want, f"alltoall at rank {i}")

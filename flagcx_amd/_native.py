@@ -115,6 +115,7 @@ _SIGS.update({
     "fxSimCommInitAll": (_i, [C.POINTER(_vp), _i]),
     "fxSimCommDestroyAll": (_i, [C.POINTER(_vp), _i]),
     "fxSimCommConfig": (_i, [_vp, _i, C.c_longlong]),
+    "fxSimCommProgress": (_i, [_vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "fxSimRegisterWindows": (_i, [_vp, C.POINTER(_vp), _sz]),
     "fxSimCommInitRank": (_i, [C.POINTER(_vp), _i, _vp, _sz, _i]),
     "fxSimCommDestroy": (_i, [_vp]),

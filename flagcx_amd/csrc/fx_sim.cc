@@ -861,6 +861,7 @@ flagcxResult_t postAndMaybeRun(flagcxComm_t comm, Kind kind, const void *send, v
 struct flagcxComm {
   Group *g;
   int rank;
+  uint64_t joined = 0;   // how many collectives the group had launched when this rank's last post was accepted
 };
 
 namespace {
@@ -903,6 +904,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   p.send = send;
   p.recv = recv;
   p.stream = stream->base;
+  comm->joined = g->launched;
   if (kind == kAlltoAllv) {
     p.sendcounts.assign(sc, sc + g->n);
     p.sdispls.assign(sd, sd + g->n);
@@ -1269,6 +1271,14 @@ const char *flagcxGetErrorString(flagcxResult_t result) {
 
 flagcxResult_t flagcxBarrier(flagcxComm_t comm, flagcxStream_t stream) {
   return postAndMaybeRun(comm, kBarrier, nullptr, nullptr, 0, 0, 0, 0, stream);
+}
+
+flagcxResult_t fxSimCommProgress(flagcxComm_t comm, uint64_t *joined, uint64_t *launched) {
+  if (!comm || !comm->g || !joined || !launched) return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(comm->g->mu);
+  *joined = comm->joined;
+  *launched = comm->g->launched;
+  return flagcxSuccess;
 }
 
 flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {

@@ -76,6 +76,12 @@ class SimGroup:
             lambda r, s: lib.flagcxAlltoAllv(sends[r], _szs(sendcounts[r]), _szs(sdispls[r]), recvs[r],
                                              _szs(recvcounts[r]), _szs(rdispls[r]), dtype, self.comms[r], s), streams)
 
+    def progress(self, rank):
+        """(launch count when `rank`'s latest collective call was accepted, launch count now)."""
+        joined, launched = C.c_uint64(), C.c_uint64()
+        N.check(lib.fxSimCommProgress(self.comms[rank], C.byref(joined), C.byref(launched)), "fxSimCommProgress")
+        return joined.value, launched.value
+
     def register_windows(self, windows, nbytes):
         arr = (C.c_void_p * self.n)(*windows) if windows else None
         return lib.fxSimRegisterWindows(self.comms[0], arr, nbytes)

@@ -9,7 +9,10 @@
 // object joins the same in-process group through the unique id rank 0 leaves in
 // the store, and a collective is launched by the last rank that posts it.  A
 // rank's results are therefore defined once every rank has posted; wait() on a
-// Work is meant to be called then (with one rank, at once).
+// Work is meant to be called then (with one rank, at once).  Copies that a
+// call owes its caller behind the collective (out of a staging tensor into a
+// list of output tensors) are enqueued, on the rank's own stream, by whichever
+// call finds the collective launched -- normally the last rank's.
 #include <dlfcn.h>
 #include <hip/hip_runtime.h>
 
@@ -24,6 +27,8 @@
 #include <algorithm>
 #include <cstring>
 #include <functional>
+#include <map>
+#include <mutex>
 #include <numeric>
 #include <string>
 #include <vector>
@@ -122,11 +127,8 @@ void checkDense(const at::Tensor &t, const char *what) {
 
 class FxWork : public Work {
  public:
-  // `finish`: what is left to do on the stream once the collective has been
-  // launched (copies out of a staging tensor into a list of output tensors);
-  // it runs at the first wait.
-  FxWork(int rank, OpType op, hipStream_t stream, Tensors outputs, std::function<void()> finish = nullptr)
-      : Work(rank, op), stream_(stream), outputs_(std::move(outputs)), finish_(std::move(finish)) {
+  FxWork(int rank, OpType op, hipStream_t stream, Tensors outputs)
+      : Work(rank, op), stream_(stream), outputs_(std::move(outputs)) {
     std::vector<c10::Device> devices;
     for (const auto &t : outputs_)
       if (std::find(devices.begin(), devices.end(), t.device()) == devices.end()) devices.push_back(t.device());
@@ -137,14 +139,12 @@ class FxWork : public Work {
     if (event_) (void)hipEventDestroy(event_);
   }
   bool isCompleted() override {
-    finishOnce();
     mark();
     return hipEventQuery(event_) == hipSuccess;
   }
   bool isSuccess() const override { return true; }
   // Orders the caller's current stream after the collective; never blocks the host.
   bool wait(std::chrono::milliseconds /*timeout*/ = kNoTimeout) override {
-    finishOnce();
     const hipStream_t cur = c10::hip::getCurrentHIPStream().stream();
     if (cur != stream_) {
       mark();
@@ -165,31 +165,49 @@ class FxWork : public Work {
     if (!event_) TORCH_CHECK(hipEventCreateWithFlags(&event_, hipEventDisableTiming) == hipSuccess, "hipEventCreate failed");
     TORCH_CHECK(hipEventRecord(event_, stream_) == hipSuccess, "hipEventRecord failed");
   }
-  void finishOnce() {
-    if (!finish_) return;
-    std::function<void()> f;
-    f.swap(finish_);
-    // the copies go where the collective went, whatever stream is current now
-    const c10::hip::HIPStream before = c10::hip::getCurrentHIPStream();
-    if (before.stream() == stream_) {
-      f();
-      return;
-    }
-    c10::hip::setCurrentHIPStream(c10::hip::getStreamFromExternal(stream_, before.device_index()));
-    try {
-      f();
-    } catch (...) {
-      c10::hip::setCurrentHIPStream(before);
-      throw;
-    }
-    c10::hip::setCurrentHIPStream(before);
-  }
   hipStream_t stream_;
   hipEvent_t event_ = nullptr;
   Tensors outputs_;
-  std::function<void()> finish_;
   c10::intrusive_ptr<c10::ivalue::Future> future_;
 };
+
+// Copies owed behind collectives that have not been launched yet, per group of
+// simulated ranks (the key is the group's unique id).
+struct Owed {
+  uint64_t joined;                 // the group's launch count when the collective was posted
+  c10::hip::HIPStream stream;      // the posting rank's stream
+  std::function<void()> finish;
+};
+std::mutex owedMu;
+std::map<std::string, std::vector<Owed>> owed;
+
+// Enqueue every owed copy of `group` whose collective has been launched, each on its own rank's stream.
+void payOwed(const std::string &group, uint64_t launched) {
+  std::vector<Owed> due;
+  {
+    std::lock_guard<std::mutex> lock(owedMu);
+    auto &v = owed[group];
+    for (size_t i = 0; i < v.size();) {
+      if (v[i].joined < launched) {
+        due.push_back(std::move(v[i]));
+        v.erase(v.begin() + (long)i);
+      } else {
+        i++;
+      }
+    }
+  }
+  const c10::hip::HIPStream before = c10::hip::getCurrentHIPStream();
+  try {
+    for (auto &o : due) {
+      c10::hip::setCurrentHIPStream(o.stream);
+      o.finish();
+    }
+  } catch (...) {
+    c10::hip::setCurrentHIPStream(before);
+    throw;
+  }
+  c10::hip::setCurrentHIPStream(before);
+}
 
 class FxBackend : public c10d::Backend {
  public:
@@ -207,9 +225,14 @@ class FxBackend : public c10d::Backend {
       std::memcpy(id.internal, bytes.data(), sizeof(id.internal));
     }
     ok(flagcxCommInitRank(&comm_, size, &id, rank), "flagcxCommInitRank");
+    group_.assign(id.internal, id.internal + sizeof(id.internal));
   }
   ~FxBackend() override {
     if (comm_) (void)flagcxCommDestroy(comm_);
+    if (getRank() == 0) {
+      std::lock_guard<std::mutex> lock(owedMu);
+      owed.erase(group_);
+    }
   }
 
   const std::string getBackendName() const override { return "flagcx"; }
@@ -223,16 +246,20 @@ class FxBackend : public c10d::Backend {
     });
   }
 
+  // One collective over the tensors laid end to end: with simulated ranks a
+  // rank may not post a second collective before the others have posted the first.
   c10::intrusive_ptr<Work> allreduce_coalesced(Tensors &tensors, const c10d::AllreduceCoalescedOptions &opts) override {
-    for (auto &t : tensors) checkDense(t, "allreduce_coalesced");
+    if (tensors.size() == 1) {
+      c10d::AllreduceOptions one;
+      one.reduceOp = opts.reduceOp;
+      return allreduce(tensors, one);
+    }
+    TORCH_CHECK(!tensors.empty(), "allreduce_coalesced: no tensors");
+    std::vector<size_t> displs, counts;
+    at::Tensor flat = flatten(tensors, "allreduce_coalesced", displs, counts);
     return run(OpType::ALLREDUCE_COALESCED, tensors, [&](flagcxStream_t s) {
-      for (auto &t : tensors) {
-        const flagcxResult_t rc = flagcxAllReduce(t.data_ptr(), t.data_ptr(), (size_t)t.numel(), dtypeOf(t),
-                                                  opOf(opts.reduceOp, t), comm_, s);
-        if (rc != flagcxSuccess) return rc;
-      }
-      return flagcxSuccess;
-    });
+      return flagcxAllReduce(flat.data_ptr(), flat.data_ptr(), (size_t)flat.numel(), dtypeOf(flat), opOf(opts.reduceOp, flat), comm_, s);
+    }, unpacker(flat, tensors, displs, counts), {flat});
   }
 
   c10::intrusive_ptr<Work> broadcast(Tensors &tensors, const c10d::BroadcastOptions &opts) override {
@@ -262,7 +289,7 @@ class FxBackend : public c10d::Backend {
     TORCH_CHECK(out.numel() == in.numel() * getSize(), "allgather_into_tensor: output must hold world_size inputs");
     return run(OpType::_ALLGATHER_BASE, {out}, [&](flagcxStream_t s) {
       return flagcxAllGather(in.data_ptr(), out.data_ptr(), (size_t)in.numel(), dtypeOf(in), comm_, s);
-    });
+    }, nullptr, {in});
   }
 
   c10::intrusive_ptr<Work> allgather(std::vector<Tensors> &outs, Tensors &ins, const c10d::AllgatherOptions &opts) override {
@@ -280,10 +307,31 @@ class FxBackend : public c10d::Backend {
     }, unpacker(flat, outs[0], displs, counts), {flat});
   }
 
+  // Every rank's inputs end to end, gathered once; output i is then rank 0's
+  // input i, rank 1's input i, ... copied out of the gathered rows.
   c10::intrusive_ptr<Work> allgather_into_tensor_coalesced(Tensors &outs, Tensors &ins, const c10d::AllgatherOptions &opts) override {
-    TORCH_CHECK(outs.size() == ins.size(), "allgather_into_tensor_coalesced: as many outputs as inputs");
-    for (size_t i = 0; i < ins.size(); i++) (void)_allgather_base(outs[i], ins[i], opts);
-    return c10::make_intrusive<FxWork>(getRank(), OpType::COALESCED, c10::hip::getCurrentHIPStream().stream(), outs);
+    TORCH_CHECK(outs.size() == ins.size() && !ins.empty(), "allgather_into_tensor_coalesced: as many outputs as inputs, at least one");
+    if (ins.size() == 1) return _allgather_base(outs[0], ins[0], opts);
+    const int n = getSize();
+    for (size_t i = 0; i < ins.size(); i++) {
+      checkDense(outs[i], "allgather_into_tensor_coalesced");
+      TORCH_CHECK(outs[i].scalar_type() == ins[i].scalar_type() && outs[i].numel() == ins[i].numel() * n,
+                  "allgather_into_tensor_coalesced: output ", i, " must hold world_size inputs of the same type");
+    }
+    std::vector<size_t> displs, counts;
+    at::Tensor flat = flatten(ins, "allgather_into_tensor_coalesced", displs, counts);
+    const int64_t total = flat.numel();
+    at::Tensor all = at::empty({(int64_t)n * total}, flat.options());
+    Tensors outsCopy = outs;
+    auto finish = [all, outsCopy, displs, counts, n, total]() mutable {
+      const at::Tensor rows = all.view({n, total});
+      for (size_t i = 0; i < outsCopy.size(); i++)
+        if (counts[i])
+          outsCopy[i].view({n, (int64_t)counts[i]}).copy_(rows.narrow(1, (int64_t)displs[i], (int64_t)counts[i]), true);
+    };
+    return run(OpType::COALESCED, outs, [&](flagcxStream_t s) {
+      return flagcxAllGather(flat.data_ptr(), all.data_ptr(), (size_t)total, dtypeOf(flat), comm_, s);
+    }, std::move(finish), {flat, all});
   }
 
   c10::intrusive_ptr<Work> _reduce_scatter_base(at::Tensor &out, at::Tensor &in, const c10d::ReduceScatterOptions &opts) override {
@@ -293,7 +341,7 @@ class FxBackend : public c10d::Backend {
     TORCH_CHECK(in.numel() == out.numel() * getSize(), "reduce_scatter_tensor: input must hold world_size outputs");
     return run(OpType::_REDUCE_SCATTER_BASE, {out}, [&](flagcxStream_t s) {
       return flagcxReduceScatter(in.data_ptr(), out.data_ptr(), (size_t)out.numel(), dtypeOf(in), opOf(opts.reduceOp, in), comm_, s);
-    });
+    }, nullptr, {in});
   }
 
   c10::intrusive_ptr<Work> reduce_scatter(Tensors &outs, std::vector<Tensors> &ins, const c10d::ReduceScatterOptions &opts) override {
@@ -310,10 +358,31 @@ class FxBackend : public c10d::Backend {
     }, nullptr, {flat});
   }
 
+  // Row r of the staged input holds part r of every input end to end, so that one
+  // reduce-scatter leaves this rank's part of every output in one row.
   c10::intrusive_ptr<Work> reduce_scatter_tensor_coalesced(Tensors &outs, Tensors &ins, const c10d::ReduceScatterOptions &opts) override {
-    TORCH_CHECK(outs.size() == ins.size(), "reduce_scatter_tensor_coalesced: as many outputs as inputs");
-    for (size_t i = 0; i < ins.size(); i++) (void)_reduce_scatter_base(outs[i], ins[i], opts);
-    return c10::make_intrusive<FxWork>(getRank(), OpType::COALESCED, c10::hip::getCurrentHIPStream().stream(), outs);
+    TORCH_CHECK(outs.size() == ins.size() && !ins.empty(), "reduce_scatter_tensor_coalesced: as many outputs as inputs, at least one");
+    if (ins.size() == 1) return _reduce_scatter_base(outs[0], ins[0], opts);
+    const int n = getSize();
+    Tensors rows;
+    std::vector<size_t> displs, counts;
+    size_t total = 0;
+    for (size_t i = 0; i < ins.size(); i++) {
+      checkDense(ins[i], "reduce_scatter_tensor_coalesced");
+      checkDense(outs[i], "reduce_scatter_tensor_coalesced");
+      TORCH_CHECK(ins[i].scalar_type() == ins[0].scalar_type() && outs[i].scalar_type() == ins[0].scalar_type(),
+                  "reduce_scatter_tensor_coalesced: one element type throughout");
+      TORCH_CHECK(ins[i].numel() == outs[i].numel() * n, "reduce_scatter_tensor_coalesced: input ", i, " must hold world_size outputs");
+      rows.push_back(ins[i].view({n, outs[i].numel()}));
+      displs.push_back(total);
+      counts.push_back((size_t)outs[i].numel());
+      total += (size_t)outs[i].numel();
+    }
+    at::Tensor staged = at::cat(rows, 1).contiguous();
+    at::Tensor mine = at::empty({(int64_t)total}, staged.options());
+    return run(OpType::COALESCED, outs, [&](flagcxStream_t s) {
+      return flagcxReduceScatter(staged.data_ptr(), mine.data_ptr(), total, dtypeOf(staged), opOf(opts.reduceOp, staged), comm_, s);
+    }, unpacker(mine, outs, displs, counts), {staged, mine});
   }
 
   c10::intrusive_ptr<Work> alltoall_base(at::Tensor &out, at::Tensor &in, std::vector<int64_t> &outSplit,
@@ -326,7 +395,7 @@ class FxBackend : public c10d::Backend {
       TORCH_CHECK(in.numel() == out.numel() && in.numel() % n == 0, "all_to_all_single: sizes must be equal and divide by world_size");
       return run(OpType::ALLTOALL_BASE, {out}, [&](flagcxStream_t s) {
         return flagcxAlltoAll(in.data_ptr(), out.data_ptr(), (size_t)(in.numel() / n), dtypeOf(in), comm_, s);
-      });
+      }, nullptr, {in});
     }
     // splits count rows of dimension 0; everything below it is one row
     auto layout = [n](const at::Tensor &t, const std::vector<int64_t> &split, std::vector<size_t> &counts, std::vector<size_t> &displs) {
@@ -349,7 +418,7 @@ class FxBackend : public c10d::Backend {
     layout(out, outSplit, rc, rd);
     return run(OpType::ALLTOALL_BASE, {out}, [&](flagcxStream_t s) {
       return flagcxAlltoAllv(in.data_ptr(), sc.data(), sd.data(), out.data_ptr(), rc.data(), rd.data(), dtypeOf(in), comm_, s);
-    });
+    }, nullptr, {in});
   }
 
   c10::intrusive_ptr<Work> alltoall(Tensors &outs, Tensors &ins, const c10d::AllToAllOptions &) override {
@@ -396,7 +465,7 @@ class FxBackend : public c10d::Backend {
     }
     return run(OpType::GATHER, getRank() == root ? outs[0] : Tensors{}, [&](flagcxStream_t s) {
       return flagcxGather(in.data_ptr(), flat.defined() ? flat.data_ptr() : nullptr, (size_t)in.numel(), dtypeOf(in), root, comm_, s);
-    }, std::move(finish), flat.defined() ? Tensors{flat} : Tensors{});
+    }, std::move(finish), flat.defined() ? Tensors{in, flat} : Tensors{in});
   }
 
   c10::intrusive_ptr<Work> scatter(Tensors &outs, std::vector<Tensors> &ins, const c10d::ScatterOptions &opts) override {
@@ -425,7 +494,7 @@ class FxBackend : public c10d::Backend {
     checkDense(t, "send");
     return run(OpType::SEND, {}, [&](flagcxStream_t s) {
       return flagcxSend(t.data_ptr(), (size_t)t.numel(), dtypeOf(t), dst, comm_, s);
-    });
+    }, nullptr, {t});
   }
 
   c10::intrusive_ptr<Work> recv(Tensors &tensors, int src, int /*tag*/) override {
@@ -442,6 +511,21 @@ class FxBackend : public c10d::Backend {
   }
 
  private:
+  // The tensors' elements end to end in a new tensor; where each one starts and how long it is.
+  static at::Tensor flatten(const Tensors &v, const char *what, std::vector<size_t> &displs, std::vector<size_t> &counts) {
+    Tensors parts;
+    size_t total = 0;
+    for (const auto &t : v) {
+      checkDense(t, what);
+      TORCH_CHECK(t.scalar_type() == v[0].scalar_type(), what, ": one element type throughout");
+      parts.push_back(t.reshape({-1}));
+      displs.push_back(total);
+      counts.push_back((size_t)t.numel());
+      total += (size_t)t.numel();
+    }
+    return at::cat(parts);
+  }
+
   // Copy pieces of a staging tensor into a list of output tensors, on the
   // collective's stream, after the launch.
   static std::function<void()> unpacker(at::Tensor flat, Tensors outs, std::vector<size_t> displs, std::vector<size_t> counts) {
@@ -451,25 +535,45 @@ class FxBackend : public c10d::Backend {
     };
   }
 
-  // `staging`: tensors of this call that the kernels read or write and the
-  // caller never sees.  With simulated ranks the launch may come from a later
-  // rank's call, so they are held here, not by the Work the caller may drop,
-  // until this rank's next collective has been accepted -- which the rank layer
-  // only does once the previous one has been launched.
+  // `staging`: tensors of this call that the kernels read or write and that
+  // nothing else keeps alive: staging the caller never sees, and inputs the
+  // caller may drop as soon as the call returns.  With simulated ranks the
+  // launch may come from a later rank's call, so they are held here, not by the
+  // Work the caller may drop, until this rank's next collective has been
+  // accepted -- which the rank layer only does once the previous one has been
+  // launched.
   template <class F>
   c10::intrusive_ptr<Work> run(OpType op, Tensors outputs, F call, std::function<void()> finish = nullptr,
                                Tensors staging = {}) {
-    const hipStream_t raw = c10::hip::getCurrentHIPStream().stream();
+    const c10::hip::HIPStream cur = c10::hip::getCurrentHIPStream();
+    const hipStream_t raw = cur.stream();
     BorrowedStream s(raw);
     ok(call(s.get()), c10d::opTypeToString(op).c_str());
-    held_ = std::move(staging);
-    auto work = c10::make_intrusive<FxWork>(getRank(), op, raw, std::move(outputs), std::move(finish));
-    if (getSize() == 1) (void)work->wait();   // one rank: the launch has happened, finish now
-    return work;
+    if (op == OpType::SEND) {
+      // The matching recv may come after this rank's next collective has been
+      // accepted, but not after the one that follows: that one is only accepted
+      // once the next has been launched, for which the receiver has posted it,
+      // and its recv before it.
+      for (auto &t : staging) sent_[0].push_back(std::move(t));
+    } else if (op != OpType::RECV) {
+      sent_[1] = std::move(sent_[0]);
+      sent_[0].clear();
+      held_ = std::move(staging);
+      uint64_t joined = 0, launched = 0;
+      ok(fxSimCommProgress(comm_, &joined, &launched), "fxSimCommProgress");
+      if (finish) {
+        std::lock_guard<std::mutex> lock(owedMu);
+        owed[group_].push_back(Owed{joined, cur, std::move(finish)});
+      }
+      if (launched > joined) payOwed(group_, launched);
+    }
+    return c10::make_intrusive<FxWork>(getRank(), op, raw, std::move(outputs));
   }
 
   flagcxComm_t comm_ = nullptr;
+  std::string group_;   // the unique id's bytes: what the ranks of one group share
   Tensors held_;
+  Tensors sent_[2];   // send buffers of the calls since the last collective, and of those before it
 };
 
 c10::intrusive_ptr<c10d::Backend> createBackend(const c10::intrusive_ptr<c10d::Store> &store, int rank, int size) {
@@ -481,4 +585,13 @@ c10::intrusive_ptr<c10d::Backend> createBackend(const c10::intrusive_ptr<c10d::S
 PYBIND11_MODULE(fx_c10d, m) {
   m.doc() = "torch.distributed backend over libflagcx_amd.so";
   m.def("create_backend", &createBackend, py::arg("store"), py::arg("rank"), py::arg("size"));
+  // torch binds these two on ProcessGroup only; a backend object on its own reaches them here
+  m.def("allgather_into_tensor_coalesced", [](const c10::intrusive_ptr<c10d::Backend> &b, Tensors outs, Tensors ins) {
+    return b->allgather_into_tensor_coalesced(outs, ins);
+  }, py::arg("backend"), py::arg("outputs"), py::arg("inputs"));
+  m.def("reduce_scatter_tensor_coalesced", [](const c10::intrusive_ptr<c10d::Backend> &b, Tensors outs, Tensors ins, const c10d::ReduceOp &op) {
+    c10d::ReduceScatterOptions o;
+    o.reduceOp = op;
+    return b->reduce_scatter_tensor_coalesced(outs, ins, o);
+  }, py::arg("backend"), py::arg("outputs"), py::arg("inputs"), py::arg("op") = c10d::ReduceOp(c10d::ReduceOp::SUM));
 }

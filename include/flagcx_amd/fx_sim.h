@@ -126,6 +126,16 @@ enum {
 };
 flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value);
 
+/* Where a rank stands (no counterpart in the reference, whose ranks are
+ * processes and whose collectives launch in the caller's own call): `joined` =
+ * the number of collectives the group had launched when this rank's latest
+ * collective call was accepted, `launched` = that number now.  The rank's
+ * latest collective has been enqueued, on its stream, once launched > joined;
+ * a caller with work to enqueue behind it (copies out of a staging buffer)
+ * asks here whether it may. */
+flagcxResult_t fxSimCommProgress(flagcxComm_t comm, uint64_t *joined,
+                                 uint64_t *launched);
+
 flagcxResult_t flagcxCommCount(const flagcxComm_t comm, int *count);
 flagcxResult_t flagcxCommUserRank(const flagcxComm_t comm, int *rank);
 

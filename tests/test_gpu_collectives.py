@@ -789,3 +789,20 @@ def test_byte_moving_collectives_over_many_ranks(dev, stream, n, count, phase):
         for i in range(n):
             want = np.concatenate([a2a[r][i * blk:(i + 1) * blk] for r in range(n)])
             check(b, db[i], want, f"alltoall at rank {i}")
+
+
+def test_progress_tells_a_rank_when_its_collective_has_been_launched(dev, stream):
+    """A collective is launched by the last rank that posts it; until then the
+    earlier ranks' calls have only been accepted."""
+    n, count = 3, 1000
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        bufs = [b.put(np.full(count, r + 1, np.float32)) for r in range(n)]
+        assert g.progress(0) == (0, 0)
+        for turn in range(2):
+            for r in range(n):
+                N.check(N.lib.flagcxAllReduce(bufs[r], bufs[r], count, N.DT_FP32, N.OP_SUM, g.comms[r], stream), "flagcxAllReduce")
+                joined, launched = g.progress(r)
+                assert joined == turn and launched == turn + (r == n - 1)
+            assert [g.progress(r) for r in range(n)] == [(turn, turn + 1)] * n
+        dev.stream_sync(stream)
+        assert (dev.to_host(bufs[0], count, np.float32) == 6 * 3).all()

@@ -172,6 +172,45 @@ def simulated(n, gen):
     wait_all([b.barrier() for b in ranks])
     print("ok  gather, scatter, send / recv, barrier", flush=True)
 
+    # coalesced forms: one collective over all the tensors of the call, so that rank after rank can post them
+    shapes = [(1001,), (3, 333), (70001,), (16,)]
+    tl = [[make(torch.float32, sh, gen) for sh in shapes] for _ in range(n)]
+    want = [O.reduce_copy([words(tl[r][i]).ravel() for r in range(n)], N.DT_FP32, N.OP_SUM) for i in range(len(shapes))]
+    wait_all([b.allreduce_coalesced(ts) for b, ts in zip(ranks, tl)])
+    for r in range(n):
+        for i in range(len(shapes)):
+            same(words(tl[r][i]).ravel(), want[i], f"allreduce_coalesced rank {r} tensor {i}")
+    ext = fxb.extension()
+    il = [[make(torch.bfloat16, sh, gen) for sh in shapes] for _ in range(n)]
+    ol = [[torch.empty((n,) + sh, device="cuda", dtype=torch.bfloat16) for sh in shapes] for _ in range(n)]
+    wait_all([ext.allgather_into_tensor_coalesced(b, ol[r], il[r]) for r, b in enumerate(ranks)])
+    for r in range(n):
+        for i in range(len(shapes)):
+            assert torch.equal(ol[r][i], torch.stack([il[q][i] for q in range(n)])), f"allgather coalesced rank {r} tensor {i}"
+    il = [[make(torch.float32, (n,) + sh, gen) for sh in shapes] for _ in range(n)]
+    ol = [[torch.empty(sh, device="cuda") for sh in shapes] for _ in range(n)]
+    wait_all([ext.reduce_scatter_tensor_coalesced(b, ol[r], il[r], ReduceOp.SUM) for r, b in enumerate(ranks)])
+    for i in range(len(shapes)):
+        want = O.reduce_copy([words(il[q][i]).ravel() for q in range(n)], N.DT_FP32, N.OP_SUM)
+        per = want.size // n
+        for r in range(n):
+            same(words(ol[r][i]).ravel(), want[r * per:(r + 1) * per], f"reduce_scatter coalesced rank {r} tensor {i}")
+    print("ok  coalesced all-reduce, all-gather, reduce-scatter", flush=True)
+
+    # a Work that is dropped without a wait still fills its output list, and an input dropped right after the call
+    # is still read
+    ins = [make(torch.int32, (4001,), gen) for _ in range(n)]
+    keep = [t.clone() for t in ins]
+    lists = [[torch.zeros(4001, device="cuda", dtype=torch.int32) for _ in range(n)] for _ in range(n)]
+    for r, b in enumerate(ranks):
+        b.allgather([lists[r]], [ins[r]])
+    del ins
+    junk = [torch.full((4001,), -7, device="cuda", dtype=torch.int32) for _ in range(4 * n)]    # would reuse freed blocks
+    torch.cuda.synchronize()
+    assert all(torch.equal(lists[r][q], keep[q]) for r in range(n) for q in range(n)), "dropped Work / dropped input"
+    del junk
+    print("ok  dropped Work, dropped input", flush=True)
+
     # what the backend refuses
     o = dist.AllreduceOptions()
     o.reduceOp = ReduceOp.BAND

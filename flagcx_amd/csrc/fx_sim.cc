@@ -54,7 +54,6 @@ struct PendingP2p {
   void *rbuf;
   size_t bytes;
   hipStream_t stream;
-  hipEvent_t posted;       // recorded on `stream` when the call was made
   uint64_t id;             // names this half for a sleeping poster (rendezvous mode)
 };
 
@@ -66,6 +65,7 @@ struct Group {
   int joined = 0, alive = 0;
   std::vector<char> taken;  // ranks that have joined
   std::vector<PendingP2p> p2p;
+  hipEvent_t p2pBefore = nullptr, p2pAfter = nullptr;   // made at the first pair whose halves sit on two streams
   uint64_t nextP2pId = 1;
   std::map<uint64_t, flagcxResult_t> p2pMatched;  // rendezvous mode: results awaiting their sleeping poster
   // pending collective
@@ -988,7 +988,8 @@ void freeGroupResources(Group *g) {
   for (auto e : g->ready)
     if (e) (void)hipEventDestroy(e);
   if (g->done) (void)hipEventDestroy(g->done);
-  for (auto &p : g->p2p) (void)hipEventDestroy(p.posted);
+  if (g->p2pBefore) (void)hipEventDestroy(g->p2pBefore);
+  if (g->p2pAfter) (void)hipEventDestroy(g->p2pAfter);
   if (g->scratch) (void)hipFree(g->scratch);
   for (void *b : g->outgrown) (void)hipFree(b);
   delete g;
@@ -1056,6 +1057,28 @@ struct DeferredP2p {
 thread_local int tGroupDepth = 0;
 thread_local std::vector<DeferredP2p> tDeferred;
 
+// Copies of pairs that were matched inside a bracket with both halves on one
+// stream (ranks posted one after another by one thread): they leave as one
+// launch per stream when the outermost bracket closes, which is where the
+// reference issues grouped operations too.  Not in rendezvous mode, where the
+// other half's thread is told "done" at the match and may enqueue behind it.
+struct BatchedCopies {
+  hipStream_t stream;
+  std::vector<fxSliceDesc> copies;
+};
+thread_local std::vector<BatchedCopies> tBatched;
+
+flagcxResult_t flushBatched() {
+  std::vector<BatchedCopies> mine;
+  mine.swap(tBatched);
+  flagcxResult_t first = flagcxSuccess;
+  for (BatchedCopies &b : mine) {
+    const flagcxResult_t rc = R(fx_copy_slices(b.copies.data(), b.copies.size(), b.stream));
+    if (first == flagcxSuccess) first = rc;
+  }
+  return first;
+}
+
 // Wait until the partner of pending half `id` has made its call (it enqueues the
 // copy and makes our stream wait for it) and hand back its result; on time-out
 // the half is withdrawn.  Called with g->mu held.
@@ -1065,7 +1088,6 @@ flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64
   if (!matched) {  // the partner never came: withdraw this half
     for (size_t i = 0; i < g->p2p.size(); i++)
       if (g->p2p[i].id == id) {
-        (void)hipEventDestroy(g->p2p[i].posted);
         g->p2p.erase(g->p2p.begin() + (long)i);
         break;
       }
@@ -1077,8 +1099,11 @@ flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64
 }
 
 // send / recv between simulated ranks: the later of the two calls performs the
-// copy on its own stream after waiting for the other side's stream, and the
-// other side's stream then waits for the copy.
+// copy on its own stream.  If the other side posted on another stream, the copy
+// first waits for all that stream holds at that moment (as a collective's
+// launch waits for the other ranks' streams: later than the post itself, which
+// is safe -- a stream can only be waiting for events recorded before this call)
+// and that stream then waits for the copy.
 flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, void *rbuf, size_t count, int dtype,
                            int peer, flagcxStream_t stream);
 
@@ -1106,14 +1131,24 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
     } else if (bytes) {
       hipStream_t s = stream->base;
       fxSliceDesc d = copyDesc(isSend ? sbuf : o.sbuf, isSend ? o.rbuf : rbuf, bytes);
-      if (o.stream != s && hipStreamWaitEvent(s, o.posted, 0) != hipSuccess) res = flagcxUnhandledDeviceError;
-      if (res == flagcxSuccess) res = R(fx_copy_slices(&d, 1, s));
-      if (res == flagcxSuccess && o.stream != s) {
-        if (hipEventRecord(o.posted, s) != hipSuccess || hipStreamWaitEvent(o.stream, o.posted, 0) != hipSuccess)
+      if (o.stream == s && tGroupDepth > 0 && g->sync != FX_SYNC_RENDEZVOUS) {
+        size_t b = 0;
+        while (b < tBatched.size() && tBatched[b].stream != s) b++;
+        if (b == tBatched.size()) tBatched.push_back(BatchedCopies{s, {}});
+        tBatched[b].copies.push_back(d);
+      } else if (o.stream == s) {
+        res = R(fx_copy_slices(&d, 1, s));
+      } else {
+        if ((!g->p2pBefore && hipEventCreateWithFlags(&g->p2pBefore, hipEventDisableTiming) != hipSuccess) ||
+            (!g->p2pAfter && hipEventCreateWithFlags(&g->p2pAfter, hipEventDisableTiming) != hipSuccess) ||
+            hipEventRecord(g->p2pBefore, o.stream) != hipSuccess || hipStreamWaitEvent(s, g->p2pBefore, 0) != hipSuccess)
+          res = flagcxUnhandledDeviceError;
+        if (res == flagcxSuccess) res = R(fx_copy_slices(&d, 1, s));
+        if (res == flagcxSuccess &&
+            (hipEventRecord(g->p2pAfter, s) != hipSuccess || hipStreamWaitEvent(o.stream, g->p2pAfter, 0) != hipSuccess))
           res = flagcxUnhandledDeviceError;
       }
     }
-    (void)hipEventDestroy(o.posted);
     if (g->sync == FX_SYNC_RENDEZVOUS) {
       g->p2pMatched[o.id] = res;
       g->cv.notify_all();
@@ -1121,20 +1156,15 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
     g->p2p.erase(g->p2p.begin() + (long)i);
     return res;
   }
-  PendingP2p p{isSend, src, dst, sbuf, rbuf, bytes, stream->base, nullptr, g->nextP2pId++};
-  if (hipEventCreateWithFlags(&p.posted, hipEventDisableTiming) != hipSuccess) return flagcxUnhandledDeviceError;
-  if (hipEventRecord(p.posted, p.stream) != hipSuccess) {
-    (void)hipEventDestroy(p.posted);
-    return flagcxUnhandledDeviceError;
-  }
-  g->p2p.push_back(p);
+  g->p2p.push_back(PendingP2p{isSend, src, dst, sbuf, rbuf, bytes, stream->base, g->nextP2pId++});
   if (g->sync != FX_SYNC_RENDEZVOUS) return flagcxSuccess;
+  const uint64_t id = g->p2p.back().id;
   if (tGroupDepth > 0) {  // inside a bracket: the wait happens when the bracket closes
-    tDeferred.push_back(DeferredP2p{g, p.id});
+    tDeferred.push_back(DeferredP2p{g, id});
     return flagcxSuccess;
   }
   // Sleep until the partner has made its call and enqueued the copy.
-  return awaitPartner(g, lock, p.id);
+  return awaitPartner(g, lock, id);
 }
 
 }  // namespace
@@ -1425,7 +1455,7 @@ flagcxResult_t flagcxGroupEnd(flagcxComm_t) {
   if (tGroupDepth == 0) return flagcxInvalidUsage;  // no bracket open on this thread
   if (--tGroupDepth > 0) return flagcxSuccess;
   return R(fx::guarded([&]() -> int {
-    flagcxResult_t first = flagcxSuccess;
+    flagcxResult_t first = flushBatched();
     std::vector<DeferredP2p> mine;
     mine.swap(tDeferred);
     for (const DeferredP2p &d : mine) {

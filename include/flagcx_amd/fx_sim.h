@@ -22,7 +22,11 @@
  *     Like the calls of one ncclGroupStart/End bracket, a collective is ordered
  *     after work a rank enqueued BEFORE the last rank posted and before work
  *     enqueued AFTER it: a single host thread that loops over the ranks, on one
- *     stream or several, needs nothing else.
+ *     stream or several, needs nothing else.  flagcxSend / flagcxRecv pairs that
+ *     meet inside a flagcxGroupStart / flagcxGroupEnd bracket of that thread,
+ *     both halves on one stream, are enqueued together -- one copy launch per
+ *     stream -- when the thread's outermost bracket closes, and that
+ *     flagcxGroupEnd returns their result.
  *   FX_SYNC_RENDEZVOUS       for one host thread per rank, each on its own
  *     stream, the way separate FlagCX processes behave: a call blocks its host
  *     thread until every rank has posted and the work is enqueued, so whatever

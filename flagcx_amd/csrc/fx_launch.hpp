@@ -189,7 +189,9 @@ flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const 
   a.count = count;
   a.k = k;
   a.nout = nout;
-  const uint64_t ntiles = tilesFor(out[0], in, k, count, R::ES, U, out + 1, nout - 1);
+  if (count == 0) return flagcxSuccess;
+  a.co = coAlignedHost(out[0], in, k, out + 1, nout - 1) ? 1 : 0;
+  const uint64_t ntiles = planTiles((uint64_t)(uintptr_t)out[0], count, R::ES, U, handOutFor(a.co != 0, k)).tiles();
   if (ntiles == 0) return flagcxSuccess;
   if (ntiles > 0x7ffffff0ull) return flagcxInvalidArgument;
   return launchKernel(reduceBcastRuntime<R, U>, (uint32_t)ntiles, s, a);
@@ -201,6 +203,7 @@ flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
   uint64_t total = 0;
   a->tileStart[0] = 0;
   for (int c = 0; c < a->nchunks; c++) {
+    a->co[c] = chunkCoAligned(*a, c) ? 1 : 0;
     total += a->cnt[c] ? chunkPlan<R::ES, U>(*a, c).tiles() : 0;
     if (total > 0x7ffffff0ull) return flagcxInvalidArgument;
     a->tileStart[c + 1] = (uint32_t)total;

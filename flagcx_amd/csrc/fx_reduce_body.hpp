@@ -639,9 +639,23 @@ struct SegMany : Seg<0> {
   int nmore;
   __device__ __forceinline__ char *outp(int o) const { return asGlobal(rawOut[o]) - mis; }
 };
+// The extra outputs four at a time: their pointers come through scalar loads,
+// and four independent ones are fetched together where a loop of single ones
+// would wait for each in turn.
+template <class SG>
+__device__ __forceinline__ void storeToMore(const SG &sg, uint64_t byteOff, u32x4 v) {
+  for (int o = 0; o < sg.nmore; o += 4) {
+    char *q[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) q[i] = sg.outp(o + i < sg.nmore ? o + i : o);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      if (o + i < sg.nmore) stg_stream(q[i] + byteOff, v);
+  }
+}
 __device__ __forceinline__ void storeVector(const SegMany &sg, uint64_t byteOff, u32x4 v) {
   stg_stream(sg.out + byteOff, v);
-  for (int o = 0; o < sg.nmore; o++) stg_stream(sg.outp(o) + byteOff, v);
+  storeToMore(sg, byteOff, v);
 }
 template <int ES>
 __device__ __forceinline__ void storeElems(const SegMany &sg, uint64_t e0, int lo, int hi, u32x4 v) {
@@ -673,7 +687,7 @@ struct SegChunk {
 };
 __device__ __forceinline__ void storeVector(const SegChunk &sg, uint64_t byteOff, u32x4 v) {
   stg_stream(sg.out + byteOff, v);
-  for (int o = 0; o < sg.nmore; o++) stg_stream(sg.outp(o) + byteOff, v);
+  storeToMore(sg, byteOff, v);
 }
 template <int ES>
 __device__ __forceinline__ void storeElems(const SegChunk &sg, uint64_t e0, int lo, int hi, u32x4 v) {
@@ -715,6 +729,11 @@ __device__ __forceinline__ u32x4 ldg_as(const void *p) {
   return TEMPORAL ? ldg_keep(p) : ldg_stream(p);
 }
 
+#ifndef FX_RUNTIME_GROUP
+#define FX_RUNTIME_GROUP 4
+#endif
+constexpr int kRuntimeGroup = FX_RUNTIME_GROUP;   // inputs a lane of a run-time-k kernel keeps in flight
+
 template <class R, int K, int U, bool TEMPORAL, class SG>
 __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, uint64_t ustride) {
   if (K > 0) {
@@ -735,20 +754,20 @@ __device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, ui
     typename R::Acc acc[U];
 #pragma unroll
     for (int u = 0; u < U; u++) R::init(acc[u], ldg_as<TEMPORAL>(sg.inp(0) + off + u * ustride));
-    // four inputs in flight at a time (folded in their order): a lane that waits for
+    // kRuntimeGroup inputs in flight at a time (folded in their order): a lane that waits for
     // every input in turn is what a small launch of many inputs spends its time on
     const int k = sg.inputs();
     int p = 1;
-    for (; p + 4 <= k; p += 4) {
-      u32x4 v[4][U];
+    for (; p + kRuntimeGroup <= k; p += kRuntimeGroup) {
+      u32x4 v[kRuntimeGroup][U];
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
+      for (int q = 0; q < kRuntimeGroup; q++) {
         const char *ip = sg.inp(p + q);
 #pragma unroll
         for (int u = 0; u < U; u++) v[q][u] = ldg_as<TEMPORAL>(ip + off + u * ustride);
       }
 #pragma unroll
-      for (int q = 0; q < 4; q++)
+      for (int q = 0; q < kRuntimeGroup; q++)
 #pragma unroll
         for (int u = 0; u < U; u++) R::fold(acc[u], v[q][u]);
     }
@@ -889,6 +908,7 @@ struct ManyArgs {
   void *out[kMaxK];
   uint64_t count;
   int k, nout;
+  int co;   // every stream sits at out[0]'s offset within a cache line (the host has looked at all k + nout pointers)
 };
 
 // k inputs (rotated by the host) folded once and stored to nout buffers.
@@ -904,10 +924,7 @@ __global__ void __launch_bounds__(kBlock) reduceBcastRuntime(ManyArgs a) {
   sg.k = a.k;
   sg.rawOut = a.out + 1;
   sg.nmore = a.nout - 1;
-  bool co = true;
-  for (int p = 0; p < a.k; p++) co = co && sameLinePhase((uint64_t)(uintptr_t)a.in[p], (uint64_t)(uintptr_t)a.out[0]);
-  for (int o = 1; o < a.nout; o++) co = co && sameLinePhase((uint64_t)(uintptr_t)a.out[o], (uint64_t)(uintptr_t)a.out[0]);
-  const TilePlan tp = planTiles((uint64_t)(uintptr_t)a.out[0], a.count, R::ES, U, handOutFor(co, a.k));
+  const TilePlan tp = planTiles((uint64_t)(uintptr_t)a.out[0], a.count, R::ES, U, handOutFor(a.co != 0, a.k));
   reduceTile<R, 0, U>(sg, tp, blockIdx.x, 0u);
 }
 
@@ -923,11 +940,13 @@ struct ChunkedArgs {
   int8_t first[kMaxK];                    // fold order starts at this input
   int8_t only[kMaxK];                     // >= 0: this input alone
   int8_t outSel[kMaxK];                   // >= 0: this output alone; -1: all nout
+  int8_t co[kMaxK];                       // chunkCoAligned of the chunk, worked out once on the host
   int k, nout, nchunks;
 };
 
 // Whether every stream of a chunk sits at the primary output's offset within a
-// cache line; shared by the kernel and by the host's tile count.
+// cache line.  The host works it out (it reads up to k + nout pointers) and
+// leaves it in co[c] for the kernel.
 __host__ __device__ inline bool chunkCoAligned(const ChunkedArgs &a, int c) {
   const int primary = a.outSel[c] >= 0 ? a.outSel[c] : 0;
   const uint64_t o = (uint64_t)(uintptr_t)a.out[primary] + a.outOff[c];
@@ -945,7 +964,7 @@ template <int ES, int U>
 __host__ __device__ inline TilePlan chunkPlan(const ChunkedArgs &a, int c) {
   const int primary = a.outSel[c] >= 0 ? a.outSel[c] : 0;
   return planTiles((uint64_t)(uintptr_t)a.out[primary] + a.outOff[c], a.cnt[c], ES, U,
-                   handOutFor(chunkCoAligned(a, c), a.only[c] >= 0 ? 1 : a.k));
+                   handOutFor(a.co[c] != 0, a.only[c] >= 0 ? 1 : a.k));
 }
 
 template <class R, int U>

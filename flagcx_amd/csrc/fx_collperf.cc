@@ -11,7 +11,7 @@
 // test/perf/host_api/test_*.cpp), so a sweep made with those programs and a
 // sweep made here can be laid side by side.  Added here: -N ranks (default 8),
 // -A direct|ring, -O rank|ring|host, -c 1 to check every rank's result after the
-// timed loop, and a second figure per line: the bytes the GPU's memory moved
+// timed loop (long results by sample), and a second figure per line: the bytes the GPU's memory moved
 // for one collective, divided by the time between two device events around
 // the timed calls.
 //
@@ -138,8 +138,13 @@ double decode(const void *src, size_t i, flagcxDataType_t t) {
   }
 }
 
+enum Coll { kAllReduce, kReduce, kReduceScatter, kAllGather, kBroadcast, kGather, kScatter, kAlltoAll, kAlltoAllv, kSendRecv, kUnknown };
+const char *kCollNames[] = {"allreduce", "reduce", "reducescatter", "allgather", "broadcast", "gather", "scatter", "alltoall",
+                            "alltoallv", "sendrecv"};
+
 struct Options {
   std::string coll;
+  Coll kind = kUnknown;
   size_t minBytes = 1ull << 20, maxBytes = 1ull << 30;
   int factor = 2, warmup = 5, iters = 20, root = 0, nranks = 8, check = 0;
   int type = 7 /* float */, op = 0;
@@ -161,6 +166,13 @@ Options parse(int argc, char **argv) {
     exit(argc < 2 ? 1 : 0);
   }
   o.coll = argv[1];
+  for (int i = 0; i < (int)kUnknown; i++)
+    if (o.coll == kCollNames[i]) o.kind = (Coll)i;
+  if (o.kind == kUnknown) {
+    fprintf(stderr, "fx_collperf: unknown collective '%s'\n", o.coll.c_str());
+    usage(argv[0]);
+    exit(1);
+  }
   static option longOpts[] = {{"minbytes", required_argument, 0, 'b'}, {"maxbytes", required_argument, 0, 'e'},
                               {"stepfactor", required_argument, 0, 'f'}, {"warmup_iters", required_argument, 0, 'w'},
                               {"iters", required_argument, 0, 'n'}, {"root", required_argument, 0, 'r'},
@@ -232,40 +244,40 @@ struct Run {
 
   Shape shape(size_t count) const {
     const double N = n, sz = (double)count * t.size, part = (double)(count / n) * t.size;
-    const std::string &c = o.coll;
-    if (c == "allreduce") return {count, count, 2 * (N - 1) / N, 2 * N * sz};
-    if (c == "reduce") return {count, count, 1, (N + 1) * sz};
-    if (c == "reducescatter") return {count, count / n, (N - 1) / N, (N * N + N) * part};
-    if (c == "allgather") return {count / n, count, (N - 1) / N, (N + N * N) * part};
-    if (c == "broadcast") return {count, count, 1, (1 + N) * sz};
-    if (c == "gather") return {count / n, count, (N - 1) / N, 2 * N * part};
-    if (c == "scatter") return {count, count / n, (N - 1) / N, 2 * N * part};
-    if (c == "alltoall") return {count, count, (N - 1) / N, 2 * N * N * part};
-    if (c == "alltoallv") {   // slots of two blocks for every rank of one's own parity (see layoutV)
-      double moved = 0;
-      for (size_t v : sc) moved += (double)v * t.size;
-      return {count + 2 * (count / n), count + 2 * (count / n), (N - 1) / N, 2 * moved};
+    switch (o.kind) {
+      case kAllReduce: return {count, count, 2 * (N - 1) / N, 2 * N * sz};
+      case kReduce: return {count, count, 1, (N + 1) * sz};
+      case kReduceScatter: return {count, count / n, (N - 1) / N, (N * N + N) * part};
+      case kAllGather: return {count / n, count, (N - 1) / N, (N + N * N) * part};
+      case kBroadcast: return {count, count, 1, (1 + N) * sz};
+      case kGather: return {count / n, count, (N - 1) / N, 2 * N * part};
+      case kScatter: return {count, count / n, (N - 1) / N, 2 * N * part};
+      case kAlltoAll: return {count, count, (N - 1) / N, 2 * N * N * part};
+      case kAlltoAllv: {   // slots of two blocks for every rank of one's own parity (see layoutV)
+        double moved = 0;
+        for (size_t v : sc) moved += (double)v * t.size;
+        return {count + 2 * (count / n), count + 2 * (count / n), (N - 1) / N, 2 * moved};
+      }
+      default: return {count, count, 1, 2 * N * sz};   // sendrecv
     }
-    if (c == "sendrecv") return {count, count, 1, 2 * N * sz};
-    fprintf(stderr, "fx_collperf: unknown collective '%s'\n", c.c_str());
-    exit(1);
   }
 
   int post(int r, size_t count) {
-    const std::string &c = o.coll;
     const flagcxRedOp_t op = (flagcxRedOp_t)o.op;
-    if (c == "allreduce") return flagcxAllReduce(send[r], recv[r], count, t.code, op, comms[r], stream);
-    if (c == "reduce") return flagcxReduce(send[r], recv[r], count, t.code, op, o.root, comms[r], stream);
-    if (c == "reducescatter") return flagcxReduceScatter(send[r], recv[r], count / n, t.code, op, comms[r], stream);
-    if (c == "allgather") return flagcxAllGather(send[r], recv[r], count / n, t.code, comms[r], stream);
-    if (c == "broadcast") return flagcxBroadcast(send[r], recv[r], count, t.code, o.root, comms[r], stream);
-    if (c == "gather") return flagcxGather(send[r], recv[r], count / n, t.code, o.root, comms[r], stream);
-    if (c == "scatter") return flagcxScatter(send[r], recv[r], count / n, t.code, o.root, comms[r], stream);
-    if (c == "alltoall") return flagcxAlltoAll(send[r], recv[r], count / n, t.code, comms[r], stream);
-    if (c == "alltoallv")
-      return flagcxAlltoAllv(send[r], &sc[(size_t)r * n], &sd[(size_t)r * n], recv[r], &rc[(size_t)r * n], &rd[(size_t)r * n],
-                             t.code, comms[r], stream);
-    return flagcxInvalidArgument;
+    switch (o.kind) {
+      case kAllReduce: return flagcxAllReduce(send[r], recv[r], count, t.code, op, comms[r], stream);
+      case kReduce: return flagcxReduce(send[r], recv[r], count, t.code, op, o.root, comms[r], stream);
+      case kReduceScatter: return flagcxReduceScatter(send[r], recv[r], count / n, t.code, op, comms[r], stream);
+      case kAllGather: return flagcxAllGather(send[r], recv[r], count / n, t.code, comms[r], stream);
+      case kBroadcast: return flagcxBroadcast(send[r], recv[r], count, t.code, o.root, comms[r], stream);
+      case kGather: return flagcxGather(send[r], recv[r], count / n, t.code, o.root, comms[r], stream);
+      case kScatter: return flagcxScatter(send[r], recv[r], count / n, t.code, o.root, comms[r], stream);
+      case kAlltoAll: return flagcxAlltoAll(send[r], recv[r], count / n, t.code, comms[r], stream);
+      case kAlltoAllv:
+        return flagcxAlltoAllv(send[r], &sc[(size_t)r * n], &sd[(size_t)r * n], recv[r], &rc[(size_t)r * n], &rd[(size_t)r * n],
+                               t.code, comms[r], stream);
+      default: return flagcxInvalidArgument;
+    }
   }
 
   // every rank sends to the next and receives from the previous, inside one bracket per rank
@@ -279,7 +291,7 @@ struct Run {
   }
 
   void once(size_t count) {
-    if (o.coll == "sendrecv") return sendrecvOnce(count);
+    if (o.kind == kSendRecv) return sendrecvOnce(count);
     for (int r = 0; r < n; r++) {
       const int rc_ = post(r, count);
       if (rc_ != flagcxSuccess) die(o.coll.c_str(), rc_);
@@ -306,11 +318,11 @@ struct Run {
   }
 
   double expected(int r, size_t i, size_t count, bool *defined) const {
-    const std::string &c = o.coll;
     const size_t part = count / n;
+    const Coll c = o.kind;
     *defined = true;
     // the n parts of count / n elements may not fill the whole size
-    if ((c == "allgather" || c == "gather" || c == "alltoall") && (part == 0 || i >= part * (size_t)n)) return (*defined = false, 0.0);
+    if ((c == kAllGather || c == kGather || c == kAlltoAll) && (part == 0 || i >= part * (size_t)n)) return (*defined = false, 0.0);
     auto fold = [&](size_t at) {
       double acc = valueAt(at, 0);
       for (int q = 1; q < n; q++) {
@@ -319,27 +331,28 @@ struct Run {
       }
       return acc;
     };
-    if (c == "allreduce") return fold(i);
-    if (c == "reduce") return r == o.root ? fold(i) : (*defined = false, 0.0);
-    if (c == "reducescatter") return fold((size_t)r * part + i);
-    if (c == "allgather") return valueAt(i % part, (int)(i / part));
-    if (c == "broadcast") return valueAt(i, o.root);
-    if (c == "gather") return r == o.root ? valueAt(i % part, (int)(i / part)) : (*defined = false, 0.0);
-    if (c == "scatter") return valueAt((size_t)r * part + i, o.root);
-    if (c == "alltoall") return valueAt((size_t)r * part + i % part, (int)(i / part));
-    if (c == "alltoallv") {   // slot q of rank r holds what the q-th rank of r's parity sent from its slot for r
-      const size_t two = 2 * part;
-      const int from = two ? (r & 1) + 2 * (int)(i / two) : n;
-      if (from >= n || from == r) return (*defined = false, 0.0);
-      return valueAt(sd[(size_t)from * n + r] + i % two, from);
+    switch (c) {
+      case kAllReduce: return fold(i);
+      case kReduce: return r == o.root ? fold(i) : (*defined = false, 0.0);
+      case kReduceScatter: return fold((size_t)r * part + i);
+      case kAllGather: return valueAt(i % part, (int)(i / part));
+      case kBroadcast: return valueAt(i, o.root);
+      case kGather: return r == o.root ? valueAt(i % part, (int)(i / part)) : (*defined = false, 0.0);
+      case kScatter: return valueAt((size_t)r * part + i, o.root);
+      case kAlltoAll: return valueAt((size_t)r * part + i % part, (int)(i / part));
+      case kAlltoAllv: {   // slot q of rank r holds what the q-th rank of r's parity sent from its slot for r
+        const size_t two = 2 * part;
+        const int from = two ? (r & 1) + 2 * (int)(i / two) : n;
+        if (from >= n || from == r) return (*defined = false, 0.0);
+        return valueAt(sd[(size_t)from * n + r] + i % two, from);
+      }
+      case kSendRecv: return valueAt(i, (r + n - 1) % n);
+      default: return (*defined = false, 0.0);
     }
-    if (c == "sendrecv") return valueAt(i, (r + n - 1) % n);
-    *defined = false;
-    return 0;
   }
 };
 
-bool reduces(const std::string &c) { return c == "allreduce" || c == "reduce" || c == "reducescatter"; }
+bool reduces(Coll c) { return c == kAllReduce || c == kReduce || c == kReduceScatter; }
 
 double seconds() {
   return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -353,7 +366,6 @@ int main(int argc, char **argv) {
   run.t = kTypes[run.o.type];
   run.n = run.o.nranks;
   const int n = run.n;
-  (void)run.shape(0);   // refuses an unknown collective before anything is set up
   loadAdaptor();
   OK(dev->setDevice(0));
   run.comms.resize(n);
@@ -366,7 +378,7 @@ int main(int argc, char **argv) {
   OK(dev->eventCreate(&t1, flagcxEventDefault));
 
   const size_t maxCount = run.o.maxBytes / run.t.size;
-  if (run.o.coll == "alltoallv") run.layoutV(maxCount);
+  if (run.o.kind == kAlltoAllv) run.layoutV(maxCount);
   const Shape big = run.shape(maxCount);
   run.send.resize(n);
   run.recv.resize(n);
@@ -377,7 +389,7 @@ int main(int argc, char **argv) {
   std::vector<char> host(std::max<size_t>(std::max(big.sendElems, big.recvElems), 1) * run.t.size);
 
   const bool exactType = run.t.size >= 4;
-  const bool checkable = run.o.check && (!reduces(run.o.coll) || (exactType && run.o.op != flagcxProd && run.o.op != flagcxAvg));
+  const bool checkable = run.o.check && (!reduces(run.o.kind) || (exactType && run.o.op != flagcxProd && run.o.op != flagcxAvg));
   printf("# %s over %d simulated ranks on one GPU; buffers and stream from the %s device adaptor\n", run.o.coll.c_str(), n,
          dev->name);
   printf("#\n# datatype: %s, op: %s\n#\n", run.t.name, kOps[run.o.op]);
@@ -387,7 +399,7 @@ int main(int argc, char **argv) {
   int failures = 0;
   for (size_t size = run.o.minBytes; size <= run.o.maxBytes; size *= (size_t)run.o.factor) {
     const size_t count = size / run.t.size;
-    if (run.o.coll == "alltoallv") run.layoutV(count);
+    if (run.o.kind == kAlltoAllv) run.layoutV(count);
     const Shape sh = run.shape(count);
     for (int r = 0; r < n; r++) {
       for (size_t i = 0; i < sh.sendElems; i++) encode(host.data(), i, valueAt(i, r), run.t.code);
@@ -419,7 +431,9 @@ int main(int argc, char **argv) {
         if (!sh.recvElems) continue;
         OK(dev->deviceMemcpy(host.data(), run.recv[r], sh.recvElems * run.t.size, flagcxMemcpyDeviceToHost, nullptr, nullptr));
         std::vector<char> want(run.t.size);
-        for (size_t i = 0; i < sh.recvElems; i++) {
+        // every element up to 4 Mi of them; of longer results the first and last 64 Ki and every 4099th between
+        const size_t edge = 65536, all = sh.recvElems <= (4u << 20) ? sh.recvElems : 0;
+        for (size_t i = 0; i < sh.recvElems; i += (all || i < edge || i + edge >= sh.recvElems) ? 1 : std::min<size_t>(4099, sh.recvElems - edge - i)) {
           bool defined;
           const double v = run.expected(r, i, count, &defined);
           if (!defined) continue;

@@ -135,6 +135,25 @@ _SIGS.update({
     "flagcxGroupStart": (_i, [_vp]),
     "flagcxGroupEnd": (_i, [_vp]),
     "flagcxCommCount": (_i, [_vp, C.POINTER(_i)]),
+    # fx_handle.h: what an application calls around the collectives
+    "flagcxDeviceHandleInit": (_i, [C.POINTER(_vp)]),
+    "flagcxDeviceHandleFree": (_i, [_vp]),
+    "flagcxHandleInit": (_i, [C.POINTER(_vp)]),
+    "flagcxHandleFree": (_i, [_vp]),
+    "flagcxMemAlloc": (_i, [C.POINTER(_vp), _sz, _i]),
+    "flagcxMemFree": (_i, [_vp, _i]),
+    "flagcxCommRegister": (_i, [_vp, _vp, _sz, C.POINTER(_vp), _i]),
+    "flagcxCommDeregister": (_i, [_vp, _vp, _i]),
+    "flagcxCommWindowRegister": (_i, [_vp, _vp, _sz, C.POINTER(_vp), _i, _i]),
+    "flagcxCommWindowDeregister": (_i, [_vp, _vp, _i]),
+    "flagcxIsHomoComm": (_i, [_vp, C.POINTER(_i)]),
+    "flagcxCommFinalize": (_i, [_vp]),
+    "flagcxCommAbort": (_i, [_vp]),
+    "flagcxCommResume": (_i, [_vp]),
+    "flagcxCommSuspend": (_i, [_vp]),
+    "flagcxGetLastError": (C.c_char_p, [_vp]),
+    "flagcxCommGetAsyncError": (_i, [_vp, C.POINTER(_i)]),
+    "flagcxCommGetDeviceNumber": (_i, [_vp, C.POINTER(_i)]),
     "flagcxCommUserRank": (_i, [_vp, C.POINTER(_i)]),
     "flagcxReduce": (_i, [_vp, _vp, _sz, _i, _i, _i, _vp, _vp]),
     "flagcxAllReduce": (_i, [_vp, _vp, _sz, _i, _i, _vp, _vp]),

@@ -17,8 +17,8 @@
 //
 // One host thread posts rank after rank on one stream, as a test program with
 // one process per rank would, minus the processes.  Host code only: buffers,
-// streams and events come from the device-adaptor plugin next to this program.
-#include <dlfcn.h>
+// streams and events come through flagcxDeviceHandleInit's table, as in the
+// reference's tests (test/perf_common.cc:27-60).
 #include <getopt.h>
 #include <unistd.h>
 
@@ -32,12 +32,12 @@
 #include <string>
 #include <vector>
 
-#include "flagcx_amd/fx_device_adaptor.h"
+#include "flagcx_amd/fx_handle.h"
 #include "flagcx_amd/fx_sim.h"
 
 namespace {
 
-const flagcxDeviceAdaptor_v1 *dev = nullptr;
+flagcxDeviceHandle_t dev = nullptr;   // flagcxDeviceHandleInit: the device operations an application may call
 
 [[noreturn]] void die(const char *what, int rc) {
   fprintf(stderr, "fx_collperf: %s failed: %s (%d)\n", what, flagcxGetErrorString((flagcxResult_t)rc), rc);
@@ -48,24 +48,6 @@ const flagcxDeviceAdaptor_v1 *dev = nullptr;
     const int rc_ = (int)(call);              \
     if (rc_ != flagcxSuccess) die(#call, rc_); \
   } while (0)
-
-void loadAdaptor() {
-  Dl_info me;
-  if (!dladdr((const void *)&flagcxAllReduce, &me) || !me.dli_fname) {
-    fprintf(stderr, "fx_collperf: cannot locate libflagcx_amd.so\n");
-    exit(1);
-  }
-  std::string path(me.dli_fname);
-  path.erase(path.find_last_of('/') + 1);
-  path += "libflagcx-device-mi355x.so";
-  void *h = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
-  void *sym = h ? dlsym(h, FX_DEVICE_ADAPTOR_SYMBOL) : nullptr;
-  if (!sym) {
-    fprintf(stderr, "fx_collperf: cannot load the device adaptor %s: %s\n", path.c_str(), dlerror());
-    exit(1);
-  }
-  dev = (const flagcxDeviceAdaptor_v1 *)sym;
-}
 
 struct TypeInfo {
   const char *name;
@@ -366,7 +348,7 @@ int main(int argc, char **argv) {
   run.t = kTypes[run.o.type];
   run.n = run.o.nranks;
   const int n = run.n;
-  loadAdaptor();
+  OK(flagcxDeviceHandleInit(&dev));
   OK(dev->setDevice(0));
   run.comms.resize(n);
   OK(fxSimCommInitAll(run.comms.data(), n));
@@ -390,8 +372,10 @@ int main(int argc, char **argv) {
 
   const bool exactType = run.t.size >= 4;
   const bool checkable = run.o.check && (!reduces(run.o.kind) || (exactType && run.o.op != flagcxProd && run.o.op != flagcxAvg));
-  printf("# %s over %d simulated ranks on one GPU; buffers and stream from the %s device adaptor\n", run.o.coll.c_str(), n,
-         dev->name);
+  char vendor[128] = "";
+  OK(dev->getVendor(vendor));
+  printf("# %s over %d simulated ranks on one GPU; buffers, stream and events through the device handle (%s)\n",
+         run.o.coll.c_str(), n, vendor);
   printf("#\n# datatype: %s, op: %s\n#\n", run.t.name, kOps[run.o.op]);
   if (run.o.check && !checkable)
     printf("# no check for this datatype / op: the pattern's sums are exact only in 4- and 8-byte types\n");
@@ -404,7 +388,7 @@ int main(int argc, char **argv) {
     for (int r = 0; r < n; r++) {
       for (size_t i = 0; i < sh.sendElems; i++) encode(host.data(), i, valueAt(i, r), run.t.code);
       if (sh.sendElems)
-        OK(dev->deviceMemcpy(run.send[r], host.data(), sh.sendElems * run.t.size, flagcxMemcpyHostToDevice, nullptr, nullptr));
+        OK(dev->deviceMemcpy(run.send[r], host.data(), sh.sendElems * run.t.size, flagcxMemcpyHostToDevice, nullptr));
       if (sh.recvElems) OK(dev->deviceMemset(run.recv[r], 0xff, sh.recvElems * run.t.size, flagcxMemDevice, nullptr));
     }
     OK(dev->deviceSynchronize());
@@ -429,7 +413,7 @@ int main(int argc, char **argv) {
     if (checkable) {
       for (int r = 0; r < n && failures < 10; r++) {
         if (!sh.recvElems) continue;
-        OK(dev->deviceMemcpy(host.data(), run.recv[r], sh.recvElems * run.t.size, flagcxMemcpyDeviceToHost, nullptr, nullptr));
+        OK(dev->deviceMemcpy(host.data(), run.recv[r], sh.recvElems * run.t.size, flagcxMemcpyDeviceToHost, nullptr));
         std::vector<char> want(run.t.size);
         // every element up to 4 Mi of them; of longer results the first and last 64 Ki and every 4099th between
         const size_t edge = 65536, all = sh.recvElems <= (4u << 20) ? sh.recvElems : 0;
@@ -464,5 +448,6 @@ int main(int argc, char **argv) {
   OK(dev->eventDestroy(t1));
   OK(dev->streamDestroy(run.stream));
   OK(fxSimCommDestroyAll(run.comms.data(), n));
+  OK(flagcxDeviceHandleFree(dev));
   return failures ? 2 : 0;
 }

@@ -311,6 +311,9 @@ def test_headers_are_plain_c_and_a_c_client_links(tmp_path):
 #include "flagcx_amd/fx_synth.h"
 #include "flagcx_amd/fx_device_adaptor.h"
 #include "flagcx_amd/fx_ccl_adaptor.h"
+#include "flagcx_amd/fx_host_staged.h"
+#include "flagcx_amd/fx_handle.h"
+_Static_assert(sizeof(struct flagcxDeviceHandle) == 28 * sizeof(void *), "device handle: 28 operations (flagcx.h:143-185)");
 _Static_assert(sizeof(fxReduceTrigger) == 32, "trigger is 32 bytes");
 _Static_assert(sizeof(struct flagcxDeviceAdaptor_v1) == 32 + 48 * sizeof(void *), "v1 device adaptor layout");
 _Static_assert(sizeof(struct flagcxCCLAdaptor_v1) == 35 * sizeof(void *), "v1 ccl adaptor layout");
@@ -332,6 +335,22 @@ int main(void) {
   if (flagcxGetVersion(&version) != flagcxSuccess || version != FX_SIM_VERSION) return 6;
   if (flagcxGetUniqueId(&a) != flagcxSuccess || flagcxGetUniqueId(&b) != flagcxSuccess) return 7;
   if (!memcmp(&a, &b, sizeof(a))) return 8;
+  /* housekeeping calls that need no GPU: argument screening and the fixed answers */
+  {
+    void *p = NULL, *h = NULL;
+    flagcxWindow_t w;
+    if (flagcxMemAlloc(NULL, 16, flagcxMemCCL) != flagcxInvalidArgument) return 9;
+    if (flagcxMemAlloc(&p, 0, flagcxMemCCL) != flagcxInvalidArgument) return 10;
+    if (flagcxMemAlloc(&p, 16, flagcxMemSHMEM) != flagcxInternalError) return 11;
+    if (flagcxMemFree(NULL, flagcxMemCCL) != flagcxSuccess) return 12;
+    if (flagcxCommRegister(NULL, NULL, 16, &h, flagcxMemCCL) != flagcxInvalidArgument) return 13;
+    if (flagcxCommRegister(NULL, &a, 16, &h, flagcxMemCCL) != flagcxSuccess || h != (void *)&a) return 14;
+    if (flagcxCommDeregister(NULL, NULL, flagcxMemCCL) != flagcxSuccess) return 15;
+    if (flagcxCommWindowRegister(NULL, &a, 16, &w, FLAGCX_WIN_COLL_SYMMETRIC, flagcxMemCCL) != flagcxNotSupported) return 16;
+    if (flagcxCommSuspend(NULL) != flagcxInvalidArgument || flagcxCommFinalize(NULL) != flagcxInvalidArgument) return 17;
+    if (strcmp(flagcxGetLastError(NULL), "Undefined: flagcxComm is not fully initialized.")) return 18;
+    if (flagcxDeviceHandleInit(NULL) != flagcxInvalidArgument || flagcxHandleFree(NULL) != flagcxSuccess) return 19;
+  }
   printf("%s\n", fx_version());
   return 0;
 }

@@ -114,3 +114,78 @@ def test_reference_closed_forms(dev, n):
         r.close()
     comm.return_stream(borrowed, dev.t)
     dev.stream_destroy(stream)
+
+
+def test_application_flow_through_the_device_handle_and_housekeeping_calls():
+    """The calls of a program written against flagcx.h, in the order its perf
+    tests make them (test/perf_common.cc:27-110): device handle, unique id,
+    communicators, stream, flagcxMemAlloc + flagcxCommRegister buffers, an
+    all-reduce with a closed form, deregistration, finalize, destroy / abort."""
+    import ctypes as C
+    L = N.lib
+    handler = C.c_void_p()
+    N.check(L.flagcxHandleInit(C.byref(handler)), "flagcxHandleInit")
+    uid_p, comm_p, dev_p = C.cast(handler, C.POINTER(C.c_void_p))[0:3]
+    assert uid_p is None and comm_p is None and dev_p, "a zeroed group with its device handle filled in"
+    ops = C.cast(dev_p, C.POINTER(C.c_void_p))
+    assert all(ops[i] for i in range(28)), "every device operation is there"
+    RES = C.c_int
+    fn = lambda i, *argtypes: C.CFUNCTYPE(RES, *argtypes)(ops[i])      # index = position in flagcx.h:143-185
+    device_sync, device_memcpy = fn(0), fn(1, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p)
+    set_device, get_count = fn(5, C.c_int), fn(7, C.POINTER(C.c_int))
+    stream_create, stream_destroy, stream_sync = fn(10, C.POINTER(C.c_void_p)), fn(11, C.c_void_p), fn(14, C.c_void_p)
+    ngpu = C.c_int()
+    N.check(get_count(C.byref(ngpu)), "getDeviceCount")
+    assert ngpu.value >= 1
+    N.check(set_device(0), "setDevice")
+    stream = C.c_void_p()
+    N.check(stream_create(C.byref(stream)), "streamCreate")
+
+    n, count = 3, 100003
+    uid = C.create_string_buffer(256)
+    N.check(L.flagcxGetUniqueId(uid), "flagcxGetUniqueId")
+    comms = [C.c_void_p() for _ in range(n)]
+    for r in range(n):
+        N.check(L.flagcxCommInitRank(C.byref(comms[r]), n, uid, r), "flagcxCommInitRank")
+    send, recv, hs, hr = ([C.c_void_p() for _ in range(n)] for _ in range(4))
+    idx = np.arange(count)
+    for r in range(n):
+        N.check(L.flagcxMemAlloc(C.byref(send[r]), count * 4, 0), "flagcxMemAlloc")
+        N.check(L.flagcxMemAlloc(C.byref(recv[r]), count * 4, 0), "flagcxMemAlloc")
+        N.check(L.flagcxCommRegister(comms[r], send[r], count * 4, C.byref(hs[r]), 0), "flagcxCommRegister")
+        N.check(L.flagcxCommRegister(comms[r], recv[r], count * 4, C.byref(hr[r]), 0), "flagcxCommRegister")
+        assert hs[r].value == send[r].value
+        host = (r * 1000 + idx % 10).astype(np.float32)              # coll_allreduce.cpp:9-37
+        N.check(device_memcpy(send[r], host.ctypes.data, count * 4, N.MEMCPY_H2D, None), "deviceMemcpy")
+    for r in range(n):
+        N.check(L.flagcxAllReduce(send[r], recv[r], count, N.DT_FP32, N.OP_SUM, comms[r], stream), "flagcxAllReduce")
+    N.check(stream_sync(stream), "streamSynchronize")
+    want = (n * (n - 1) // 2 * 1000 + n * (idx % 10)).astype(np.float32)
+    for r in range(n):
+        got = np.empty(count, np.float32)
+        N.check(device_memcpy(got.ctypes.data, recv[r], count * 4, N.MEMCPY_D2H, None), "deviceMemcpy")
+        assert np.array_equal(got, want)
+
+    v, err = C.c_int(-1), C.c_int(-1)
+    N.check(L.flagcxIsHomoComm(comms[0], C.byref(v)), "flagcxIsHomoComm")
+    assert v.value == 1
+    N.check(L.flagcxCommGetDeviceNumber(comms[1], C.byref(v)), "flagcxCommGetDeviceNumber")
+    assert v.value == 0
+    N.check(L.flagcxCommGetAsyncError(comms[2], C.byref(err)), "flagcxCommGetAsyncError")
+    assert err.value == N.SUCCESS and L.flagcxGetLastError(comms[0]) == b""
+    assert L.flagcxCommSuspend(comms[0]) == N.INVALID_USAGE and L.flagcxCommResume(comms[0]) == N.INVALID_USAGE
+    win = C.c_void_p(1)
+    assert L.flagcxCommWindowRegister(comms[0], send[0], count * 4, C.byref(win), 1, 0) == N.NOT_SUPPORTED and not win.value
+    for r in range(n):
+        N.check(L.flagcxCommDeregister(comms[r], hs[r], 0), "flagcxCommDeregister")
+        N.check(L.flagcxCommDeregister(comms[r], hr[r], 0), "flagcxCommDeregister")
+        N.check(L.flagcxCommFinalize(comms[r]), "flagcxCommFinalize")
+    N.check(L.flagcxCommAbort(comms[0]), "flagcxCommAbort")
+    for r in range(1, n):
+        N.check(L.flagcxCommDestroy(comms[r]), "flagcxCommDestroy")
+    for r in range(n):
+        N.check(L.flagcxMemFree(send[r], 0), "flagcxMemFree")
+        N.check(L.flagcxMemFree(recv[r], 0), "flagcxMemFree")
+    N.check(device_sync(), "deviceSynchronize")
+    N.check(stream_destroy(stream), "streamDestroy")
+    N.check(L.flagcxHandleFree(handler), "flagcxHandleFree")

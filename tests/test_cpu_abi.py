@@ -426,3 +426,42 @@ def test_torch_backend_module_loads_and_fails_loudly_without_a_gpu():
         pytest.skip("a GPU is visible: the refusal cannot be shown")
     with pytest.raises(RuntimeError, match="flagcxCommInitRank failed"):
         fxb.new_backend(dist.HashStore(), 0, 2)
+
+
+REFERENCE = "/root/reference/flagcx"
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE), reason="the reference's headers are not on this machine")
+def test_headers_agree_with_the_reference_headers(tmp_path):
+    """A translation unit that includes the reference's own flagcx.h and adaptor
+    headers first and this library's headers after them must compile: C++
+    rejects a second declaration of an extern "C" function whose types differ,
+    so every entry point declared here has the reference's signature.  The
+    structures that cross the boundary have the same size either way."""
+    import shutil
+    import subprocess
+    if not shutil.which("g++"):
+        pytest.skip("no g++")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    inc = [f"-I{REFERENCE}/include", f"-I{REFERENCE}/adaptor/include", f"-I{REFERENCE}/core", f"-I{root}/include"]
+    ours = "\n".join(f'#include "flagcx_amd/{h}"' for h in
+                     ["fx_types.h", "fx_device_adaptor.h", "fx_ccl_adaptor.h", "fx_sim.h", "fx_handle.h", "fx_kernels.h"])
+    theirs = '#include <cstring>\n#include "flagcx.h"\n#include "flagcx_device_adaptor.h"\n#include "flagcx_ccl_adaptor.h"\n'
+    sizes = r'''
+#include <cstdio>
+int main() {
+  printf("%zu %zu %zu %zu %zu %d %d %d %d\n", sizeof(flagcxDeviceAdaptor_v1), sizeof(flagcxCCLAdaptor_v1),
+         sizeof(flagcxDeviceHandle), sizeof(flagcxHandlerGroup), sizeof(flagcxUniqueId), (int)flagcxBfloat16, (int)flagcxAvg,
+         (int)flagcxNotSupported, (int)flagcxMemcpyDeviceToDevice);
+  return 0;
+}
+'''
+    out = []
+    for name, text in (("both", theirs + ours + sizes), ("ours", "#include <cstring>\n" + ours + sizes)):
+        src = tmp_path / f"{name}.cc"
+        src.write_text(text)
+        exe = tmp_path / name
+        subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", *inc[-1 if name == "ours" else 0:], str(src), "-o", str(exe)],
+                       check=True)
+        out.append(subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout)
+    assert out[0] == out[1], out

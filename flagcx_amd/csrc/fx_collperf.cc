@@ -16,7 +16,9 @@
 // the timed calls.
 //
 // One host thread posts rank after rank on one stream, as a test program with
-// one process per rank would, minus the processes.  Host code only: buffers,
+// one process per rank would, minus the processes; with -T 1 every rank has a
+// host thread and a stream of its own and a call blocks until all ranks have
+// made it (FX_SYNC_RENDEZVOUS), which is how separate processes behave.  Host code only: buffers,
 // streams and events come through flagcxDeviceHandleInit's table, as in the
 // reference's tests (test/perf_common.cc:27-60).
 #include <getopt.h>
@@ -30,6 +32,7 @@
 #include <cstring>
 #include <functional>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "flagcx_amd/fx_handle.h"
@@ -131,13 +134,15 @@ struct Options {
   int factor = 2, warmup = 5, iters = 20, root = 0, nranks = 8, check = 0;
   int type = 7 /* float */, op = 0;
   int algo = -1, order = -1;
+  int threads = 0;   // -T 1: one host thread and one stream per rank, calls that block until every rank has posted
 };
 
 void usage(const char *argv0) {
   printf("Usage: %s <allreduce|reduce|reducescatter|allgather|broadcast|gather|scatter|alltoall|alltoallv|sendrecv>\n\t"
          "[-b <minbytes K/M/G>] [-e <maxbytes K/M/G>] [-f <stepfactor>] [-w <warmupiters>] [-n <iters>]\n\t"
          "[-r <root>] [-o <sum|prod|max|min|avg>] [-d <int8|uint8|int32|uint32|int64|uint64|half|float|double|bfloat16>]\n\t"
-         "[-N <simulated ranks, 1..64>] [-A <direct|ring>] [-O <rank|ring|host>] [-c <check 0/1>]\n",
+         "[-N <simulated ranks, 1..64>] [-A <direct|ring>] [-O <rank|ring|host>] [-c <check 0/1>]\n\t"
+         "[-T <0: one thread posts every rank on one stream | 1: a thread and a stream per rank>]\n",
          argv0);
 }
 
@@ -161,9 +166,10 @@ Options parse(int argc, char **argv) {
                               {"op", required_argument, 0, 'o'}, {"datatype", required_argument, 0, 'd'},
                               {"nranks", required_argument, 0, 'N'}, {"algo", required_argument, 0, 'A'},
                               {"order", required_argument, 0, 'O'}, {"check", required_argument, 0, 'c'},
+                              {"threads", required_argument, 0, 'T'},
                               {"help", no_argument, 0, 'h'}, {}};
   optind = 2;
-  for (int c; (c = getopt_long(argc, argv, "b:e:f:w:n:r:o:d:N:A:O:c:h", longOpts, nullptr)) != -1;) {
+  for (int c; (c = getopt_long(argc, argv, "b:e:f:w:n:r:o:d:N:A:O:c:T:h", longOpts, nullptr)) != -1;) {
     const std::string a = optarg ? optarg : "";
     bool bad = false;
     switch (c) {
@@ -175,6 +181,7 @@ Options parse(int argc, char **argv) {
       case 'r': o.root = atoi(optarg); break;
       case 'N': o.nranks = atoi(optarg); bad = o.nranks < 1 || o.nranks > 64; break;
       case 'c': o.check = atoi(optarg); break;
+      case 'T': o.threads = atoi(optarg); bad = o.threads != 0 && o.threads != 1; break;
       case 'o':
         bad = true;
         for (int i = 0; i < 5; i++)
@@ -221,7 +228,8 @@ struct Run {
   int n;
   std::vector<flagcxComm_t> comms;
   std::vector<void *> send, recv;
-  flagcxStream_t stream = nullptr;
+  flagcxStream_t stream = nullptr;         // rank 0's, and everybody's without -T 1
+  std::vector<flagcxStream_t> streams;     // one per rank (all the same without -T 1)
   std::vector<size_t> sc, sd, rc, rd;   // alltoallv, one row of n per rank
 
   Shape shape(size_t count) const {
@@ -247,17 +255,17 @@ struct Run {
   int post(int r, size_t count) {
     const flagcxRedOp_t op = (flagcxRedOp_t)o.op;
     switch (o.kind) {
-      case kAllReduce: return flagcxAllReduce(send[r], recv[r], count, t.code, op, comms[r], stream);
-      case kReduce: return flagcxReduce(send[r], recv[r], count, t.code, op, o.root, comms[r], stream);
-      case kReduceScatter: return flagcxReduceScatter(send[r], recv[r], count / n, t.code, op, comms[r], stream);
-      case kAllGather: return flagcxAllGather(send[r], recv[r], count / n, t.code, comms[r], stream);
-      case kBroadcast: return flagcxBroadcast(send[r], recv[r], count, t.code, o.root, comms[r], stream);
-      case kGather: return flagcxGather(send[r], recv[r], count / n, t.code, o.root, comms[r], stream);
-      case kScatter: return flagcxScatter(send[r], recv[r], count / n, t.code, o.root, comms[r], stream);
-      case kAlltoAll: return flagcxAlltoAll(send[r], recv[r], count / n, t.code, comms[r], stream);
+      case kAllReduce: return flagcxAllReduce(send[r], recv[r], count, t.code, op, comms[r], streams[r]);
+      case kReduce: return flagcxReduce(send[r], recv[r], count, t.code, op, o.root, comms[r], streams[r]);
+      case kReduceScatter: return flagcxReduceScatter(send[r], recv[r], count / n, t.code, op, comms[r], streams[r]);
+      case kAllGather: return flagcxAllGather(send[r], recv[r], count / n, t.code, comms[r], streams[r]);
+      case kBroadcast: return flagcxBroadcast(send[r], recv[r], count, t.code, o.root, comms[r], streams[r]);
+      case kGather: return flagcxGather(send[r], recv[r], count / n, t.code, o.root, comms[r], streams[r]);
+      case kScatter: return flagcxScatter(send[r], recv[r], count / n, t.code, o.root, comms[r], streams[r]);
+      case kAlltoAll: return flagcxAlltoAll(send[r], recv[r], count / n, t.code, comms[r], streams[r]);
       case kAlltoAllv:
         return flagcxAlltoAllv(send[r], &sc[(size_t)r * n], &sd[(size_t)r * n], recv[r], &rc[(size_t)r * n], &rd[(size_t)r * n],
-                               t.code, comms[r], stream);
+                               t.code, comms[r], streams[r]);
       default: return flagcxInvalidArgument;
     }
   }
@@ -278,6 +286,35 @@ struct Run {
       const int rc_ = post(r, count);
       if (rc_ != flagcxSuccess) die(o.coll.c_str(), rc_);
     }
+  }
+
+  // -T 1: every rank's thread makes `times` calls of its own; a call returns when all ranks have made theirs
+  void threaded(size_t count, int times) {
+    std::vector<std::thread> ts;
+    for (int r = 0; r < n; r++)
+      ts.emplace_back([this, r, count, times] {
+        for (int i = 0; i < times; i++) {
+          if (o.kind == kSendRecv) {
+            OK(flagcxGroupStart(comms[r]));
+            OK(flagcxSend(send[r], count, t.code, (r + 1) % n, comms[r], streams[r]));
+            OK(flagcxRecv(recv[r], count, t.code, (r + n - 1) % n, comms[r], streams[r]));
+            OK(flagcxGroupEnd(comms[r]));
+          } else {
+            const int rc_ = post(r, count);
+            if (rc_ != flagcxSuccess) die(o.coll.c_str(), rc_);
+          }
+        }
+      });
+    for (auto &th : ts) th.join();
+  }
+
+  void repeat(size_t count, int times) {
+    if (o.threads) return threaded(count, times);
+    for (int i = 0; i < times; i++) once(count);
+  }
+
+  void syncAll() {
+    for (int r = 0; r < (o.threads ? n : 1); r++) OK(dev->streamSynchronize(streams[r]));
   }
 
   // alltoallv with the ragged pattern of the reference's test (test_alltoallv.cpp:10-52): a rank
@@ -355,6 +392,11 @@ int main(int argc, char **argv) {
   if (run.o.algo >= 0) OK(fxSimCommConfig(run.comms[0], FX_SIM_ALGO, run.o.algo));
   if (run.o.order >= 0) OK(fxSimCommConfig(run.comms[0], FX_SIM_ORDER, run.o.order));
   OK(dev->streamCreate(&run.stream));
+  run.streams.assign(n, run.stream);
+  if (run.o.threads) {
+    OK(fxSimCommConfig(run.comms[0], FX_SIM_SYNC, FX_SYNC_RENDEZVOUS));
+    for (int r = 1; r < n; r++) OK(dev->streamCreate(&run.streams[r]));
+  }
   flagcxEvent_t t0, t1;
   OK(dev->eventCreate(&t0, flagcxEventDefault));
   OK(dev->eventCreate(&t1, flagcxEventDefault));
@@ -374,8 +416,10 @@ int main(int argc, char **argv) {
   const bool checkable = run.o.check && (!reduces(run.o.kind) || (exactType && run.o.op != flagcxProd && run.o.op != flagcxAvg));
   char vendor[128] = "";
   OK(dev->getVendor(vendor));
-  printf("# %s over %d simulated ranks on one GPU; buffers, stream and events through the device handle (%s)\n",
-         run.o.coll.c_str(), n, vendor);
+  printf("# %s over %d simulated ranks on one GPU; buffers, stream and events through the device handle (%s); %s\n",
+         run.o.coll.c_str(), n, vendor,
+         run.o.threads ? "a host thread and a stream per rank, calls block until every rank has posted"
+                       : "one host thread posts rank after rank on one stream");
   printf("#\n# datatype: %s, op: %s\n#\n", run.t.name, kOps[run.o.op]);
   if (run.o.check && !checkable)
     printf("# no check for this datatype / op: the pattern's sums are exact only in 4- and 8-byte types\n");
@@ -392,14 +436,14 @@ int main(int argc, char **argv) {
       if (sh.recvElems) OK(dev->deviceMemset(run.recv[r], 0xff, sh.recvElems * run.t.size, flagcxMemDevice, nullptr));
     }
     OK(dev->deviceSynchronize());
-    for (int i = 0; i < run.o.warmup; i++) run.once(count);
-    OK(dev->streamSynchronize(run.stream));
+    run.repeat(count, run.o.warmup);
+    run.syncAll();
 
     OK(dev->eventRecord(t0, run.stream));
     const double w0 = seconds();
-    for (int i = 0; i < run.o.iters; i++) run.once(count);
+    run.repeat(count, run.o.iters);
     OK(dev->eventRecord(t1, run.stream));
-    OK(dev->streamSynchronize(run.stream));
+    run.syncAll();
     const double elapsed = (seconds() - w0) / run.o.iters;
     float ms = 0;
     OK(dev->eventElapsedTime(&ms, t0, t1));
@@ -446,6 +490,7 @@ int main(int argc, char **argv) {
   }
   OK(dev->eventDestroy(t0));
   OK(dev->eventDestroy(t1));
+  for (int r = 1; r < n && run.o.threads; r++) OK(dev->streamDestroy(run.streams[r]));
   OK(dev->streamDestroy(run.stream));
   OK(fxSimCommDestroyAll(run.comms.data(), n));
   OK(flagcxDeviceHandleFree(dev));

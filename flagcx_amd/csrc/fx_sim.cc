@@ -43,6 +43,7 @@ struct Post {
   const void *send = nullptr;
   void *recv = nullptr;
   hipStream_t stream = nullptr;
+  bool marked = false;     // rendezvous mode: the rank's own event already stands on its stream
   std::vector<size_t> sendcounts, sdispls, recvcounts, rdispls;
 };
 
@@ -77,11 +78,12 @@ struct Group {
   hipEvent_t done = nullptr;
   // rendezvous mode: posters sleep here until the collective they joined is launched
   std::condition_variable cv;
-  uint64_t launched = 0;       // collectives launched (or abandoned) so far
+  std::atomic<uint64_t> launched{0};   // collectives launched (or abandoned) so far
+  hipStream_t launchStream = nullptr;  // rendezvous mode: where the last collective went, for the ranks it woke
   flagcxResult_t lastResult = flagcxSuccess;
   long long timeoutMs = 30000;
   // configuration
-  long long sync = FX_SYNC_GROUP;
+  std::atomic<long long> sync{FX_SYNC_GROUP};   // read without the lock by a rank that marks its stream before posting
   long long algo = FX_ALGO_DIRECT, order = FX_ORDER_RANK;
   long long nslices = 1, nredslices = 0, redslicesize = 65536;
   // scratch: ring reduce-scatter partials / alltoallv staging.  Outgrown
@@ -884,6 +886,12 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   if (!comm || !comm->g || !stream) return flagcxInvalidArgument;
   Group *g = comm->g;
   const int rank = comm->rank;
+  // Rendezvous mode: this rank's thread stays in the call until the launch, so
+  // its stream stands where it will stand then.  Every rank marks the spot
+  // itself, before queueing for the lock, instead of leaving all the marks to
+  // the last rank in.
+  const bool marked = g->n > 1 && g->sync.load(std::memory_order_relaxed) == FX_SYNC_RENDEZVOUS &&
+                      hipEventRecord(g->ready[rank], stream->base) == hipSuccess;
   std::unique_lock<std::mutex> lock(g->mu);
   if (g->nposted == 0) {
     g->kind = kind;
@@ -904,6 +912,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   p.send = send;
   p.recv = recv;
   p.stream = stream->base;
+  p.marked = marked;
   comm->joined = g->launched;
   if (kind == kAlltoAllv) {
     p.sendcounts.assign(sc, sc + g->n);
@@ -913,16 +922,25 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   }
   if (++g->nposted < g->n) {
     if (g->sync != FX_SYNC_RENDEZVOUS) return flagcxSuccess;
-    // Sleep until the last rank has launched this collective (it also makes this
-    // rank's stream wait for the result before it wakes us).
+    // Wait until the last rank has launched this collective.
     const uint64_t mine = g->launched;
     if (!g->cv.wait_for(lock, std::chrono::milliseconds(g->timeoutMs), [&] { return g->launched != mine; })) {
       resetPending(g);  // a rank never arrived: give up for everybody
       g->lastResult = flagcxInternalError;
       g->launched++;
       g->cv.notify_all();
+      return flagcxInternalError;
     }
-    return g->lastResult;
+    // What this rank enqueues next comes after the collective: each woken rank
+    // makes its own stream wait (the next collective cannot move the event before
+    // this rank has posted again).
+    const flagcxResult_t res = g->lastResult;
+    const hipStream_t where = g->launchStream, own = stream->base;
+    hipEvent_t done = g->done;
+    lock.unlock();
+    if (res == flagcxSuccess && where != own && hipStreamWaitEvent(own, done, 0) != hipSuccess)
+      return flagcxUnhandledDeviceError;
+    return res;
   }
 
   // Last rank in: order the launch after everything the other ranks' streams
@@ -932,7 +950,12 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   flagcxResult_t res = flagcxSuccess;
   for (int r = 0; r < g->n && res == flagcxSuccess; r++) {
     hipStream_t s = g->posts[r].stream;
-    bool seen = (s == c.s);
+    if (s == c.s) continue;
+    if (g->posts[r].marked) {   // the rank's thread has recorded its own event
+      if (hipStreamWaitEvent(c.s, g->ready[r], 0) != hipSuccess) res = flagcxUnhandledDeviceError;
+      continue;
+    }
+    bool seen = false;
     for (int q = 0; q < r && !seen; q++) seen = (g->posts[q].stream == s);
     if (seen) continue;
     if (hipEventRecord(g->ready[r], s) != hipSuccess || hipStreamWaitEvent(c.s, g->ready[r], 0) != hipSuccess)
@@ -959,7 +982,9 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
     for (int r = 0; r < g->n; r++) others = others || (g->posts[r].stream != c.s);
     if (others) {
       if (hipEventRecord(g->done, c.s) != hipSuccess) res = flagcxUnhandledDeviceError;
-      for (int r = 0; r < g->n && res == flagcxSuccess; r++) {
+      // group mode: the other ranks' calls have returned, so their streams are made to wait here;
+      // rendezvous mode: every rank does that for itself when it wakes
+      for (int r = 0; r < g->n && res == flagcxSuccess && g->sync != FX_SYNC_RENDEZVOUS; r++) {
         hipStream_t s = g->posts[r].stream;
         bool seen = (s == c.s);
         for (int q = 0; q < r && !seen; q++) seen = (g->posts[q].stream == s);
@@ -967,6 +992,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
       }
     }
   }
+  g->launchStream = c.s;
   resetPending(g);
   g->lastResult = res;
   g->launched++;

@@ -29,6 +29,14 @@ def test_tool_checks_its_own_results(coll):
         assert len(lines) == 3 and all("Bus bandwidth" in ln and "on the device" in ln for ln in lines), out
 
 
+@pytest.mark.parametrize("coll", ["allreduce", "reducescatter", "allgather", "alltoallv", "sendrecv"])
+def test_a_thread_and_a_stream_per_rank(coll):
+    """-T 1: every rank's calls come from its own host thread on its own stream
+    and block until all ranks have posted, the way separate processes behave."""
+    out = run(coll, "-b", "64K", "-e", "4M", "-f", "8", "-w", "2", "-n", "10", "-c", "1", "-T", "1", "-N", "4")
+    assert "a host thread and a stream per rank" in out and "# check: every rank's result as expected" in out, out
+
+
 def test_tool_moves_narrow_types_and_reports_what_it_cannot_check():
     out = run("allgather", "-b", "64K", "-e", "64K", "-d", "bfloat16", "-c", "1", "-n", "2")
     assert "# check: every rank's result as expected" in out

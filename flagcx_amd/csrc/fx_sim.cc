@@ -44,6 +44,7 @@ struct Post {
   void *recv = nullptr;
   hipStream_t stream = nullptr;
   bool marked = false;     // rendezvous mode: the rank's own event already stands on its stream
+  bool idle = false;       // rendezvous mode: the rank's stream had nothing left to do when it posted
   std::vector<size_t> sendcounts, sdispls, recvcounts, rdispls;
 };
 
@@ -890,8 +891,16 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   // its stream stands where it will stand then.  Every rank marks the spot
   // itself, before queueing for the lock, instead of leaving all the marks to
   // the last rank in.
-  const bool marked = g->n > 1 && g->sync.load(std::memory_order_relaxed) == FX_SYNC_RENDEZVOUS &&
-                      hipEventRecord(g->ready[rank], stream->base) == hipSuccess;
+  // A stream with nothing left to do needs no mark at all: nothing can be added
+  // to it while its rank's thread is in here.
+  bool marked = false, idle = false;
+  if (g->n > 1 && g->sync.load(std::memory_order_relaxed) == FX_SYNC_RENDEZVOUS) {
+    idle = hipStreamQuery(stream->base) == hipSuccess;
+    if (!idle) {
+      (void)hipGetLastError();   // "not ready" is an answer, not an error to leave behind for the caller's next check
+      marked = hipEventRecord(g->ready[rank], stream->base) == hipSuccess;
+    }
+  }
   std::unique_lock<std::mutex> lock(g->mu);
   if (g->nposted == 0) {
     g->kind = kind;
@@ -913,6 +922,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   p.recv = recv;
   p.stream = stream->base;
   p.marked = marked;
+  p.idle = idle;
   comm->joined = g->launched;
   if (kind == kAlltoAllv) {
     p.sendcounts.assign(sc, sc + g->n);
@@ -938,8 +948,11 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
     const hipStream_t where = g->launchStream, own = stream->base;
     hipEvent_t done = g->done;
     lock.unlock();
-    if (res == flagcxSuccess && where != own && hipStreamWaitEvent(own, done, 0) != hipSuccess)
-      return flagcxUnhandledDeviceError;
+    if (res == flagcxSuccess && where != own) {
+      if (hipEventQuery(done) == hipSuccess) return res;   // already over: anything enqueued from now on is after it
+      (void)hipGetLastError();                             // "not ready" is an answer, not an error
+      if (hipStreamWaitEvent(own, done, 0) != hipSuccess) return flagcxUnhandledDeviceError;
+    }
     return res;
   }
 
@@ -950,7 +963,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   flagcxResult_t res = flagcxSuccess;
   for (int r = 0; r < g->n && res == flagcxSuccess; r++) {
     hipStream_t s = g->posts[r].stream;
-    if (s == c.s) continue;
+    if (s == c.s || g->posts[r].idle) continue;
     if (g->posts[r].marked) {   // the rank's thread has recorded its own event
       if (hipStreamWaitEvent(c.s, g->ready[r], 0) != hipSuccess) res = flagcxUnhandledDeviceError;
       continue;

@@ -31,9 +31,9 @@
  *     stream, the way separate FlagCX processes behave: a call blocks its host
  *     thread until every rank has posted and the work is enqueued, so whatever
  *     the rank enqueues after the call returns is ordered after the collective.
- *     Ordering n streams around one launch costs n - 1 event marks and waits on
- *     either side (tens of microseconds for eight ranks); the default mode on one
- *     stream needs none.
+ *     Handing n threads through the group's lock and ordering n streams
+ *     around one launch costs tens of microseconds for eight ranks; the
+ *     default mode on one stream needs neither.
  *     A rank that never arrives makes the others return flagcxInternalError
  *     after FX_SIM_RENDEZVOUS_TIMEOUT_MS (environment, default 30000).
  *     flagcxSend / flagcxRecv posted between flagcxGroupStart and

@@ -806,3 +806,49 @@ def test_progress_tells_a_rank_when_its_collective_has_been_launched(dev, stream
             assert [g.progress(r) for r in range(n)] == [(turn, turn + 1)] * n
         dev.stream_sync(stream)
         assert (dev.to_host(bufs[0], count, np.float32) == 6 * 3).all()
+
+
+def test_rendezvous_mode_with_busy_streams_and_no_host_waits(dev):
+    """One host thread and one stream per rank, nothing but stream order between
+    the steps: every round a rank fills its send buffer on its own stream behind
+    a long copy (so the stream is busy when the rank posts), all-reduces, and
+    copies the result into that round's slot of a history buffer -- the only
+    host wait is at the very end.  A collective that ran before a rank's fill, or
+    a result copy that ran before the collective, shows up as a wrong slot."""
+    import threading
+    n, count, rounds = 6, 1 << 20, 10          # 4 MiB of int32 per rank
+    big = 96 << 20
+    errors = []
+    with DevBufs(dev) as b, S.SimGroup(n, sync=S.SYNC_RENDEZVOUS) as g:
+        send = [b.alloc(count * 4) for _ in range(n)]
+        recv = [b.alloc(count * 4) for _ in range(n)]
+        hist = [b.alloc(rounds * count * 4) for _ in range(n)]
+        ballast = [(b.alloc(big), b.alloc(big)) for _ in range(n)]
+
+        def rank_main(r):
+            try:
+                dev.set_device()
+                s = dev.stream_create()
+                for it in range(rounds):
+                    if (it + r) % 3:                                   # two rounds in three: keep the stream busy
+                        dev.copy(ballast[r][1], ballast[r][0], big, s)
+                    dev.memset(send[r], (r + 1) * (it + 1) % 41, count * 4, s)     # every byte, so every int32 = 0x01010101 * v
+                    N.check(N.lib.flagcxAllReduce(send[r], recv[r], count, N.DT_INT32, N.OP_SUM, g.comms[r], s))
+                    dev.copy(hist[r] + it * count * 4, recv[r], count * 4, s)
+                dev.stream_sync(s)
+                got = dev.to_host(hist[r], rounds * count, np.uint32).reshape(rounds, count)
+                for it in range(rounds):
+                    want = 0x01010101 * sum((q + 1) * (it + 1) % 41 for q in range(n))
+                    if not (got[it] == want).all():
+                        errors.append((r, it, hex(int(got[it][0])), hex(want)))
+                dev.stream_destroy(s)
+            except Exception as e:                      # noqa: BLE001 - reported below
+                errors.append((r, repr(e)))
+
+        threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=100)
+        assert not any(t.is_alive() for t in threads)
+        assert not errors, errors[:6]

@@ -57,6 +57,15 @@ struct PendingP2p {
   size_t bytes;
   hipStream_t stream;
   uint64_t id;             // names this half for a sleeping poster (rendezvous mode)
+  int owner;               // the rank that posted it
+  bool idle, marked;       // rendezvous mode: its stream had nothing left to do / carries the owner's mark (ready[owner])
+};
+
+// What a sleeping poster finds when its partner has come (rendezvous mode).
+struct P2pOutcome {
+  flagcxResult_t res;
+  int by;                  // the rank whose call enqueued the copy, -1 if nothing was enqueued
+  hipStream_t where;       // on this stream
 };
 
 struct Group {
@@ -69,7 +78,8 @@ struct Group {
   std::vector<PendingP2p> p2p;
   hipEvent_t p2pBefore = nullptr, p2pAfter = nullptr;   // made at the first pair whose halves sit on two streams
   uint64_t nextP2pId = 1;
-  std::map<uint64_t, flagcxResult_t> p2pMatched;  // rendezvous mode: results awaiting their sleeping poster
+  std::map<uint64_t, P2pOutcome> p2pMatched;      // rendezvous mode: results awaiting their sleeping poster
+  std::vector<hipEvent_t> after;                  // rendezvous mode: after[r] follows the latest copy rank r enqueued for a partner
   // pending collective
   Kind kind = kNone;
   size_t count = 0;
@@ -1027,6 +1037,8 @@ void freeGroupResources(Group *g) {
   for (auto e : g->ready)
     if (e) (void)hipEventDestroy(e);
   if (g->done) (void)hipEventDestroy(g->done);
+  for (auto e : g->after)
+    if (e) (void)hipEventDestroy(e);
   if (g->p2pBefore) (void)hipEventDestroy(g->p2pBefore);
   if (g->p2pAfter) (void)hipEventDestroy(g->p2pAfter);
   if (g->scratch) (void)hipFree(g->scratch);
@@ -1083,18 +1095,34 @@ void freeGroup(Group *g) {
 }
 
 // Group brackets are per host thread (the CCL adaptor's groupStart / groupEnd
-// carry no communicator).  They matter in rendezvous mode only: a send or recv
-// posted inside a bracket does not sleep until its partner arrives -- every
-// rank's thread would sit in its first call and none would reach its second --
-// it is remembered here and waited for when the outermost bracket closes, which
-// is where the reference issues the grouped operations (flagcx/flagcx.cc group
-// semantics; rccl_adaptor.cc:322-332 forwards the bracket to the vendor library).
+// carry no communicator).  In rendezvous mode a send or recv made inside a
+// bracket must not sleep until its partner arrives -- every rank's thread would
+// sit in its first call and none would reach its second -- so it is written
+// down, and the outermost flagcxGroupEnd of the thread posts the bracket's
+// halves and then waits for their partners: where the reference issues grouped
+// operations too (flagcx/flagcx.cc group semantics; rccl_adaptor.cc:322-332
+// forwards the bracket to the vendor library).
 struct DeferredP2p {
   Group *g;
   uint64_t id;
+  hipStream_t stream;
+};
+// Rendezvous mode: a send or recv made inside a bracket is only written down;
+// the outermost flagcxGroupEnd of the thread posts them all, then waits for the
+// partners of those that found none waiting.
+struct QueuedP2p {
+  flagcxComm_t comm;
+  bool isSend;
+  const void *sbuf;
+  void *rbuf;
+  size_t count;
+  int dtype, peer;
+  flagcxStream_t stream;
 };
 thread_local int tGroupDepth = 0;
+thread_local bool tClosingBracket = false;
 thread_local std::vector<DeferredP2p> tDeferred;
+thread_local std::vector<QueuedP2p> tQueued;
 
 // Copies of pairs that were matched inside a bracket with both halves on one
 // stream (ranks posted one after another by one thread): they leave as one
@@ -1119,9 +1147,10 @@ flagcxResult_t flushBatched() {
 }
 
 // Wait until the partner of pending half `id` has made its call (it enqueues the
-// copy and makes our stream wait for it) and hand back its result; on time-out
-// the half is withdrawn.  Called with g->mu held.
-flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64_t id) {
+// copy) and hand back its result, with this rank's stream ordered after the
+// copy unless that is over already; on time-out the half is withdrawn.  Called
+// with g->mu held; returns with it released.
+flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64_t id, hipStream_t own) {
   const bool matched = g->cv.wait_for(lock, std::chrono::milliseconds(g->timeoutMs),
                                       [&] { return g->p2pMatched.count(id) != 0; });
   if (!matched) {  // the partner never came: withdraw this half
@@ -1130,11 +1159,20 @@ flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64
         g->p2p.erase(g->p2p.begin() + (long)i);
         break;
       }
+    lock.unlock();
     return flagcxInternalError;
   }
-  const flagcxResult_t res = g->p2pMatched[id];
+  const P2pOutcome out = g->p2pMatched[id];
   g->p2pMatched.erase(id);
-  return res;
+  hipEvent_t follows = (out.by >= 0 && out.where != own) ? g->after[(size_t)out.by] : nullptr;
+  lock.unlock();
+  if (out.res == flagcxSuccess && follows) {
+    // the partner may have moved its event on to a later copy of its own by now: later on the same stream, so still after ours
+    if (hipEventQuery(follows) == hipSuccess) return out.res;
+    (void)hipGetLastError();   // "not ready" is an answer, not an error
+    if (hipStreamWaitEvent(own, follows, 0) != hipSuccess) return flagcxUnhandledDeviceError;
+  }
+  return out.res;
 }
 
 // send / recv between simulated ranks: the later of the two calls performs the
@@ -1158,25 +1196,50 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
   const size_t ts = fx_dtype_size(dtype);
   if (ts == 0 || peer < 0 || peer >= g->n) return flagcxInvalidArgument;
   if (count && !(isSend ? sbuf : (const void *)rbuf)) return flagcxInvalidArgument;
+  const bool rendezvous = g->sync.load(std::memory_order_relaxed) == FX_SYNC_RENDEZVOUS;
+  if (rendezvous && tGroupDepth > 0 && !tClosingBracket) {
+    tQueued.push_back(QueuedP2p{comm, isSend, sbuf, rbuf, count, dtype, peer, stream});
+    return flagcxSuccess;
+  }
   const int src = isSend ? comm->rank : peer, dst = isSend ? peer : comm->rank;
   const size_t bytes = count * ts;
+  hipStream_t s = stream->base;
   std::unique_lock<std::mutex> lock(g->mu);
   for (size_t i = 0; i < g->p2p.size(); i++) {
     PendingP2p &o = g->p2p[i];
     if (o.isSend == isSend || o.src != src || o.dst != dst) continue;
     flagcxResult_t res = flagcxSuccess;
+    bool enqueued = false;
     if (o.bytes != bytes) {
       res = flagcxInvalidArgument;  // the two sides disagree on the message size
     } else if (bytes) {
-      hipStream_t s = stream->base;
       fxSliceDesc d = copyDesc(isSend ? sbuf : o.sbuf, isSend ? o.rbuf : rbuf, bytes);
-      if (o.stream == s && tGroupDepth > 0 && g->sync != FX_SYNC_RENDEZVOUS) {
+      if (o.stream == s && tGroupDepth > 0 && !rendezvous) {
         size_t b = 0;
         while (b < tBatched.size() && tBatched[b].stream != s) b++;
         if (b == tBatched.size()) tBatched.push_back(BatchedCopies{s, {}});
         tBatched[b].copies.push_back(d);
       } else if (o.stream == s) {
         res = R(fx_copy_slices(&d, 1, s));
+      } else if (rendezvous) {
+        // The other half's thread is inside its call (or its flagcxGroupEnd) until we are done: its stream stands
+        // still.  An idle one needs no waiting for, a busy one carries its owner's mark; and the owner makes
+        // its own stream wait for the copy when it wakes, through after[this rank].
+        if (g->after.empty()) g->after.assign((size_t)g->n, nullptr);
+        hipEvent_t &mine = g->after[(size_t)comm->rank];
+        if (o.marked) {
+          if (hipStreamWaitEvent(s, g->ready[(size_t)o.owner], 0) != hipSuccess) res = flagcxUnhandledDeviceError;
+        } else if (!o.idle) {   // posted before the group was switched to this mode: mark its stream from here
+          if ((!g->p2pBefore && hipEventCreateWithFlags(&g->p2pBefore, hipEventDisableTiming) != hipSuccess) ||
+              hipEventRecord(g->p2pBefore, o.stream) != hipSuccess || hipStreamWaitEvent(s, g->p2pBefore, 0) != hipSuccess)
+            res = flagcxUnhandledDeviceError;
+        }
+        if (res == flagcxSuccess) res = R(fx_copy_slices(&d, 1, s));
+        if (res == flagcxSuccess &&
+            ((!mine && hipEventCreateWithFlags(&mine, hipEventDisableTiming) != hipSuccess) ||
+             hipEventRecord(mine, s) != hipSuccess))
+          res = flagcxUnhandledDeviceError;
+        enqueued = res == flagcxSuccess;
       } else {
         if ((!g->p2pBefore && hipEventCreateWithFlags(&g->p2pBefore, hipEventDisableTiming) != hipSuccess) ||
             (!g->p2pAfter && hipEventCreateWithFlags(&g->p2pAfter, hipEventDisableTiming) != hipSuccess) ||
@@ -1188,22 +1251,33 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
           res = flagcxUnhandledDeviceError;
       }
     }
-    if (g->sync == FX_SYNC_RENDEZVOUS) {
-      g->p2pMatched[o.id] = res;
+    if (rendezvous) {
+      g->p2pMatched[o.id] = P2pOutcome{res, enqueued ? comm->rank : -1, s};
       g->cv.notify_all();
     }
     g->p2p.erase(g->p2p.begin() + (long)i);
     return res;
   }
-  g->p2p.push_back(PendingP2p{isSend, src, dst, sbuf, rbuf, bytes, stream->base, g->nextP2pId++});
-  if (g->sync != FX_SYNC_RENDEZVOUS) return flagcxSuccess;
+  // No partner yet.  In rendezvous mode this thread now stays inside the library until one comes, so the stream's
+  // state is final: idle, or marked here for the partner to wait on.
+  bool idle = false, marked = false;
+  if (rendezvous && bytes) {
+    idle = hipStreamQuery(s) == hipSuccess;
+    if (!idle) {
+      (void)hipGetLastError();   // "not ready" is an answer, not an error
+      marked = hipEventRecord(g->ready[(size_t)comm->rank], s) == hipSuccess;
+      if (!marked) return flagcxUnhandledDeviceError;
+    }
+  }
+  g->p2p.push_back(PendingP2p{isSend, src, dst, sbuf, rbuf, bytes, s, g->nextP2pId++, comm->rank, idle, marked});
+  if (!rendezvous) return flagcxSuccess;
   const uint64_t id = g->p2p.back().id;
-  if (tGroupDepth > 0) {  // inside a bracket: the wait happens when the bracket closes
-    tDeferred.push_back(DeferredP2p{g, id});
+  if (tClosingBracket) {  // flagcxGroupEnd posts all of the bracket's halves before it waits for any
+    tDeferred.push_back(DeferredP2p{g, id, s});
     return flagcxSuccess;
   }
   // Sleep until the partner has made its call and enqueued the copy.
-  return awaitPartner(g, lock, id);
+  return awaitPartner(g, lock, id, s);
 }
 
 }  // namespace
@@ -1495,11 +1569,23 @@ flagcxResult_t flagcxGroupEnd(flagcxComm_t) {
   if (--tGroupDepth > 0) return flagcxSuccess;
   return R(fx::guarded([&]() -> int {
     flagcxResult_t first = flushBatched();
+    std::vector<QueuedP2p> queued;
+    queued.swap(tQueued);
+    {
+      struct Closing {
+        Closing() { tClosingBracket = true; }
+        ~Closing() { tClosingBracket = false; }
+      } closing;
+      for (const QueuedP2p &q : queued) {
+        const flagcxResult_t rc = postP2pImpl(q.comm, q.isSend, q.sbuf, q.rbuf, q.count, q.dtype, q.peer, q.stream);
+        if (first == flagcxSuccess) first = rc;
+      }
+    }
     std::vector<DeferredP2p> mine;
     mine.swap(tDeferred);
     for (const DeferredP2p &d : mine) {
       std::unique_lock<std::mutex> lock(d.g->mu);
-      const flagcxResult_t rc = awaitPartner(d.g, lock, d.id);
+      const flagcxResult_t rc = awaitPartner(d.g, lock, d.id, d.stream);
       if (first == flagcxSuccess) first = rc;
     }
     return first;

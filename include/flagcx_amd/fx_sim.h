@@ -36,10 +36,12 @@
  *     default mode on one stream needs neither.
  *     A rank that never arrives makes the others return flagcxInternalError
  *     after FX_SIM_RENDEZVOUS_TIMEOUT_MS (environment, default 30000).
- *     flagcxSend / flagcxRecv posted between flagcxGroupStart and
+ *     flagcxSend / flagcxRecv made between flagcxGroupStart and
  *     flagcxGroupEnd on a host thread do not block: the outermost
- *     flagcxGroupEnd of that thread waits for their partners, so every rank's
- *     thread can run GroupStart, Send(next), Recv(prev), GroupEnd.
+ *     flagcxGroupEnd of that thread posts them and waits for their partners,
+ *     so every rank's thread can run GroupStart, Send(next), Recv(prev),
+ *     GroupEnd; argument errors of such calls are reported at once, everything
+ *     else by that flagcxGroupEnd.
  *
  * Scratch (partials of the tree reduce and of the ring reduce-scatter, the
  * host order's floating max / min, staging of in-place all-to-all(v)) is grown

@@ -450,9 +450,12 @@ def test_headers_agree_with_the_reference_headers(tmp_path):
     sizes = r'''
 #include <cstdio>
 int main() {
-  printf("%zu %zu %zu %zu %zu %d %d %d %d\n", sizeof(flagcxDeviceAdaptor_v1), sizeof(flagcxCCLAdaptor_v1),
-         sizeof(flagcxDeviceHandle), sizeof(flagcxHandlerGroup), sizeof(flagcxUniqueId), (int)flagcxBfloat16, (int)flagcxAvg,
-         (int)flagcxNotSupported, (int)flagcxMemcpyDeviceToDevice);
+  /* the unique ids as test/unittest/service/test_unique_id.cpp pins them: 256 bytes in public, 4120 inside, 8-aligned */
+  static_assert(sizeof(flagcxUniqueId) == 256 && sizeof(flagcxInnerUniqueId) == 4120, "unique id sizes");
+  static_assert(alignof(flagcxInnerUniqueId) >= alignof(uint64_t), "inner unique id alignment");
+  printf("%zu %zu %zu %zu %zu %zu %d %d %d %d\n", sizeof(flagcxDeviceAdaptor_v1), sizeof(flagcxCCLAdaptor_v1),
+         sizeof(flagcxDeviceHandle), sizeof(flagcxHandlerGroup), sizeof(flagcxUniqueId), sizeof(flagcxInnerUniqueId),
+         (int)flagcxBfloat16, (int)flagcxAvg, (int)flagcxNotSupported, (int)flagcxMemcpyDeviceToDevice);
   return 0;
 }
 '''

@@ -18,6 +18,12 @@ namespace {
 // values outside the enums are invalid arguments.
 flagcxResult_t screen(int dtype, int op) {
   if (dtype < 0 || dtype >= flagcxNumTypes) return flagcxInvalidArgument;
+  if (op >= 0 && (op & FX_OP_ELEMENT_FOLD)) {   // the reference device kernel's own arithmetic, where it differs from the default
+    const int base = op & ~FX_OP_ELEMENT_FOLD;
+    if (base >= flagcxNumRedOps) return flagcxInvalidArgument;
+    const bool sixteen = dtype == flagcxFloat16 || dtype == flagcxBfloat16;
+    return (sixteen && (base == flagcxSum || base == flagcxMax || base == flagcxMin)) ? flagcxSuccess : flagcxNotSupported;
+  }
   if (op < 0 || op >= flagcxNumRedOps) return flagcxInvalidArgument;
   if (dtypeSize(dtype) == 0) return flagcxNotSupported;
   if (!opSupported(op)) return flagcxNotSupported;
@@ -25,6 +31,10 @@ flagcxResult_t screen(int dtype, int op) {
 }
 
 const KernelSet *setFor(int dtype, int op) {
+  if (op & FX_OP_ELEMENT_FOLD) {
+    const int base = op & ~FX_OP_ELEMENT_FOLD;
+    return &kernelSetsElem()[3 * (dtype == flagcxBfloat16) + (base == flagcxSum ? 0 : base == flagcxMax ? 1 : 2)];
+  }
   switch (dtype) {
     case flagcxFloat32: return &kernelSetsF32()[op];
     case flagcxInt32: return &kernelSetsI32()[op];

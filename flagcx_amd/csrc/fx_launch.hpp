@@ -276,5 +276,6 @@ const KernelSet *kernelSetsI64();
 const KernelSet *kernelSetsU64();
 const KernelSet *kernelSetsF64();
 const KernelSet *kernelSetsCopy();  // index log2(ES): 0 -> 1 byte, 1 -> 2, 2 -> 4
+const KernelSet *kernelSetsElem();  // RedElem: index 3 * (dtype == bf16) + (sum 0, max 1, min 2)
 
 }  // namespace fx

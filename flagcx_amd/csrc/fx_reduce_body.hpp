@@ -365,6 +365,57 @@ struct Red<flagcxFloat16, OP> {
   }
 };
 
+// The 16-bit types folded in the element type itself, as the reference's device
+// kernel does (custom_allreduce.cu:326-361: acc = reduceOp(acc, x) on half /
+// nv_bfloat16 values): a sum is rounded to 16 bits after every addition, and
+// max / min hand on the LATER operand unless the earlier one compares greater /
+// smaller (a > b ? a : b), so a NaN or a zero of the other sign replaces the
+// accumulator where the host rule keeps it.  Sum, max and min only, the ops
+// that kernel accepts.  The accumulator is the eight raw 16-bit patterns.
+template <int DT, int OP>
+struct RedElem {
+  static_assert(DT == flagcxFloat16 || DT == flagcxBfloat16, "16-bit element types only");
+  static_assert(OP == flagcxSum || OP == flagcxMax || OP == flagcxMin, "sum, max, min only");
+  static constexpr int ES = 2;
+  struct Acc {
+    uint32_t h[8];
+  };
+  static __device__ __forceinline__ float widen(uint32_t bits16) {
+    return DT == flagcxBfloat16 ? __uint_as_float(bits16 << 16) : halfToF32(bits16);
+  }
+  // One rounding per step: the hardware converters (round to nearest even; gfx950 has one for bf16 too), where
+  // the default reducer's single bf16 rounding is integer arithmetic.
+  static __device__ __forceinline__ uint32_t narrow(float f) {
+    return DT == flagcxBfloat16 ? (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f) : f32ToHalf(f);
+  }
+  static __device__ __forceinline__ uint32_t step(uint32_t a, uint32_t b) {
+    const float x = widen(a), y = widen(b);
+    if (OP == flagcxSum) return narrow(x + y);   // the exact sum of two 16-bit values, rounded once: what a native add gives
+    if (OP == flagcxMax) return (x > y) ? a : b;
+    return (x < y) ? a : b;
+  }
+  static __device__ __forceinline__ void init(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      c.h[2 * i] = v[i] & 0xffffu;
+      c.h[2 * i + 1] = v[i] >> 16;
+    }
+  }
+  static __device__ __forceinline__ void fold(Acc &c, u32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      c.h[2 * i] = step(c.h[2 * i], v[i] & 0xffffu);
+      c.h[2 * i + 1] = step(c.h[2 * i + 1], v[i] >> 16);
+    }
+  }
+  static __device__ __forceinline__ u32x4 finish(const Acc &c, uint32_t) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = (c.h[2 * i + 1] << 16) | (c.h[2 * i] & 0xffffu);
+    return r;
+  }
+};
+
 // Plain byte mover with ES-byte granularity (ES = 1, 2 or 4), used with k = 1
 // for the all-gather copy phase and the alltoallv pack / unpack.
 template <int ESZ>

@@ -96,6 +96,7 @@ struct Group {
   // configuration
   std::atomic<long long> sync{FX_SYNC_GROUP};   // read without the lock by a rank that marks its stream before posting
   long long algo = FX_ALGO_DIRECT, order = FX_ORDER_RANK;
+  long long arith = FX_ARITH_DEFAULT;
   long long nslices = 1, nredslices = 0, redslicesize = 65536;
   // scratch: ring reduce-scatter partials / alltoallv staging.  Outgrown
   // blocks stay allocated until the group is destroyed: kernels enqueued earlier
@@ -984,6 +985,14 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
     if (hipEventRecord(g->ready[r], s) != hipSuccess || hipStreamWaitEvent(c.s, g->ready[r], 0) != hipSuccess)
       res = flagcxUnhandledDeviceError;
   }
+  // The reference device kernel's own arithmetic for the 16-bit types, where asked for and where the schedule is
+  // that kernel's (every element folded over the ranks 0, 1, .., n-1 in one pass).
+  if (g->arith == FX_ARITH_ELEMENT && (dtype == flagcxFloat16 || dtype == flagcxBfloat16) &&
+      (op == flagcxSum || op == flagcxMax || op == flagcxMin) &&
+      (kind == kCustomAllReduce ||
+       ((kind == kAllReduce || kind == kReduce || kind == kReduceScatter) && g->algo == FX_ALGO_DIRECT &&
+        g->order == FX_ORDER_RANK)))
+    g->op = op | FX_OP_ELEMENT_FOLD;
   if (res == flagcxSuccess) {
     switch (kind) {
       case kAllReduce: res = runAllReduce(c); break;
@@ -1076,6 +1085,8 @@ flagcxResult_t newGroup(int nranks, Group **out) {
   if (g->nslices < 1) g->nslices = 1;
   if (g->nredslices < 0) g->nredslices = 0;
   if (g->redslicesize < 0) g->redslicesize = 0;
+  const char *arith = getenv("FX_SIM_ARITH");
+  if (arith && !strcmp(arith, "element")) g->arith = FX_ARITH_ELEMENT;
   const char *sync = getenv("FX_SIM_SYNC");
   if (sync && !strcmp(sync, "rendezvous")) g->sync = FX_SYNC_RENDEZVOUS;
   g->timeoutMs = envParam("FX_SIM_RENDEZVOUS_TIMEOUT_MS", 30000);
@@ -1453,6 +1464,10 @@ flagcxResult_t fxSimCommConfig(flagcxComm_t comm, int key, long long value) {
       if (value != FX_SYNC_GROUP && value != FX_SYNC_RENDEZVOUS) return flagcxInvalidArgument;
       if (g->nposted) return flagcxInvalidUsage;  // not while a collective is half posted
       g->sync = value;
+      break;
+    case FX_SIM_ARITH:
+      if (value != FX_ARITH_DEFAULT && value != FX_ARITH_ELEMENT) return flagcxInvalidArgument;
+      g->arith = value;
       break;
     case FX_SIM_SCRATCH_BYTES:  // reserve now what the scratch users would otherwise allocate at their first call
       if (value < 0) return flagcxInvalidArgument;

@@ -6,10 +6,11 @@ from . import _native as N
 
 lib = N.lib
 
-ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE, SYNC, SCRATCH_BYTES = 0, 1, 2, 3, 4, 5, 6
+ALGO, ORDER, NSLICES, NREDSLICES, REDSLICESIZE, SYNC, SCRATCH_BYTES, ARITH = 0, 1, 2, 3, 4, 5, 6, 7
 ALGO_DIRECT, ALGO_RING = 0, 1
 ORDER_RANK, ORDER_RING, ORDER_TREE, ORDER_HOST = 0, 1, 2, 3
 SYNC_GROUP, SYNC_RENDEZVOUS = 0, 1
+ARITH_DEFAULT, ARITH_ELEMENT = 0, 1
 
 
 def _szs(v):
@@ -24,9 +25,9 @@ class SimGroup:
         self.configure(**config)
 
     def configure(self, algo=None, order=None, nslices=None, nredslices=None, redslicesize=None, sync=None,
-                  scratch_bytes=None):
+                  scratch_bytes=None, arith=None):
         for key, val in ((ALGO, algo), (ORDER, order), (NSLICES, nslices), (NREDSLICES, nredslices),
-                         (REDSLICESIZE, redslicesize), (SYNC, sync), (SCRATCH_BYTES, scratch_bytes)):
+                         (REDSLICESIZE, redslicesize), (SYNC, sync), (SCRATCH_BYTES, scratch_bytes), (ARITH, arith)):
             if val is not None:
                 N.check(lib.fxSimCommConfig(self.comms[0], key, val), f"fxSimCommConfig({key})")
 

@@ -29,6 +29,21 @@ extern "C" {
 #define FX_MAX_SLICE_INPUTS 8 /* k accepted by the slice descriptors     */
 
 /*
+ * Added to a reduction op (flagcxSum | FX_OP_ELEMENT_FOLD, also flagcxMax,
+ * flagcxMin) for flagcxFloat16 / flagcxBfloat16: fold in the element type
+ * itself, as the reference's device kernel does (reduceOp on half /
+ * nv_bfloat16, flagcx/adaptor/kernel/nvidia/custom_allreduce.cu:326-361).  A
+ * sum is then rounded to 16 bits after every addition instead of once at the
+ * end, and max / min are a > b ? a : b / a < b ? a : b with a the accumulator:
+ * on a tie (+0 and -0) or an unordered pair (NaN) the LATER operand is handed
+ * on.  Any other type or op with the flag is flagcxNotSupported, as in that
+ * kernel's dispatch (:498-518); for fp32 / fp64 sums the default arithmetic is
+ * that kernel's already.  Accepted wherever a dtype / op pair is, except in
+ * reduce triggers, whose op field has four bits.
+ */
+#define FX_OP_ELEMENT_FOLD 0x100
+
+/*
  * k-way element-wise reduce-copy over peer buffers:
  *   out[i] = in[first][i] (op) in[(first+1)%k][i] (op) ... left to right.
  * Replaces lsa_reduce + flagcxLsaAllReduceKernel

@@ -106,7 +106,18 @@ enum {
   FX_SIM_NREDSLICES = 3,   /* FLAGCX_UNIRUNNER_NREDSLICES (0 = automatic) */
   FX_SIM_REDSLICESIZE = 4, /* FLAGCX_UNIRUNNER_REDSLICESIZE (65536 elems) */
   FX_SIM_SYNC = 5,         /* FX_SYNC_*; environment FX_SIM_SYNC=group|rendezvous */
-  FX_SIM_SCRATCH_BYTES = 6 /* reserve at least this much scratch now            */
+  FX_SIM_SCRATCH_BYTES = 6, /* reserve at least this much scratch now           */
+  FX_SIM_ARITH = 7         /* FX_ARITH_*; environment FX_SIM_ARITH=element      */
+};
+/* How fp16 / bf16 sums, maxima and minima are folded by flagcxAllReduce, flagcxReduce, flagcxReduceScatter (direct
+ * algorithm, rank order) and flagcxCustomAllReduceImpl. */
+enum {
+  FX_ARITH_DEFAULT = 0, /* widen to fp32, accumulate, round once; max / min keep
+                           the earlier operand on ties and NaN (std::max / min) */
+  FX_ARITH_ELEMENT = 1  /* in the element type, as the reference's device kernel
+                           does (custom_allreduce.cu:326-361): rounded after every
+                           addition, a > b ? a : b (FX_OP_ELEMENT_FOLD of
+                           fx_kernels.h)                                        */
 };
 enum {
   FX_SYNC_GROUP = 0,

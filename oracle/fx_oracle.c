@@ -31,6 +31,15 @@
  *       its own host path, service/bootstrap.cc:872-874); defined as the sum
  *       divided once by k (IEEE division before the final rounding; C division
  *       of the wrapped sum for integers) and checked against numpy only.
+ *   oracle_reduce_copy_elem (16-bit types folded in the element type, the
+ *       reference device kernel's own arithmetic) .. hand-derived cases where
+ *       rounding after every addition and rounding once differ (bf16 256+1+1,
+ *       fp16 2048+1+1), the order of its steps on a non-associative triple, its
+ *       a > b ? a : b rule on +0 / -0 and on NaN in every position of a triple
+ *       (worked out from custom_allreduce.cu:326-334 by hand); k = 2 sums equal
+ *       the pinned oracle_reduce_copy (one rounding either way); every step is
+ *       numpy's float16 addition for fp16.  The NaN PAYLOAD a sum produces is
+ *       unpinned (the reference's comes from the GPU's converter).
  *   oracle_split / plans ...................... tiling invariants + closed
  *       forms of the reference's divisible cases.
  *   oracle_tree_reduce ........................ hand-derived associations for
@@ -299,6 +308,46 @@ int oracle_reduce_copy(void *out, const void *const *in, int k, size_t count,
         o[i] = hb;
       }
     }
+  }
+  return RC_OK;
+}
+
+/*
+ * The reference device kernel's own arithmetic for the 16-bit types
+ * (adaptor/kernel/nvidia/custom_allreduce.cu:326-361): lsa_reduce keeps the
+ * accumulator in the element type, acc = reduceOp(acc, x), with
+ *   sum: a + b on half / nv_bfloat16 -- the exact sum rounded to 16 bits, at
+ *        every step;
+ *   max: a > b ? a : b,  min: a < b ? a : b  -- on a tie or an unordered pair
+ *        the later operand b is handed on.
+ * Peers are folded 0, 1, .., k-1 (rotated by `first` like oracle_reduce_copy).
+ * Only what that kernel's dispatch accepts (:498-518): fp16 / bf16 with sum,
+ * max, min.
+ */
+int oracle_reduce_copy_elem(void *out, const void *const *in, int k, size_t count, int dtype, int op, int first) {
+  if (dtype != DT_FP16 && dtype != DT_BF16) return RC_UNSUPPORTED;
+  if (op != OP_SUM && op != OP_MAX && op != OP_MIN) return RC_UNSUPPORTED;
+  if (k < 1 || first < 0 || first >= k) return RC_INVALID;
+  const int bf = (dtype == DT_BF16);
+  uint16_t *o = (uint16_t *)out;
+  for (size_t i = 0; i < count; i++) {
+    uint16_t a = ((const uint16_t *)in[first])[i];
+    for (int j = 1; j < k; j++) {
+      const uint16_t b = ((const uint16_t *)in[(first + j) % k])[i];
+      const float x = bf ? oracle_bf16_to_f32(a) : oracle_f16_to_f32(a);
+      const float y = bf ? oracle_bf16_to_f32(b) : oracle_f16_to_f32(b);
+      if (op == OP_SUM) {
+        /* both operands have at most 11 significant bits, so the float sum is the exact sum (or differs from it
+         * far below half a 16-bit ulp) and one rounding of it is the native 16-bit addition */
+        const float s = x + y;
+        a = bf ? oracle_f32_to_bf16(s) : oracle_f32_to_f16(s);
+      } else if (op == OP_MAX) {
+        a = (x > y) ? a : b;
+      } else {
+        a = (x < y) ? a : b;
+      }
+    }
+    o[i] = a;
   }
   return RC_OK;
 }

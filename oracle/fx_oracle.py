@@ -29,6 +29,8 @@ class RedNode(C.Structure):
 
 lib.oracle_reduce_copy.restype = _i
 lib.oracle_reduce_copy.argtypes = [_vp, C.POINTER(_vp), _i, _sz, _i, _i, _i]
+lib.oracle_reduce_copy_elem.restype = _i
+lib.oracle_reduce_copy_elem.argtypes = [_vp, C.POINTER(_vp), _i, _sz, _i, _i, _i]
 lib.oracle_reduce2.restype = _i
 lib.oracle_reduce2.argtypes = [_vp, _vp, _vp, _sz, _i, _i]
 lib.oracle_host_ring_passes.restype = _i
@@ -90,6 +92,16 @@ def reduce_copy(ins, dtype, op, first=0, out=None):
     rc = lib.oracle_reduce_copy(out.ctypes.data, _ptrs(ins), len(ins), ins[0].size, dtype, op, first)
     if rc:
         raise ValueError(f"oracle_reduce_copy rc={rc}")
+    return out
+
+
+def reduce_copy_elem(ins, dtype, op, first=0):
+    """16-bit types folded in the element type itself (the reference device kernel's arithmetic); uint16 arrays."""
+    ins = [np.ascontiguousarray(a) for a in ins]
+    out = np.empty_like(ins[0])
+    rc = lib.oracle_reduce_copy_elem(out.ctypes.data, _ptrs(ins), len(ins), ins[0].size, dtype, op, first)
+    if rc:
+        raise ValueError(f"oracle_reduce_copy_elem rc={rc}")
     return out
 
 

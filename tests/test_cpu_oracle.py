@@ -627,3 +627,81 @@ def test_trigger_layout_constants():
     # fields are masked, not allowed to spill into their neighbours
     v = O.trigger_encode(0, 0, 0, 2**40 - 1, 2**20 - 1, 31, 31, 7)
     assert v[3] == 0xffffffff | (0xffff << 32) | (0xf << 48) | (0xf << 52) | (0x3 << 56)
+
+
+# --- the reference device kernel's own 16-bit arithmetic (custom_allreduce.cu:326-361) -----------------------------
+
+BF = lambda *v: [np.array([x], np.uint16) for x in v]            # one element per input, given as bit patterns
+
+
+def test_element_fold_rounds_after_every_addition():
+    """bf16 has 8 significant bits: 256 + 1 = 257 is a tie between 256 and 258
+    and goes to the even one, 256, and so does the next + 1; rounding once gives
+    258.  fp16 has 11: the same with 2048 and 2050.  Worked out by hand."""
+    b256, b1, b258, b2 = 0x4380, 0x3F80, 0x4381, 0x4000
+    assert O.reduce_copy_elem(BF(b256, b1, b1), BF16, SUM)[0] == b256
+    assert O.reduce_copy(BF(b256, b1, b1), BF16, SUM)[0] == b258          # the default arithmetic
+    h2048, h1, h2050 = 0x6800, 0x3C00, 0x6801
+    assert O.reduce_copy_elem(BF(h2048, h1, h1), F16, SUM)[0] == h2048
+    assert O.reduce_copy(BF(h2048, h1, h1), F16, SUM)[0] == h2050
+    # the steps run left to right from `first`: 1 + 1 = 2, 2 + 256 = 258 exactly; 256 + 1 first loses both ones
+    assert O.reduce_copy_elem(BF(b1, b1, b256), BF16, SUM)[0] == b258
+    assert O.reduce_copy_elem(BF(b256, b1, b1), BF16, SUM, first=1)[0] == b258
+    assert O.reduce_copy_elem(BF(b1, b256, b1), BF16, SUM)[0] == b256
+    assert O.reduce_copy_elem(BF(b1, b1), BF16, SUM)[0] == b2
+
+
+@pytest.mark.parametrize("dtype", [BF16, F16])
+def test_element_fold_max_min_hand_on_the_later_operand(dtype):
+    """a > b ? a : b with a the accumulator (custom_allreduce.cu:329-331): a
+    tie or an unordered pair yields b.  Every case below is that rule applied by
+    hand; the host rule (std::max, the default here) gives the other answer
+    wherever the comment says so."""
+    if dtype == BF16:
+        one, two, three, five, pz, nz, nan = 0x3F80, 0x4000, 0x4040, 0x40A0, 0x0000, 0x8000, 0x7FC0
+    else:
+        one, two, three, five, pz, nz, nan = 0x3C00, 0x4000, 0x4200, 0x4500, 0x0000, 0x8000, 0x7E00
+    e = lambda op, *v: int(O.reduce_copy_elem(BF(*v), dtype, op)[0])
+    d = lambda op, *v: int(O.reduce_copy(BF(*v), dtype, op)[0])
+    assert e(MAX, pz, nz) == nz and d(MAX, pz, nz) == pz          # +0 > -0 is false: the later one
+    assert e(MAX, nz, pz) == pz and d(MAX, nz, pz) == nz
+    assert e(MIN, nz, pz) == pz and e(MIN, pz, nz) == nz
+    assert e(MAX, one, nan, pz) == pz and d(MAX, one, nan, pz) == one      # 1 -> NaN -> 0: the NaN resets the fold
+    assert e(MAX, nan, three, five) == five and d(MAX, nan, three, five) == nan
+    assert e(MAX, one, two, nan) == nan and d(MAX, one, two, nan) == two
+    assert e(MIN, one, nan, five) == five and e(MIN, five, three, nan) == nan
+    assert e(MAX, one, five, three) == five and e(MIN, five, one, three) == one     # ordered values: plain max / min
+    with pytest.raises(ValueError):
+        O.reduce_copy_elem(BF(one, two), dtype, PROD)
+    with pytest.raises(ValueError):
+        O.reduce_copy_elem([np.ones(3, np.float32)] * 2, F32, SUM)
+
+
+@pytest.mark.parametrize("dtype", [BF16, F16])
+def test_element_fold_steps_are_single_correctly_rounded_additions(dtype):
+    """Two inputs: one addition, one rounding -- the pinned default oracle's
+    answer.  More inputs, fp16: every step is numpy's float16 addition."""
+    rng = np.random.default_rng(7)
+    n = 200000
+    if dtype == F16:
+        ins = [(rng.standard_normal(n) * 10 ** rng.uniform(-4, 4, n)).astype(np.float16).view(np.uint16) for _ in range(5)]
+    else:
+        ins = [((rng.standard_normal(n) * 10 ** rng.uniform(-6, 6, n)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+               for _ in range(5)]
+    assert np.array_equal(O.reduce_copy_elem(ins[:2], dtype, SUM), O.reduce_copy(ins[:2], dtype, SUM))
+    if dtype == F16:
+        with np.errstate(over="ignore", invalid="ignore"):
+            acc = ins[0].view(np.float16)
+            for x in ins[1:]:
+                acc = acc + x.view(np.float16)
+        got = O.reduce_copy_elem(ins, dtype, SUM).view(np.float16)
+        same = (got.view(np.uint16) == acc.view(np.uint16)) | (np.isnan(got) & np.isnan(acc))
+        assert same.all()
+    else:   # bf16: a second, arithmetic rounding of each exact step (float64 holds the sum of two bf16 values exactly)
+        acc = (ins[0].astype(np.uint32) << 16).view(np.float32)
+        for x in ins[1:]:
+            exact = acc.astype(np.float64) + (x.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+            m, ex = np.frexp(exact)                            # exact = m * 2**ex, 0.5 <= |m| < 1: keep 8 significant bits
+            acc = np.ldexp(np.rint(m * 256.0), ex - 8).astype(np.float32)      # rint is round-half-even
+        got = (O.reduce_copy_elem(ins, dtype, SUM).astype(np.uint32) << 16).view(np.float32)
+        assert np.array_equal(got, acc)

@@ -9,7 +9,7 @@ import pytest
 from flagcx_amd import _native as N
 from flagcx_amd import sim as S
 from oracle import fx_oracle as O
-from tests.util import DTYPES, DevBufs, assert_parity, seeded_inputs
+from tests.util import DTYPES, DevBufs, assert_parity, is_nan16, seeded_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -852,3 +852,61 @@ def test_rendezvous_mode_with_busy_streams_and_no_host_waits(dev):
             t.join(timeout=100)
         assert not any(t.is_alive() for t in threads)
         assert not errors, errors[:6]
+
+
+@pytest.mark.parametrize("dname", ["bf16", "fp16"])
+def test_element_arithmetic_mode_reproduces_the_reference_device_kernel(dev, stream, dname):
+    """FX_SIM_ARITH = element: the all-reduce, reduce, reduce-scatter and the
+    custom all-reduce hook fold fp16 / bf16 the way lsa_reduce does
+    (custom_allreduce.cu:326-361) -- rounded after every addition, max / min
+    handing on the later operand -- bit for bit against the oracle's
+    restatement; the default mode keeps this build's own contract."""
+    dtype = DTYPES[dname]
+    n, count = 8, 8 * 12501
+    nanbits = 0x7FC0 if dname == "bf16" else 0x7E00
+    rng = np.random.default_rng(3)
+    sends = seeded_inputs(dtype, n, count, seed=21, dist=(0.0, 300.0))
+    for a in sends:
+        where = rng.random(count) < 0.01
+        a[where] = rng.choice(np.array([0x0000, 0x8000, nanbits], np.uint16), int(where.sum()))
+    for op in (N.OP_SUM, N.OP_MAX, N.OP_MIN):
+        want = O.reduce_copy_elem(sends, dtype, op)
+        plain = O.reduce_copy(sends, dtype, op)
+        assert (want != plain).sum() > 100
+        nan = (lambda a: is_nan16(a, dtype)) if op == N.OP_SUM else (lambda a: np.zeros(a.shape, bool))
+
+        def same(got, ref, what):
+            assert np.array_equal(nan(got), nan(ref)) and np.array_equal(got[~nan(got)], ref[~nan(ref)]), what
+
+        for arith, ref in ((S.ARITH_ELEMENT, want), (S.ARITH_DEFAULT, plain)):
+            with DevBufs(dev) as b, S.SimGroup(n, arith=arith) as g:
+                ds = [b.put(a) for a in sends]
+                dr = [b.alloc(count * 2) for _ in range(n)]
+                N.check(g.all_reduce(ds, dr, count, dtype, op, stream), "flagcxAllReduce")
+                dev.stream_sync(stream)
+                for r in range(n):
+                    same(dev.to_host(dr[r], count, np.uint16), ref, f"all-reduce {dname} op={op} arith={arith} rank {r}")
+                if arith == S.ARITH_DEFAULT:
+                    continue
+                rc = count // n
+                N.check(g.reduce_scatter(ds, dr, rc, dtype, op, stream), "flagcxReduceScatter")
+                N.check(g.reduce(ds, [dr[r] + rc * 2 if r == 5 else None for r in range(n)], count - rc, dtype, op, 5, stream),
+                        "flagcxReduce")
+                dev.stream_sync(stream)
+                for r in range(n):
+                    same(dev.to_host(dr[r], rc, np.uint16), want[r * rc:(r + 1) * rc], f"reduce-scatter rank {r}")
+                same(dev.to_host(dr[5] + rc * 2, count - rc, np.uint16), want[:count - rc], "reduce to rank 5")
+                # the hook, on registered windows
+                win = [b.alloc(count * 2) for _ in range(n)]
+                N.check(g.register_windows(win, count * 2), "fxSimRegisterWindows")
+                N.check(g.custom_all_reduce(ds, dr, count, dtype, op, stream), "flagcxCustomAllReduceImpl")
+                dev.stream_sync(stream)
+                for r in (0, n - 1):
+                    same(dev.to_host(dr[r], count, np.uint16), want, f"custom all-reduce rank {r}")
+                # the ring order is not that kernel's schedule: the mode leaves it alone
+                g.configure(order=S.ORDER_RING)
+                N.check(g.all_reduce(ds, dr, count, dtype, op, stream), "flagcxAllReduce")
+                dev.stream_sync(stream)
+                ring = np.concatenate([O.reduce_copy([a[lo:hi] for a in sends], dtype, op, first=c)
+                                       for c, (lo, hi) in enumerate((c * rc, (c + 1) * rc) for c in range(n))])
+                assert_parity(dev.to_host(dr[0], count, np.uint16), ring, dtype, op, "ring order keeps the default arithmetic")

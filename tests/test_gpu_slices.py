@@ -7,7 +7,7 @@ import pytest
 from flagcx_amd import _native as N
 from flagcx_amd import kernels as K
 from oracle import fx_oracle as O
-from tests.util import DTYPES, OPS, DevBufs, assert_parity, seeded_inputs
+from tests.util import DTYPES, OPS, DevBufs, assert_parity, is_nan16, seeded_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -443,3 +443,71 @@ def test_more_slices_than_one_kernel_argument_table_holds(dev):
     want = full.reshape(nsl, seg + gap).copy()
     want[:, seg:] = 0
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("dname", ["bf16", "fp16"])
+def test_element_fold_is_the_reference_device_kernels_arithmetic(dev, dname):
+    """op | FX_OP_ELEMENT_FOLD: the 16-bit types folded in the element type, as
+    lsa_reduce does (custom_allreduce.cu:326-361) -- rounded after every
+    addition, max / min handing on the later operand on ties and NaN.  Bit for
+    bit against the oracle's restatement (NaN for NaN where a sum makes one),
+    through the direct kernel, the slice table, the multi-output kernel and the
+    run-time-k kernels; specials sprinkled over random data."""
+    dtype = DTYPES[dname]
+    ELEM = 0x100
+    rng = np.random.default_rng(11)
+    specials = np.array([0x0000, 0x8000, 0x7FC0 if dname == "bf16" else 0x7E00, 0x7F80 if dname == "bf16" else 0x7C00,
+                         0xFF80 if dname == "bf16" else 0xFC00, 0x0001, 0x8001, 0x4380, 0x3F80, 0x6800, 0x3C00], np.uint16)
+
+    def inputs(k, n, seed):
+        ins = seeded_inputs(dtype, k, n, seed=seed, dist=(0.0, 300.0))      # large enough that step rounding shows
+        for a in ins:
+            where = rng.random(n) < 0.02
+            a[where] = rng.choice(specials, int(where.sum()))
+        return ins
+
+    def same(got, want, op, what):
+        if op == N.OP_SUM:
+            gn, wn = is_nan16(got, dtype), is_nan16(want, dtype)
+            assert np.array_equal(gn, wn), f"{what}: NaN positions differ"
+            assert np.array_equal(got[~gn], want[~wn]), what
+        else:
+            assert np.array_equal(got, want), what
+
+    differs = 0
+    for op in (N.OP_SUM, N.OP_MAX, N.OP_MIN):
+        for k, n, first, mis in [(1, 1001, 0, 0), (2, 40001, 1, 1), (3, 7, 2, 0), (5, 300007, 0, 3), (8, 1 << 20, 5, 0),
+                                 (12, 70001, 7, 1), (33, 4099, 0, 0)]:
+            ins = inputs(k, n, seed=k * 10 + op)
+            want = O.reduce_copy_elem(ins, dtype, op, first=first)
+            differs += int((want != O.reduce_copy(ins, dtype, op, first=first)).sum())
+            with DevBufs(dev) as b:
+                dins = [b.put(a, pad_before=mis * 2) for a in ins]
+                out = b.alloc(n * 2 + 64)
+                N.check(K.reduce_copy(out, dins, n, dtype, op | ELEM, first), f"fx_reduce_copy k={k}")
+                dev.sync()
+                same(dev.to_host(out, n, np.uint16), want, op, f"{dname} op={op} k={k} n={n} direct")
+                if k <= 8:                                   # the slice table and the multi-output kernel, in two pieces
+                    rot = [dins[(first + j) % k] for j in range(k)]
+                    cut = n // 3
+                    outs = [b.alloc(n * 2 + 64) for _ in range(3)]
+                    descs = [(rot, outs[0], cut), ([p + cut * 2 for p in rot], outs[0] + cut * 2, n - cut)]
+                    N.check(K.reduce_slices(descs, k, dtype, op | ELEM), "fx_reduce_slices")
+                    bd = [(rot, outs[1:], cut), ([p + cut * 2 for p in rot], [o + cut * 2 for o in outs[1:]], n - cut)]
+                    N.check(K.reduce_bcast_slices(bd, k, 2, dtype, op | ELEM), "fx_reduce_bcast_slices")
+                    dev.sync()
+                    for o in outs:
+                        same(dev.to_host(o, n, np.uint16), want, op, f"{dname} op={op} k={k} slices / bcast")
+                else:
+                    outs = [b.alloc(n * 2 + 64) for _ in range(k)]
+                    N.check(K.reduce_bcast(outs, dins, n, dtype, op | ELEM, first), "fx_reduce_bcast")
+                    dev.sync()
+                    for o in outs[:: max(k // 3, 1)]:
+                        same(dev.to_host(o, n, np.uint16), want, op, f"{dname} op={op} k={k} run-time k")
+    assert differs > 1000, "the inputs never showed the difference from the default arithmetic"
+    # what the reference kernel's dispatch refuses (custom_allreduce.cu:498-518)
+    assert K.reduce_copy(16, [16, 32], 4, dtype, N.OP_PROD | ELEM) == N.NOT_SUPPORTED
+    assert K.reduce_copy(16, [16, 32], 4, dtype, N.OP_AVG | ELEM) == N.NOT_SUPPORTED
+    assert K.reduce_copy(16, [16, 32], 4, N.DT_FP32, N.OP_MAX | ELEM) == N.NOT_SUPPORTED
+    assert K.reduce_copy(16, [16, 32], 4, N.DT_INT32, N.OP_SUM | ELEM) == N.NOT_SUPPORTED
+    assert K.reduce_copy(16, [16, 32], 4, dtype, 7 | ELEM) == N.INVALID_ARGUMENT

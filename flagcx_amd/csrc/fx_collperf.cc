@@ -10,7 +10,7 @@
 // Elapsed time: .. Algo bandwidth: .. Bus bandwidth: .."; the bus factors of
 // test/perf/host_api/test_*.cpp), so a sweep made with those programs and a
 // sweep made here can be laid side by side.  Added here: -N ranks (default 8),
-// -A direct|ring, -O rank|ring|host, -c 1 to check every rank's result after the
+// -A direct|ring, -O rank|ring|host, -a default|element, -c 1 to check every rank's result after the
 // timed loop (long results by sample), and a second figure per line: the bytes the GPU's memory moved
 // for one collective, divided by the time between two device events around
 // the timed calls.
@@ -134,6 +134,7 @@ struct Options {
   int factor = 2, warmup = 5, iters = 20, root = 0, nranks = 8, check = 0;
   int type = 7 /* float */, op = 0;
   int algo = -1, order = -1;
+  int arith = -1;    // -a element: fp16 / bf16 folded in the element type, as the reference's device kernel does
   int threads = 0;   // -T 1: one host thread and one stream per rank, calls that block until every rank has posted
 };
 
@@ -142,7 +143,8 @@ void usage(const char *argv0) {
          "[-b <minbytes K/M/G>] [-e <maxbytes K/M/G>] [-f <stepfactor>] [-w <warmupiters>] [-n <iters>]\n\t"
          "[-r <root>] [-o <sum|prod|max|min|avg>] [-d <int8|uint8|int32|uint32|int64|uint64|half|float|double|bfloat16>]\n\t"
          "[-N <simulated ranks, 1..64>] [-A <direct|ring>] [-O <rank|ring|host>] [-c <check 0/1>]\n\t"
-         "[-T <0: one thread posts every rank on one stream | 1: a thread and a stream per rank>]\n",
+         "[-T <0: one thread posts every rank on one stream | 1: a thread and a stream per rank>]\n\t"
+         "[-a <default|element: how fp16 / bf16 are folded>]\n",
          argv0);
 }
 
@@ -166,10 +168,10 @@ Options parse(int argc, char **argv) {
                               {"op", required_argument, 0, 'o'}, {"datatype", required_argument, 0, 'd'},
                               {"nranks", required_argument, 0, 'N'}, {"algo", required_argument, 0, 'A'},
                               {"order", required_argument, 0, 'O'}, {"check", required_argument, 0, 'c'},
-                              {"threads", required_argument, 0, 'T'},
+                              {"threads", required_argument, 0, 'T'}, {"arith", required_argument, 0, 'a'},
                               {"help", no_argument, 0, 'h'}, {}};
   optind = 2;
-  for (int c; (c = getopt_long(argc, argv, "b:e:f:w:n:r:o:d:N:A:O:c:T:h", longOpts, nullptr)) != -1;) {
+  for (int c; (c = getopt_long(argc, argv, "b:e:f:w:n:r:o:d:N:A:O:c:T:a:h", longOpts, nullptr)) != -1;) {
     const std::string a = optarg ? optarg : "";
     bool bad = false;
     switch (c) {
@@ -181,6 +183,7 @@ Options parse(int argc, char **argv) {
       case 'r': o.root = atoi(optarg); break;
       case 'N': o.nranks = atoi(optarg); bad = o.nranks < 1 || o.nranks > 64; break;
       case 'c': o.check = atoi(optarg); break;
+      case 'a': o.arith = a == "default" ? FX_ARITH_DEFAULT : a == "element" ? FX_ARITH_ELEMENT : -1; bad = o.arith < 0; break;
       case 'T': o.threads = atoi(optarg); bad = o.threads != 0 && o.threads != 1; break;
       case 'o':
         bad = true;
@@ -391,6 +394,7 @@ int main(int argc, char **argv) {
   OK(fxSimCommInitAll(run.comms.data(), n));
   if (run.o.algo >= 0) OK(fxSimCommConfig(run.comms[0], FX_SIM_ALGO, run.o.algo));
   if (run.o.order >= 0) OK(fxSimCommConfig(run.comms[0], FX_SIM_ORDER, run.o.order));
+  if (run.o.arith >= 0) OK(fxSimCommConfig(run.comms[0], FX_SIM_ARITH, run.o.arith));
   OK(dev->streamCreate(&run.stream));
   run.streams.assign(n, run.stream);
   if (run.o.threads) {

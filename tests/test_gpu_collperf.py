@@ -42,6 +42,8 @@ def test_tool_moves_narrow_types_and_reports_what_it_cannot_check():
     assert "# check: every rank's result as expected" in out
     out = run("allreduce", "-b", "64K", "-e", "64K", "-d", "half", "-c", "1", "-n", "2")
     assert "no check for this datatype / op" in out
+    out = run("allreduce", "-b", "1M", "-e", "1M", "-d", "bfloat16", "-a", "element", "-n", "3")
+    assert len([ln for ln in out.splitlines() if ln.startswith("Comm size:")]) == 1
     bad = subprocess.run([TOOL, "allreduce", "-N", "65"], capture_output=True, text=True, timeout=60)
     assert bad.returncode == 1 and "bad value for -N" in bad.stderr
     bad = subprocess.run([TOOL, "allsomething"], capture_output=True, text=True, timeout=60)

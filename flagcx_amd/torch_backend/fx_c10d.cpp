@@ -237,6 +237,16 @@ class FxBackend : public c10d::Backend {
 
   const std::string getBackendName() const override { return "flagcx"; }
 
+  // A coalescing bracket is the library's group bracket (the reference's backend does the same,
+  // backend_flagcx.cpp:525-537): sends and recvs that meet inside it leave as one copy launch when it closes.
+  // What torch.distributed.batch_isend_irecv uses.
+  bool supportsCoalescing() const override { return true; }
+  void startCoalescing() override { ok(flagcxGroupStart(comm_), "flagcxGroupStart"); }
+  c10::intrusive_ptr<Work> endCoalescing() override {
+    ok(flagcxGroupEnd(comm_), "flagcxGroupEnd");
+    return c10::make_intrusive<FxWork>(getRank(), OpType::COALESCED, c10::hip::getCurrentHIPStream().stream(), Tensors{});
+  }
+
   c10::intrusive_ptr<Work> allreduce(Tensors &tensors, const c10d::AllreduceOptions &opts) override {
     checkOne(tensors, "allreduce");
     at::Tensor &t = tensors[0];

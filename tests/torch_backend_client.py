@@ -172,6 +172,19 @@ def simulated(n, gen):
     wait_all([b.barrier() for b in ranks])
     print("ok  gather, scatter, send / recv, barrier", flush=True)
 
+    # a coalescing bracket per rank (what batch_isend_irecv opens): the ring exchange, every rank sends right, receives left
+    msgs = [make(torch.float32, (4099,), gen) for _ in range(n)]
+    boxes = [torch.empty(4099, device="cuda") for _ in range(n)]
+    works = []
+    for r, b in enumerate(ranks):
+        b._start_coalescing()
+        b.send([msgs[r]], (r + 1) % n, 0)
+        b.recv([boxes[r]], (r - 1) % n, 0)
+        works.append(b._end_coalescing())
+    wait_all(works)
+    assert all(torch.equal(boxes[r], msgs[(r - 1) % n]) for r in range(n))
+    print("ok  send / recv inside coalescing brackets", flush=True)
+
     # coalesced forms: one collective over all the tensors of the call, so that rank after rank can post them
     shapes = [(1001,), (3, 333), (70001,), (16,)]
     tl = [[make(torch.float32, sh, gen) for sh in shapes] for _ in range(n)]
@@ -255,6 +268,16 @@ def one_rank(gen):
         dist.barrier()
         torch.cuda.synchronize()
         assert torch.equal(t, keep)
+        # batched point-to-point (a coalescing bracket) and the coalescing manager around collectives
+        box = torch.empty_like(t)
+        for w in dist.batch_isend_irecv([dist.P2POp(dist.isend, t, 0), dist.P2POp(dist.irecv, box, 0)]):
+            w.wait()
+        a, b2 = t.clone(), t[:77].clone()
+        with dist._coalescing_manager(device=torch.device("cuda")):
+            dist.all_reduce(a)
+            dist.all_reduce(b2)
+        torch.cuda.synchronize()
+        assert torch.equal(box, keep) and torch.equal(a, keep) and torch.equal(b2, keep[:77])
         # DistributedDataParallel: parameter broadcast, shape check and gradient buckets all go through the backend
         torch.manual_seed(0)
         model = torch.nn.Sequential(torch.nn.Linear(64, 128), torch.nn.ReLU(), torch.nn.Linear(128, 8)).cuda()

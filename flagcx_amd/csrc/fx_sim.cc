@@ -12,9 +12,11 @@
 // the reference would receive a copy of it.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -719,10 +721,47 @@ flagcxResult_t runAlltoAllv(const Ctx &c) {
     base[r + 1] = base[r] + ((tot * ts + 255) & ~(size_t)255);
   }
   if (base[n] == 0) return flagcxSuccess;
+  // Does any receive segment overlap any send segment?  First by rank: the span of all a rank sends against the
+  // span of all a rank receives (n * n pairs instead of one per pair of segments); only where two spans meet, by
+  // segment, in address order.
   bool overlap = false;
-  for (size_t a = 0; a < recvR.size() && !overlap; a++)
-    for (size_t b = 0; b < sendR.size() && !overlap; b++)
-      overlap = recvR[a].lo < sendR[b].hi && sendR[b].lo < recvR[a].hi;
+  {
+    std::vector<Range> sendSpan(n, Range{UINTPTR_MAX, 0}), recvSpan(n, Range{UINTPTR_MAX, 0});
+    size_t at = 0;
+    for (int r = 0; r < n; r++)
+      for (int i = 0; i < n; i++) {
+        if (!g->posts[r].sendcounts[i]) continue;
+        const Range &sr = sendR[at], &rr = recvR[at];   // pushed pairwise above: rank r's segment for rank i, and where it lands
+        at++;
+        sendSpan[r].lo = std::min(sendSpan[r].lo, sr.lo);
+        sendSpan[r].hi = std::max(sendSpan[r].hi, sr.hi);
+        recvSpan[i].lo = std::min(recvSpan[i].lo, rr.lo);
+        recvSpan[i].hi = std::max(recvSpan[i].hi, rr.hi);
+      }
+    bool spansMeet = false;
+    for (int r = 0; r < n && !spansMeet; r++)
+      for (int i = 0; i < n && !spansMeet; i++)
+        spansMeet = recvSpan[i].lo < sendSpan[r].hi && sendSpan[r].lo < recvSpan[i].hi;
+    if (spansMeet) {
+      struct Tagged {
+        uintptr_t lo, hi;
+        int recv;
+      };
+      std::vector<Tagged> all;
+      all.reserve(sendR.size() + recvR.size());
+      for (const Range &x : sendR) all.push_back(Tagged{x.lo, x.hi, 0});
+      for (const Range &x : recvR) all.push_back(Tagged{x.lo, x.hi, 1});
+      std::sort(all.begin(), all.end(), [](const Tagged &a, const Tagged &b) { return a.lo < b.lo; });
+      uintptr_t reach[2] = {0, 0};   // how far the segments of either kind seen so far extend
+      for (const Tagged &x : all) {
+        if (reach[1 - x.recv] > x.lo) {
+          overlap = true;
+          break;
+        }
+        reach[x.recv] = std::max(reach[x.recv], x.hi);
+      }
+    }
+  }
   if (!overlap) {
     SliceList direct;
     for (size_t a = 0; a < recvR.size(); a++)

@@ -762,7 +762,18 @@ __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
     return ldg_stream(sg.inp(p) + j * 16);
   };
   R::init(acc, fetch(0));
-  for (int p = 1; p < k; p++) R::fold(acc, fetch(p));
+  // Sixteen inputs in flight at a time, folded in their order: a launch smaller than one full tile comes through
+  // here, and with a run-time k nothing else overlaps the loads -- one after the other they cost 0.3 us per input.
+  constexpr int kGroup = 16;
+  int p = 1;
+  for (; p + kGroup <= k; p += kGroup) {
+    u32x4 v[kGroup];
+#pragma unroll
+    for (int q = 0; q < kGroup; q++) v[q] = fetch(p + q);
+#pragma unroll
+    for (int q = 0; q < kGroup; q++) R::fold(acc, v[q]);
+  }
+  for (; p < k; p++) R::fold(acc, fetch(p));
   u32x4 r = R::finish(acc, (uint32_t)k);
   if (full)
     storeVector(sg, j * 16, r);

@@ -13,6 +13,9 @@ namespace fx {
 //    workgroups than the device has compute units and each lane waits for 32
 //    loads: an eight-input reduction of 1 MiB per input takes 4.8 us against
 //    2.9 us, the eight-rank all-reduce of 64 KiB per rank 6.2 against 4.3 us.
+//    The run-time-k kernels (nine inputs and more, 2 otherwise) likewise: the
+//    all-reduce of 16 KiB per rank over 12 / 16 / 32 ranks 5.0 / 5.8 / 10.4
+//    against 4.0 / 4.5 / 8.2 us.
 //  * Larger launches: 4 (2 for one and two inputs); 8 for 8 inputs once the
 //    launch is large enough not to miss the extra workgroups and every input is
 //    aligned like the output (256 VGPRs; unaligned: 4 is 7-10 % faster).  Between
@@ -22,7 +25,7 @@ namespace fx {
 //    pack / unpack and four-input sums from 8 MiB to 1 GiB, and 0.5-1 % in favour
 //    of 4 over 1 for the eight-rank all-reduce from 64 MiB per rank.
 constexpr int unrollFor(int K) { return K <= 2 ? 2 : 4; }
-constexpr int smallUnrollFor(int K) { return K >= 3 ? 1 : unrollFor(K); }
+constexpr int smallUnrollFor(int K) { return (K >= 3 || K == 0) ? 1 : unrollFor(K); }   // K = 0: run-time k, nine inputs and more
 constexpr int bigUnrollFor(int K) { return K == 8 ? 8 : unrollFor(K); }
 constexpr uint64_t kBigLaunchTiles = 1024;  // use bigUnrollFor only above this many of its tiles (32 MiB per input)
 constexpr uint64_t kSmallLaunchVecs = 256 * 1024;  // fewer 16-byte vectors of output than this: one vector per lane
@@ -179,10 +182,9 @@ flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s)
   return small ? launchBcastMany<R, K, kSmallBcastUnroll>(d, n, s) : launchBcastMany<R, K, kBcastUnroll>(d, n, s);
 }
 
-template <class R>
-flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const *in, int k, uint64_t count,
-                                  hipStream_t s) {
-  constexpr int U = unrollFor(0);
+template <class R, int U>
+flagcxResult_t launchBcastRuntimeU(void *const *out, int nout, const void *const *in, int k, uint64_t count,
+                                   hipStream_t s) {
   ManyArgs a = {};
   for (int p = 0; p < k; p++) a.in[p] = in[p];
   for (int o = 0; o < nout; o++) a.out[o] = out[o];
@@ -197,9 +199,16 @@ flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const 
   return launchKernel(reduceBcastRuntime<R, U>, (uint32_t)ntiles, s, a);
 }
 
+// One vector per lane while a launch writes less than 4 MiB per buffer, as for the fixed-k kernels.
 template <class R>
-flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
-  constexpr int U = unrollFor(0);
+flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const *in, int k, uint64_t count,
+                                  hipStream_t s) {
+  if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchBcastRuntimeU<R, 1>(out, nout, in, k, count, s);
+  return launchBcastRuntimeU<R, unrollFor(0)>(out, nout, in, k, count, s);
+}
+
+template <class R, int U>
+flagcxResult_t launchChunksRuntimeU(ChunkedArgs *a, hipStream_t s) {
   uint64_t total = 0;
   a->tileStart[0] = 0;
   for (int c = 0; c < a->nchunks; c++) {
@@ -210,6 +219,14 @@ flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
   }
   if (total == 0) return flagcxSuccess;
   return launchKernel(reduceChunksRuntime<R, U>, (uint32_t)total, s, *a);
+}
+
+template <class R>
+flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
+  uint64_t vecs = 0;
+  for (int c = 0; c < a->nchunks; c++) vecs += vectorsOf(a->cnt[c], R::ES);
+  if (vecs < kSmallLaunchVecs) return launchChunksRuntimeU<R, 1>(a, s);
+  return launchChunksRuntimeU<R, unrollFor(0)>(a, s);
 }
 
 template <class R, int K, bool BCAST = true>

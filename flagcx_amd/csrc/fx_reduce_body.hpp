@@ -468,13 +468,16 @@ constexpr uint32_t kPieceVecs = FX_PIECE_VECS;
 constexpr uint32_t kStripeTiles = FX_STRIPE_TILES;
 constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;      // 32 KiB
 #ifndef FX_STRIPE_MIN_BYTES
-#define FX_STRIPE_MIN_BYTES (1ull << 20)
+#define FX_STRIPE_MIN_BYTES (1ull << 19)
 #endif
-// Segments shorter than this (output bytes) stay contiguous: they have no
-// whole region to stripe.  (It was 4 MiB at first; the chunks of a collective
-// over eight ranks of 16 MiB are 2 MiB each, and striping them takes the
-// ring-order all-reduce from 57 to 47 us and the reduce-scatter from 28 to
-// 25 us; single segments of 1-4 MiB measure the same either way.)
+// Segments shorter than this (output bytes) stay contiguous: the smallest region
+// (two vectors per lane) is 512 KiB.  (It was 4 MiB at first; the chunks of a
+// collective over eight ranks of 16 MiB are 2 MiB each, and striping them takes
+// the ring-order all-reduce from 57 to 47 us and the reduce-scatter from 28 to
+// 25 us; from 1 MiB down to 512 KiB the 512 KiB blocks of an all-gather over
+// sixteen ranks of 8 MiB gain, 29.4 -> 24.5 us, and those of the eight-rank
+// all-to-all of 4 MiB, 12.8 -> 12.0 us; single segments of 0.5-4 MiB measure
+// the same either way, and 256 KiB the same as 512 KiB.)
 constexpr uint64_t kStripeMinBytes = FX_STRIPE_MIN_BYTES;
 
 // Streams a and b sit at the same offset within a cache line.

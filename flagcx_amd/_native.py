@@ -80,6 +80,7 @@ _SIGS = {
     "fx_copy_slices": (_i, [C.POINTER(SliceDesc), _sz, _vp]),
     "fx_reduce_bcast": (_i, [C.POINTER(_vp), _i, C.POINTER(_vp), _i, _sz, _i, _i, _i, _vp]),
     "fx_reduce_chunks": (_i, [C.POINTER(_vp), _i, C.POINTER(_vp), _i, C.POINTER(Chunk), _i, _i, _i, _vp]),
+    "fx_alltoall": (_i, [C.POINTER(_vp), C.POINTER(_vp), _i, _sz, _vp]),
     "fx_plan_create": (_i, [C.POINTER(_vp), C.POINTER(SliceDesc), _sz, _i, _i, _i]),
     "fx_plan_launch": (_i, [_vp, _vp]),
     "fx_plan_destroy": (_i, [_vp]),

@@ -534,6 +534,20 @@ int fx_reduce_chunks(void *const *outs, int nout, const void *const *ins, int k,
   });
 }
 
+int fx_alltoall(void *const *recv, const void *const *send, int n, size_t block_bytes, void *stream) {
+  if (!recv || !send || n < 1 || n > FX_MAX_INPUTS) return flagcxInvalidArgument;
+  if (block_bytes == 0) return flagcxSuccess;
+  return guarded([&]() -> int {
+    uintptr_t bits = (uintptr_t)block_bytes;
+    for (int r = 0; r < n; r++) {
+      if (!recv[r] || !send[r]) return flagcxInvalidArgument;
+      bits |= (uintptr_t)recv[r] | (uintptr_t)send[r];
+    }
+    const int es = (bits & 1) ? 1 : ((bits & 2) ? 2 : 4);   // the widest unit every address and the block size allow
+    return copySetFor(es)->allToAll(recv, send, n, (uint64_t)block_bytes / (uint64_t)es, (hipStream_t)stream);
+  });
+}
+
 int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, int dtype, int op) {
   if (!plan) return flagcxInvalidArgument;
   *plan = nullptr;

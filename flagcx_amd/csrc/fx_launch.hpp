@@ -48,6 +48,8 @@ struct KernelSet {
                                  hipStream_t s);
   // chunks of a collective over up to kMaxK ranks; tileStart is filled here
   flagcxResult_t (*chunksRuntime)(ChunkedArgs *a, hipStream_t s);
+  // copy sets only: all-to-all of n * n equal blocks in one launch
+  flagcxResult_t (*allToAll)(void *const *recv, const void *const *send, int n, uint64_t blockElems, hipStream_t s);
   int elemSize;
 };
 
@@ -229,6 +231,31 @@ flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
   return launchChunksRuntimeU<R, unrollFor(0)>(a, s);
 }
 
+// The workgroups a block of the all-to-all can need at most: its tiles, plus one for a head before the first
+// region boundary and one for a tail after the last (where the block lies in memory decides, block by block).
+template <class R, int U>
+flagcxResult_t launchAllToAllU(void *const *recv, const void *const *send, int n, uint64_t blockElems, hipStream_t s) {
+  AllToAllArgs a = {};
+  for (int r = 0; r < n; r++) {
+    a.send[r] = send[r];
+    a.recv[r] = recv[r];
+  }
+  a.blockElems = blockElems;
+  a.n = n;
+  const uint64_t V = (uint64_t)U * kBlock, nv = vectorsOf(blockElems, R::ES) + 1;   // + 1: a block off 16-byte alignment spans one vector more
+  const uint64_t striped = blockElems * (uint64_t)R::ES >= kStripeMinBytes ? 2 : 0;   // shorter blocks have no regions
+  const uint64_t per = (nv + V - 1) / V + striped, total = per * (uint64_t)n * (uint64_t)n;
+  if (total > 0x7ffffff0ull) return flagcxInvalidArgument;
+  a.tilesPerBlock = (uint32_t)per;
+  return launchKernel(allToAllBlocks<R, U>, (uint32_t)total, s, a);
+}
+
+template <class R>
+flagcxResult_t launchAllToAll(void *const *recv, const void *const *send, int n, uint64_t blockElems, hipStream_t s) {
+  if (blockElems == 0) return flagcxSuccess;
+  return launchAllToAllU<R, unrollFor(1)>(recv, send, n, blockElems, s);
+}
+
 template <class R, int K, bool BCAST = true>
 void fillSet(KernelSet &ks) {
   ks.direct[K] = &launchDirect<R, K>;
@@ -269,6 +296,7 @@ KernelSet makeCopySet() {
   fillSet<CopyRed<ES>, 1, true>(ks);
   ks.bcastRuntime = &launchBcastRuntime<CopyRed<ES>>;
   ks.chunksRuntime = &launchChunksRuntime<CopyRed<ES>>;
+  ks.allToAll = &launchAllToAll<CopyRed<ES>>;
   ks.elemSize = ES;
   return ks;
 }

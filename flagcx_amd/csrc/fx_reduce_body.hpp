@@ -1129,6 +1129,34 @@ reduceSlicesTable(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n) 
   reduceSlicesBody<R, K, U>(d, tileStart, n);
 }
 
+// All-to-all of equal blocks over up to kMaxK ranks in one launch: block (r, i)
+// -- block i of rank r's send buffer, which becomes block r of rank i's receive
+// buffer -- is a copy segment whose two addresses follow from the 2 n base
+// pointers, so no table of n * n descriptors has to travel (4,096 of them for
+// 64 ranks, 29 argument blocks).  Every block gets the same number of
+// workgroups, the most any of them can need; those a block has no tile for
+// leave at once.
+struct AllToAllArgs {
+  const void *send[kMaxK];
+  void *recv[kMaxK];
+  uint64_t blockElems;      // elements of the kernel's copy type per block
+  uint32_t tilesPerBlock;
+  int n;
+};
+
+template <class R, int U>
+__global__ void __launch_bounds__(kBlock) allToAllBlocks(AllToAllArgs a) {
+  const uint32_t blk = blockIdx.x / a.tilesPerBlock, tile = blockIdx.x % a.tilesPerBlock;
+  const uint32_t r = blk / (uint32_t)a.n, i = blk % (uint32_t)a.n;
+  const uint64_t bytes = a.blockElems * R::ES;
+  const void *in = (const char *)a.send[r] + (uint64_t)i * bytes;
+  void *out = (char *)a.recv[i] + (uint64_t)r * bytes;
+  Seg<1> sg;
+  const TilePlan tp = makeSeg<R::ES, U>(sg, &in, out, a.blockElems, 1);
+  if (tile >= tp.tiles()) return;
+  reduceTile<R, 1, U>(sg, tp, tile, (blockIdx.x - tile) & 7u);
+}
+
 // One read of the inputs, several outputs: slices whose result goes to up to
 // kMaxFixedK buffers at once.
 struct BcastDescDev {

@@ -843,11 +843,14 @@ flagcxResult_t runAlltoAll(const Ctx &c) {
   bool inplace = false;
   for (int r = 0; r < n; r++) inplace = inplace || (c.send(r) == c.recv(r));
   SliceList d;
-  if (!inplace) {
-    for (int r = 0; r < n; r++)
-      for (int i = 0; i < n; i++)
-        d.push_back(copyDesc(cadd(c.send(r), (size_t)i * bytes), madd(c.recv(i), (size_t)r * bytes), bytes));
-    return R(fx_copy_slices(d.data(), d.size(), c.s));
+  if (!inplace) {   // every block straight from its sender to its receiver, one launch
+    PtrList sends;
+    fx::SmallVec<void *, 16> recvs;
+    for (int r = 0; r < n; r++) {
+      sends.push_back(c.send(r));
+      recvs.push_back(c.recv(r));
+    }
+    return R(fx_alltoall(recvs.data(), sends.data(), n, bytes, c.s));
   }
   flagcxResult_t rc = ensureScratch(g, (size_t)n * n * bytes, c.s);
   if (rc != flagcxSuccess) return rc;
@@ -855,11 +858,13 @@ flagcxResult_t runAlltoAll(const Ctx &c) {
     d.push_back(copyDesc(c.send(r), madd(g->scratch, (size_t)r * n * bytes), (size_t)n * bytes));
   rc = R(fx_copy_slices(d.data(), d.size(), c.s));
   if (rc != flagcxSuccess) return rc;
-  d.clear();
-  for (int r = 0; r < n; r++)
-    for (int i = 0; i < n; i++)
-      d.push_back(copyDesc(cadd(g->scratch, ((size_t)r * n + i) * bytes), madd(c.recv(i), (size_t)r * bytes), bytes));
-  return R(fx_copy_slices(d.data(), d.size(), c.s));
+  PtrList staged;
+  fx::SmallVec<void *, 16> recvs;
+  for (int r = 0; r < n; r++) {
+    staged.push_back(cadd(g->scratch, (size_t)r * n * bytes));
+    recvs.push_back(c.recv(r));
+  }
+  return R(fx_alltoall(recvs.data(), staged.data(), n, bytes, c.s));
 }
 
 flagcxResult_t runCustomAllReduce(const Ctx &c) {

@@ -62,6 +62,11 @@ def reduce_chunks(outs, ins, chunks, dtype, op, stream=None):
     return lib.fx_reduce_chunks(_ptr_array(outs), len(outs), _ptr_array(ins), len(ins), arr, len(chunks), dtype, op, stream)
 
 
+def alltoall(recvs, sends, block_bytes, stream=None):
+    """Block i of sends[r] becomes block r of recvs[i]; one launch for any number of ranks up to 64."""
+    return lib.fx_alltoall(_ptr_array(recvs), _ptr_array(sends), len(sends), block_bytes, stream)
+
+
 def copy_slices(descs, stream=None):
     """descs: iterable of (src, dst, nbytes)."""
     arr, n = make_slices(([s], d, b) for s, d, b in descs)

@@ -236,6 +236,19 @@ int fx_reduce_chunks(void *const *outs, int nout, const void *const *ins, int k,
                      void *stream);
 
 /*
+ * All-to-all of equal blocks over n <= FX_MAX_INPUTS ranks in ONE launch:
+ * block i of send[r] (block_bytes each) becomes block r of recv[i], for every
+ * r and i -- the data movement of flagcxAlltoAll (flagcx/include/flagcx.h:
+ * 466-470; the reference builds it from n grouped send / recv pairs per rank,
+ * flagcx/adaptor/ccl/rccl_adaptor.cc:222-246).  The kernel works out each
+ * block's two addresses from the 2 n base pointers, so nothing grows with
+ * n * n but the grid.  No send block may overlap a receive block (in place:
+ * stage first); any alignment.
+ */
+int fx_alltoall(void *const *recv, const void *const *send, int n, size_t block_bytes, void *stream);
+
+
+/*
  * Copy n independent byte ranges (in[0] -> out, `count` = BYTES): the Cpy node
  * and the all-gather landing copies (uni_runner_impl.cc:322-344,1649-1662;
  * flagcx/core/p2p.cc:257-283) as one launch.

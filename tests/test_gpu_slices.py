@@ -511,3 +511,32 @@ def test_element_fold_is_the_reference_device_kernels_arithmetic(dev, dname):
     assert K.reduce_copy(16, [16, 32], 4, N.DT_FP32, N.OP_MAX | ELEM) == N.NOT_SUPPORTED
     assert K.reduce_copy(16, [16, 32], 4, N.DT_INT32, N.OP_SUM | ELEM) == N.NOT_SUPPORTED
     assert K.reduce_copy(16, [16, 32], 4, dtype, 7 | ELEM) == N.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("n,block,smis,rmis", [(1, 7, 0, 0), (2, 1, 1, 3), (3, 4099, 2, 0), (8, 64 << 10, 0, 0), (8, (1 << 20) + 36, 4, 4),
+                                               (13, 30001, 0, 1), (33, 1000, 0, 0), (64, 516, 4, 8), (5, 3 << 20, 0, 0)])
+def test_alltoall_in_one_launch(dev, n, block, smis, rmis):
+    """fx_alltoall: block i of send[r] becomes block r of recv[i] for every
+    pair, whatever the alignment of the buffers and the block size (odd sizes,
+    blocks long enough for the striped hand-out, 64 ranks); nothing is written
+    outside the n * block bytes of a receive buffer."""
+    rng = np.random.default_rng(n * 7 + block)
+    sends = [rng.integers(0, 256, n * block, dtype=np.uint8) for _ in range(n)]
+    with DevBufs(dev) as b:
+        ds = [b.put(a, pad_before=smis) for a in sends]
+        dr = []
+        for r in range(n):
+            base = b.alloc(16 + rmis + n * block + 64)
+            dev.memset(base, 0xA5, 16 + rmis + n * block + 64)
+            dr.append(base + 16 + rmis)
+        dev.sync()
+        N.check(K.alltoall(dr, ds, block), "fx_alltoall")
+        dev.sync()
+        for i in range(n):
+            got = dev.to_host(dr[i] - 16, 16 + n * block + 32, np.uint8)
+            want = np.concatenate([sends[r][i * block:(i + 1) * block] for r in range(n)])
+            assert (got[:16] == 0xA5).all() and (got[16 + n * block:] == 0xA5).all(), f"rank {i}: wrote outside its buffer"
+            assert np.array_equal(got[16:16 + n * block], want), f"rank {i}"
+    assert K.alltoall([16] * 65, [16] * 65, 4) == N.INVALID_ARGUMENT
+    assert K.alltoall([16, 0], [16, 32], 4) == N.INVALID_ARGUMENT
+    assert K.alltoall([16], [32], 0) == N.SUCCESS

@@ -77,6 +77,7 @@ _SIGS = {
     "fx_reduce_triggers": (_i, [C.POINTER(ReduceTrigger), _sz, _vp]),
     "fx_reduce_slices": (_i, [C.POINTER(SliceDesc), _sz, _i, _i, _i, _vp]),
     "fx_reduce_bcast_slices": (_i, [C.POINTER(BcastDesc), _sz, _i, _i, _i, _i, _vp]),
+    "fx_reduce_ordered": (_i, [C.POINTER(BcastDesc), _sz, _i, _i, _i, _i, _i, _vp]),
     "fx_copy_slices": (_i, [C.POINTER(SliceDesc), _sz, _vp]),
     "fx_reduce_bcast": (_i, [C.POINTER(_vp), _i, C.POINTER(_vp), _i, _sz, _i, _i, _i, _vp]),
     "fx_reduce_chunks": (_i, [C.POINTER(_vp), _i, C.POINTER(_vp), _i, C.POINTER(Chunk), _i, _i, _i, _vp]),

@@ -216,6 +216,7 @@ struct fxPlan {
   SliceDescDev *dDesc;
   uint32_t *dTileStart;
   uint32_t n, grid;
+  uint32_t keep;   // cache policy for what the whole plan touches
   int k;
 };
 
@@ -428,6 +429,87 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
   });
 }
 
+int fx_reduce_ordered(const fxBcastDesc *slices, size_t n, int k, int nout, int dtype, int op, int order, void *stream) {
+  flagcxResult_t rc = screen(dtype, op);
+  if (rc != flagcxSuccess) return rc;
+  if (order != FX_FOLD_CHAIN && order != FX_FOLD_TREE && order != FX_FOLD_KEEP_LOCAL) return flagcxInvalidArgument;
+  if (k < 1 || k > FX_MAX_SLICE_INPUTS || nout < 1 || nout > FX_MAX_SLICE_INPUTS) return flagcxInvalidArgument;
+  if ((op & FX_OP_ELEMENT_FOLD) || (op == flagcxAvg && order != FX_FOLD_CHAIN)) return flagcxNotSupported;
+  if (n == 0) return flagcxSuccess;
+  if (!slices) return flagcxInvalidArgument;
+  const KernelSet *ks = setFor(dtype, op);
+  const bool select = (op == flagcxMax || op == flagcxMin);
+  const bool floating = dtype == flagcxFloat16 || dtype == flagcxBfloat16 || dtype == flagcxFloat32 || dtype == flagcxFloat64;
+  // Which association has a kernel of its own.  Everything else is the
+  // input-order fold of the inputs in a suitable order:
+  //  * integers give the same bits in every association and operand order
+  //    (sum / prod wrap, max / min pick one of two equal patterns on a tie);
+  //  * two inputs: tree and keep-local are both in[1] (op) in[0];
+  //  * keep-local sums and products: the two operands of a step commute bit for
+  //    bit, so res = in[j] (op) res is res = res (op) in[j].
+  const bool reversePair = (k == 2 && order != FX_FOLD_CHAIN);
+  int kernel = -1;   // index into KernelSet::ordered, -1 = the input-order fold
+  if (floating && k >= 3) {
+    if (order == FX_FOLD_TREE) kernel = 0;
+    else if (order == FX_FOLD_KEEP_LOCAL && select) kernel = 1;
+  }
+  // 16-bit sums and products in the keep-local chain would round after every
+  // step; the host ring does not carry those types (utils.h:690-694), so there is
+  // no kernel for them.
+  const bool sixteen = dtype == flagcxFloat16 || dtype == flagcxBfloat16;
+  if (sixteen && !select && order == FX_FOLD_KEEP_LOCAL && k >= 3) return flagcxNotSupported;
+  if (kernel < 0 && !reversePair) return fx_reduce_bcast_slices(slices, n, k, nout, dtype, op, stream);
+  return guarded([&]() -> int {
+    const int es = (int)dtypeSize(dtype);
+    SmallVec<fxBcastDesc, kFewSlices> swapped;
+    SmallVec<BcastDescDev, kFewSlices> dev;
+    for (size_t i = 0; i < n; i++) {
+      fxBcastDesc d = slices[i];
+      if (d.count == 0) continue;
+      uintptr_t bits = 0;
+      for (int p = 0; p < k; p++) {
+        if (!d.in[p]) return flagcxInvalidArgument;
+        bits |= (uintptr_t)d.in[p];
+      }
+      for (int o = 0; o < nout; o++) {
+        if (!d.out[o]) return flagcxInvalidArgument;
+        bits |= (uintptr_t)d.out[o];
+      }
+      if (bits & (uintptr_t)(es - 1)) return flagcxInvalidArgument;
+      if (reversePair) {
+        const void *t = d.in[0];
+        d.in[0] = d.in[1];
+        d.in[1] = t;
+        swapped.push_back(d);
+        continue;
+      }
+      for (int o = 1; o < nout; o++)   // the one-read-n-stores kernels share byte offsets between the outputs
+        if ((((uintptr_t)d.out[o] ^ (uintptr_t)d.out[0]) & 15u) != 0) return flagcxInvalidArgument;
+      // descriptors that continue each other in every stream are one longer descriptor
+      if (!dev.empty()) {
+        BcastDescDev &l = dev.back();
+        const size_t bytes = l.count * (size_t)es;
+        bool cont = true;
+        for (int p = 0; p < k && cont; p++) cont = (const char *)d.in[p] == (const char *)l.in[p] + bytes;
+        for (int o = 0; o < nout && cont; o++) cont = (const char *)d.out[o] == (const char *)l.out[o] + bytes;
+        if (cont) {
+          l.count += d.count;
+          continue;
+        }
+      }
+      BcastDescDev dd;
+      for (int p = 0; p < kMaxFixedK; p++) dd.in[p] = (p < k) ? d.in[p] : nullptr;
+      for (int o = 0; o < kMaxFixedK; o++) dd.out[o] = (o < nout) ? d.out[o] : nullptr;
+      dd.count = d.count;
+      dd.nout = (uint32_t)nout;
+      dev.push_back(dd);
+    }
+    if (reversePair) return fx_reduce_bcast_slices(swapped.data(), swapped.size(), k, nout, dtype, op, stream);
+    if (dev.empty()) return flagcxSuccess;
+    return ks->ordered[kernel][k](dev.data(), dev.size(), (hipStream_t)stream);
+  });
+}
+
 int fx_reduce_bcast(void *const *outs, int nout, const void *const *ins, int k, size_t count, int dtype, int op,
                     int first, void *stream) {
   const bool copy = (op == -1);
@@ -572,6 +654,7 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
     const int U = unrollFor(k);
     std::vector<SliceDescDev> desc;
     std::vector<uint32_t> start(1, 0u);
+    uint64_t elems = 0;
     std::vector<fxSliceDesc> scaled(slices, slices + n);
     for (auto &d : scaled) {
       if (d.count && !d.out) return flagcxInvalidArgument;
@@ -592,6 +675,7 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
       for (int p = 0; p < kMaxFixedK; p++) d.in[p] = (p < k) ? s.in[p] : nullptr;
       d.out = s.out;
       d.count = s.count;
+      elems += s.count;
       desc.push_back(d);
       start.push_back(start.back() + (uint32_t)tiles);
     }
@@ -601,6 +685,7 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
     pl->k = k;
     pl->n = (uint32_t)desc.size();
     pl->grid = start.back();
+    pl->keep = cachePolicyFor(touchedBytes(elems, ks->elemSize, k, 1));
     pl->dDesc = nullptr;
     pl->dTileStart = nullptr;
     if (pl->n) {
@@ -621,7 +706,8 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
 int fx_plan_launch(fxPlan_t plan, void *stream) {
   if (!plan) return flagcxInvalidArgument;
   if (plan->n == 0) return flagcxSuccess;
-  return plan->ks->slicesTable[plan->k](plan->dDesc, plan->dTileStart, plan->n, plan->grid, (hipStream_t)stream);
+  return plan->ks->slicesTable[plan->k](plan->dDesc, plan->dTileStart, plan->n, plan->grid, plan->keep,
+                                        (hipStream_t)stream);
 }
 
 int fx_plan_destroy(fxPlan_t plan) {
@@ -660,7 +746,7 @@ int fx_reduce_slices_static(const fxSliceDesc *slices, size_t n, int k, int dtyp
   const size_t es = (size_t)ks->elemSize;
   // first walk: validate everything and size the table, so that an error leaves nothing enqueued
   size_t entries = 0;
-  uint64_t grid = 0;
+  uint64_t grid = 0, elems = 0;
   int rc = forEachMerged(slices, n, k, es, div, [&](const fxSliceDesc &d) -> int {
     uint64_t t = 0;
     const flagcxResult_t r = sliceTiles(d, k, (int)es, U, &t);
@@ -668,6 +754,7 @@ int fx_reduce_slices_static(const fxSliceDesc *slices, size_t n, int k, int dtyp
     if (t == 0) return 0;
     entries++;
     grid += t;
+    elems += d.count;
     return (grid > 0x7ffffff0ull) ? (int)flagcxInvalidArgument : 0;
   });
   if (rc) return rc;
@@ -708,7 +795,7 @@ int fx_reduce_slices_static(const fxSliceDesc *slices, size_t n, int k, int dtyp
   if (rc) return rc;
   rc = flush();
   if (rc) return rc;
-  return ks->slicesTable[k](dDesc, dTileStart, (uint32_t)entries, next, s);
+  return ks->slicesTable[k](dDesc, dTileStart, (uint32_t)entries, next, cachePolicyFor(touchedBytes(elems, (int)es, k, 1)), s);
 }
 
 static int packOrUnpack(bool pack, void *a, const void *b, const size_t *counts, const size_t *displs, int npeers,

@@ -34,8 +34,11 @@
 #include <sched.h>
 
 #include <cstddef>
+#include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
+#include <vector>
 
 #include "flagcx_amd/fx_kernels.h"
 #include "fx_fifo_share.hpp"
@@ -116,6 +119,7 @@ __device__ __forceinline__ void runShare(const void *in1, const void *in2, void 
   using R = Red<DT, OP>;
   const void *in[2] = {in1, in2};
   SegWT<2> sg;  // written through: see the count-in below
+  sg.keep = 0;  // inputs stream: a trigger's buffers were written by other agents, nothing of them is worth keeping
   const TilePlan tp = makeSeg<R::ES, kFifoU>(static_cast<Seg<2> &>(sg), in, out, count, 2);
   const uint64_t tiles = tp.tiles();
   // (tiles go to whichever workgroups the trigger's share names: no die grouping of columns here)
@@ -448,6 +452,70 @@ struct fxFifoConsumer {
   uint32_t inOrder;
 };
 
+namespace {
+
+// Grid of the consumer on the current device (see fifoGridFor) and whether the
+// environment asks for the in-order mode.
+flagcxResult_t consumerShape(uint32_t *grid, uint32_t *inOrder) {
+  int dev = 0, cus = 0, resident = 0;  // resident: workgroups of this kernel one compute unit holds at the same time
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, fifoConsumer, kBlock, 0) != hipSuccess || resident < 1)
+    return flagcxUnhandledDeviceError;
+  long wanted = 0;
+  if (const char *e = getenv("FX_FIFO_WGS")) wanted = atol(e);
+  else if (const char *e = getenv("FX_FIFO_WGS_PER_CU")) wanted = atol(e) * (long)(cus > 0 ? cus : 1);
+  *grid = fifoGridFor(cus, resident, wanted);
+  const char *io = getenv("FX_FIFO_IN_ORDER");
+  *inOrder = (io && atoi(io) != 0) ? 1u : 0u;
+  return flagcxSuccess;
+}
+
+flagcxResult_t launchConsumer(FifoMirror *mirror, uint32_t grid, uint32_t capacity, uint32_t inOrder, void *fifoDevicePointer,
+                              unsigned long long maxIdlePolls, hipStream_t s) {
+  static_assert(sizeof(FifoMirror) % sizeof(uint64_t) == 0, "FifoMirror is cleared in 8-byte words");
+  const uint32_t words = (uint32_t)(sizeof(FifoMirror) / sizeof(uint64_t));
+  flagcxResult_t rc = launchKernel(clearMirror, (words + kBlock - 1) / kBlock, s, (uint64_t *)mirror, words);
+  if (rc != flagcxSuccess) return rc;
+  // The kernel starts where the last consumer stopped (it reads the ring's
+  // `consumed` itself): triggers enqueued before this launch are waiting between
+  // `consumed` and `produced` and are served first.
+  return launchKernel(fifoConsumer, grid, s, (uint64_t *)fifoDevicePointer, mirror, capacity, inOrder,
+                      (uint64_t)maxIdlePolls);
+}
+
+// ---- mirrors of flagcxLaunchCollectiveKernel ----
+// That entry point has no handle to hang per-ring state on, so the device-side
+// mirror a launch needs comes from a per-device pool: taken at launch, handed
+// back by a host function enqueued behind the kernel on the same stream (it
+// only touches the pool; no device call is made from it).  The pool only grows
+// to the number of consumers that ran at the same time, and is kept until the
+// process ends.
+constexpr int kMaxPoolDevices = 64;
+struct MirrorPool {
+  std::mutex mu;
+  std::vector<FifoMirror *> idle[kMaxPoolDevices];
+};
+MirrorPool &mirrorPool() {
+  static MirrorPool *pool = new MirrorPool();   // never destroyed: a host function may still run at exit
+  return *pool;
+}
+struct MirrorTicket {
+  int dev;
+  FifoMirror *mirror;
+};
+void returnMirror(void *arg) {
+  MirrorTicket *t = static_cast<MirrorTicket *>(arg);
+  {
+    MirrorPool &pool = mirrorPool();
+    std::lock_guard<std::mutex> lock(pool.mu);
+    pool.idle[t->dev].push_back(t->mirror);
+  }
+  delete t;
+}
+
+}  // namespace
+
 extern "C" {
 #pragma GCC visibility push(default)
 
@@ -551,26 +619,11 @@ int fx_fifo_consumer_create(fxFifoConsumer_t *consumer, size_t capacity) {
   *consumer = nullptr;
   fxFifoConsumer *c = new (std::nothrow) fxFifoConsumer();
   if (!c) return flagcxSystemError;
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-      hipMalloc((void **)&c->mirror, sizeof(FifoMirror)) != hipSuccess) {
-    delete c;
-    return flagcxUnhandledDeviceError;
-  }
   c->capacity = (uint32_t)capacity;
-  int resident = 0;  // workgroups of this kernel one compute unit holds at the same time
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, fifoConsumer, kBlock, 0) != hipSuccess || resident < 1) {
-    (void)hipFree(c->mirror);
+  if (consumerShape(&c->grid, &c->inOrder) != flagcxSuccess || hipMalloc((void **)&c->mirror, sizeof(FifoMirror)) != hipSuccess) {
     delete c;
     return flagcxUnhandledDeviceError;
   }
-  long wanted = 0;
-  if (const char *e = getenv("FX_FIFO_WGS")) wanted = atol(e);
-  else if (const char *e = getenv("FX_FIFO_WGS_PER_CU")) wanted = atol(e) * (long)(cus > 0 ? cus : 1);
-  c->grid = fifoGridFor(cus, resident, wanted);
-  const char *io = getenv("FX_FIFO_IN_ORDER");
-  c->inOrder = (io && atoi(io) != 0) ? 1u : 0u;
   *consumer = c;
   return flagcxSuccess;
 }
@@ -579,18 +632,7 @@ int fx_fifo_consumer_launch(fxFifoConsumer_t c, void *fifoDevicePointer, const u
                             unsigned long long maxIdlePolls, void *stream) {
   if (!c || !fifoDevicePointer || !fifoHost || maxIdlePolls == 0) return flagcxInvalidArgument;
   if (fifoHost[0] != c->capacity) return flagcxInvalidArgument;
-  hipStream_t s = (hipStream_t)stream;
-  static_assert(sizeof(FifoMirror) % sizeof(uint64_t) == 0, "FifoMirror is cleared in 8-byte words");
-  const uint32_t words = (uint32_t)(sizeof(FifoMirror) / sizeof(uint64_t));
-  flagcxResult_t rc = launchKernel(clearMirror, (words + kBlock - 1) / kBlock, s, (uint64_t *)c->mirror, words);
-  if (rc != flagcxSuccess) return rc;
-  // The kernel starts where the last consumer stopped (it reads the ring's
-  // `consumed` itself): triggers enqueued before this launch are waiting between
-  // `consumed` and `produced` and are served first.
-  rc = launchKernel(fifoConsumer, c->grid, s, (uint64_t *)fifoDevicePointer, c->mirror, c->capacity, c->inOrder,
-                    (uint64_t)maxIdlePolls);
-  if (rc != flagcxSuccess) return rc;
-  return flagcxSuccess;
+  return launchConsumer(c->mirror, c->grid, c->capacity, c->inOrder, fifoDevicePointer, maxIdlePolls, (hipStream_t)stream);
 }
 
 int fx_fifo_consumer_status(fxFifoConsumer_t c, int *exitReason, uint64_t *completed, uint64_t *badTriggers) {
@@ -612,4 +654,77 @@ int fx_fifo_consumer_destroy(fxFifoConsumer_t c) {
 }
 
 #pragma GCC visibility pop
+}
+
+// The reference's own entry point, under its own name and C++ linkage
+// (flagcx/include/flagcx_kernel_internal.h:56, defined in
+// flagcx/adaptor/kernel/nvidia/flagcx_reduce_kernel_device.cu:188-192, called by
+// runUniRunner, flagcx/runner/uni_runner_impl.cc:1872-1874), so that the
+// scheduler links and runs unmodified: launch the consumer of the ring at
+// `fifoBuffer` (the device pointer of the pinned ring) on `stream`.  nthreads
+// and nblocks are accepted and ignored -- they size the reference's kernel, one
+// block of 32 threads by default; this consumer sizes itself to the device.  The
+// capacity is read from word 0 of the ring.  The kernel ends when the ring's
+// terminate word is set and the ring is drained, as the reference's does; the
+// bound every wait in it carries is FX_FIFO_MAX_IDLE_POLLS polls of an idle ring
+// (environment; default 2^36, about a day).  There is no result to return:
+// failures are reported on stderr, and a scheduler that then waits for a trigger
+// to complete waits forever, as it would after a failed launch of the
+// reference's kernel.
+struct flagcxStream {   // the device adaptor's stream handle (flagcx/adaptor/include/amd_adaptor.h:13-23)
+  hipStream_t base;
+};
+
+__attribute__((visibility("default"))) void flagcxLaunchCollectiveKernel(void *fifoBuffer, size_t nthreads, size_t nblocks,
+                                                                         flagcxStream_t stream) {
+  (void)nthreads;
+  (void)nblocks;
+  auto fail = [](const char *what) { fprintf(stderr, "flagcxLaunchCollectiveKernel: %s\n", what); };
+  if (!fifoBuffer) return fail("no ring");
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxPoolDevices) return fail("no current device");
+  // word 0 of the ring: through the host mapping of the pinned buffer when the runtime knows one, else a copy
+  uint64_t capacity = 0;
+  hipPointerAttribute_t attr;
+  memset(&attr, 0, sizeof(attr));
+  if (hipPointerGetAttributes(&attr, fifoBuffer) == hipSuccess && attr.hostPointer) {
+    capacity = __atomic_load_n(static_cast<const uint64_t *>(attr.hostPointer), __ATOMIC_ACQUIRE);
+  } else {
+    (void)hipGetLastError();
+    if (hipMemcpy(&capacity, fifoBuffer, sizeof(capacity), hipMemcpyDeviceToHost) != hipSuccess) return fail("cannot read the ring's capacity");
+  }
+  if (capacity == 0 || capacity > kMaxCapacity) return fail("ring capacity out of range (1..1024)");
+  uint32_t grid = 0, inOrder = 0;
+  if (consumerShape(&grid, &inOrder) != flagcxSuccess) return fail("cannot size the consumer");
+  unsigned long long maxIdlePolls = 1ull << 36;
+  if (const char *e = getenv("FX_FIFO_MAX_IDLE_POLLS")) {
+    const unsigned long long v = strtoull(e, nullptr, 0);
+    if (v) maxIdlePolls = v;
+  }
+  MirrorTicket *ticket = new (std::nothrow) MirrorTicket();
+  if (!ticket) return fail("out of memory");
+  ticket->dev = dev;
+  ticket->mirror = nullptr;
+  {
+    MirrorPool &pool = mirrorPool();
+    std::lock_guard<std::mutex> lock(pool.mu);
+    if (!pool.idle[dev].empty()) {
+      ticket->mirror = pool.idle[dev].back();
+      pool.idle[dev].pop_back();
+    }
+  }
+  if (!ticket->mirror && hipMalloc((void **)&ticket->mirror, sizeof(FifoMirror)) != hipSuccess) {
+    delete ticket;
+    return fail("cannot allocate the device-side mirror");
+  }
+  hipStream_t s = stream ? stream->base : nullptr;
+  if (launchConsumer(ticket->mirror, grid, (uint32_t)capacity, inOrder, fifoBuffer, maxIdlePolls, s) != flagcxSuccess) {
+    returnMirror(ticket);
+    return fail("kernel launch failed");
+  }
+  // behind the kernel on the same stream: the mirror is free again once the consumer has ended
+  if (hipLaunchHostFunc(s, returnMirror, ticket) != hipSuccess) {
+    (void)hipGetLastError();   // the mirror stays out of the pool (one leaked block); the consumer itself runs
+    fail("could not enqueue the mirror's return; it is not reused");
+  }
 }

@@ -13,25 +13,65 @@ namespace fx {
 //    workgroups than the device has compute units and each lane waits for 32
 //    loads: an eight-input reduction of 1 MiB per input takes 4.8 us against
 //    2.9 us, the eight-rank all-reduce of 64 KiB per rank 6.2 against 4.3 us.
-//    The run-time-k kernels (nine inputs and more, 2 otherwise) likewise: the
-//    all-reduce of 16 KiB per rank over 12 / 16 / 32 ranks 5.0 / 5.8 / 10.4
-//    against 4.0 / 4.5 / 8.2 us.
-//  * Larger launches: 4 (2 for one and two inputs); 8 for 8 inputs once the
-//    launch is large enough not to miss the extra workgroups and every input is
-//    aligned like the output (256 VGPRs; unaligned: 4 is 7-10 % faster).  Between
-//    1, 2 and 4 the difference at these sizes is within 1 % and changes sign with
-//    where the buffers sit: builds that differ only in this number, run
-//    alternately on one box, gave the same figures for two-input sums, copies,
-//    pack / unpack and four-input sums from 8 MiB to 1 GiB, and 0.5-1 % in favour
-//    of 4 over 1 for the eight-rank all-reduce from 64 MiB per rank.
+//    The run-time-k kernels (nine inputs and more, 2 otherwise) likewise.
+//  * Larger launches: 4 (2 for one and two inputs).  Between 1, 2, 4 and 8 the
+//    difference at these sizes is within 1 % and changes sign with where the
+//    buffers sit.
+// LEAN kernel sets (the types only the host path of the reference carries, and
+// the element-type fold) have one variant per input count: no separate
+// small-launch kernels and one table size.
 constexpr int unrollFor(int K) { return K <= 2 ? 2 : 4; }
-constexpr int smallUnrollFor(int K) { return (K >= 3 || K == 0) ? 1 : unrollFor(K); }   // K = 0: run-time k, nine inputs and more
-constexpr int bigUnrollFor(int K) { return K == 8 ? 8 : unrollFor(K); }
-constexpr uint64_t kBigLaunchTiles = 1024;  // use bigUnrollFor only above this many of its tiles (32 MiB per input)
+constexpr int smallUnrollFor(int K, bool lean) {
+  return (!lean && (K >= 3 || K == 0)) ? 1 : unrollFor(K);   // K = 0: run-time k, nine inputs and more
+}
 constexpr uint64_t kSmallLaunchVecs = 256 * 1024;  // fewer 16-byte vectors of output than this: one vector per lane
-constexpr int kBcastUnroll = 4, kSmallBcastUnroll = 1;   // the multi-output kernels, any number of inputs
+constexpr int kBcastUnroll = 4;
+constexpr int smallBcastUnroll(bool lean) { return lean ? kBcastUnroll : 1; }   // the multi-output kernels, any number of inputs
+constexpr int kOrderedUnroll = 2;   // the tree / keep-local kernels: one variant for every size
 
 inline uint64_t vectorsOf(uint64_t count, int es) { return (count * (uint64_t)es + 15) / 16; }
+
+// ---- cache policy of a launch ----
+//
+// MI355X has 256 MiB of memory-side cache behind the 4 MiB L2 of each die.
+// Nontemporal accesses stream past it, which is what a launch wants whose
+// operands could never fit: they would only push out what could.  A launch
+// whose operands do fit wants the opposite -- its inputs were usually written
+// by the kernel just before it and its output is read by the one just after --
+// so a launch that touches no more than temporalMaxBytes() uses ordinary loads
+// and stores.  FX_TEMPORAL_MAX_BYTES (environment, read once) moves the
+// threshold; FX_CACHE_POLICY = stream | keep | keep-loads | keep-stores forces
+// one policy for every launch (measurements).
+struct CachePolicyConfig {
+  uint64_t maxBytes;
+  int forced;        // -1: by size; otherwise the policy bits for every launch
+};
+constexpr uint64_t kTemporalMaxBytesDefault = 256ull << 20;
+constexpr uint32_t kAutoKeepBits = kKeepAllLoads | kKeepStores;
+inline CachePolicyConfig readCachePolicyConfig() {
+  CachePolicyConfig c = {kTemporalMaxBytesDefault, -1};
+  if (const char *e = getenv("FX_TEMPORAL_MAX_BYTES")) {
+    char *end = nullptr;
+    const unsigned long long v = strtoull(e, &end, 0);
+    if (end != e) c.maxBytes = v;
+  }
+  if (const char *e = getenv("FX_CACHE_POLICY")) {
+    if (!strcmp(e, "stream")) c.forced = 0;
+    else if (!strcmp(e, "keep")) c.forced = (int)(kKeepAllLoads | kKeepStores);
+    else if (!strcmp(e, "keep-loads")) c.forced = (int)kKeepAllLoads;
+    else if (!strcmp(e, "keep-stores")) c.forced = (int)kKeepStores;
+  }
+  return c;
+}
+inline uint32_t cachePolicyFor(uint64_t bytesTouched) {
+  static const CachePolicyConfig cfg = readCachePolicyConfig();
+  if (cfg.forced >= 0) return (uint32_t)cfg.forced;
+  return bytesTouched <= cfg.maxBytes ? kAutoKeepBits : 0u;
+}
+// Bytes a reduction of `count` elements of `es` bytes touches: k inputs, nout outputs.
+inline uint64_t touchedBytes(uint64_t count, int es, int k, int nout) {
+  return count * (uint64_t)es * (uint64_t)(k + nout);
+}
 
 struct KernelSet {
   // index = compile-time input count, 0 = runtime-k kernel
@@ -40,9 +80,12 @@ struct KernelSet {
   flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const fxSliceDesc *slices, size_t n, hipStream_t s);
   // device-resident tables, tile counts made with unrollFor(k)
   flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
-                                                uint32_t grid, hipStream_t s);
+                                                uint32_t grid, uint32_t keep, hipStream_t s);
   // n validated, non-empty multi-output slices
   flagcxResult_t (*bcastInline[kMaxFixedK + 1])(const BcastDescDev *d, size_t n, hipStream_t s);
+  // the same with the inputs combined in the tree ([0]) or keep-local ([1]) association; nullptr where the
+  // association cannot differ from the input-order fold (integers) or is not defined (avg)
+  flagcxResult_t (*ordered[2][kMaxFixedK + 1])(const BcastDescDev *d, size_t n, hipStream_t s);
   // one segment, up to kMaxK inputs and kMaxK outputs (outputs aligned alike within 16 bytes)
   flagcxResult_t (*bcastRuntime)(void *const *out, int nout, const void *const *in, int k, uint64_t count,
                                  hipStream_t s);
@@ -68,27 +111,26 @@ flagcxResult_t launchDirectU(void *out, const void *const *in, int k, uint64_t c
   a.out = out;
   a.count = count;
   a.k = kk;
+  a.keep = cachePolicyFor(touchedBytes(count, R::ES, kk, 1));
   uint64_t ntiles = tilesFor(out, in, kk, count, R::ES, U);
   if (ntiles == 0) return flagcxSuccess;
   if (ntiles > 0x7ffffff0ull) return flagcxInvalidArgument;
   return launchKernel(reduceCopyDirect<R, K, U>, (uint32_t)ntiles, s, a);
 }
 
-template <class R, int K>
+template <class R, int K, bool LEAN>
 flagcxResult_t launchDirect(void *out, const void *const *in, int k, uint64_t count, hipStream_t s) {
-  constexpr int US = smallUnrollFor(K), UD = unrollFor(K), UB = bigUnrollFor(K);
+  constexpr int US = smallUnrollFor(K, LEAN), UD = unrollFor(K);
   if constexpr (US != UD)
     if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchDirectU<R, K, US>(out, in, k, count, s);
-  if constexpr (UB != UD)
-    if (coAlignedHost(out, in, (K > 0) ? K : k) && tilesFor(out, in, (K > 0) ? K : k, count, R::ES, UB) >= kBigLaunchTiles)
-      return launchDirectU<R, K, UB>(out, in, k, count, s);
   return launchDirectU<R, K, UD>(out, in, k, count, s);
 }
 
 template <class R, int K, int U, int NS>
-flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, size_t n, hipStream_t s) {
+flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, size_t n, uint32_t keep, hipStream_t s) {
   InlineSliceTable<K, NS> t;
   t.n = 0;
+  t.keep = keep;
   t.tileStart[0] = 0;
   for (size_t i = 0; i <= n; i++) {
     uint64_t tiles = 0;
@@ -114,24 +156,30 @@ flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, size_t n, hipS
   return flagcxSuccess;
 }
 
-template <class R, int K>
+// The policy follows what the whole call touches (a batch that spreads over
+// several launches still shares the caches).
+template <class R, int K, bool LEAN>
 flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, size_t n, hipStream_t s) {
-  constexpr int US = smallUnrollFor(K), UD = unrollFor(K);
-  if (n > (size_t)kSmallSliceTable) return launchSlicesInlineSized<R, K, UD, 0>(slices, n, s);
-  if constexpr (US != UD) {
-    uint64_t vecs = 0;
-    for (size_t i = 0; i < n; i++) vecs += vectorsOf(slices[i].count, R::ES);
-    if (vecs < kSmallLaunchVecs) return launchSlicesInlineSized<R, K, US, kSmallSliceTable>(slices, n, s);
+  constexpr int US = smallUnrollFor(K, LEAN), UD = unrollFor(K);
+  uint64_t vecs = 0, elems = 0;
+  for (size_t i = 0; i < n; i++) {
+    vecs += vectorsOf(slices[i].count, R::ES);
+    elems += slices[i].count;
   }
-  return launchSlicesInlineSized<R, K, UD, kSmallSliceTable>(slices, n, s);
+  const uint32_t keep = cachePolicyFor(touchedBytes(elems, R::ES, K, 1));
+  if constexpr (LEAN) return launchSlicesInlineSized<R, K, UD, kSmallSliceTable>(slices, n, keep, s);
+  if (n > (size_t)kSmallSliceTable) return launchSlicesInlineSized<R, K, UD, 0>(slices, n, keep, s);
+  if constexpr (US != UD)
+    if (vecs < kSmallLaunchVecs) return launchSlicesInlineSized<R, K, US, kSmallSliceTable>(slices, n, keep, s);
+  return launchSlicesInlineSized<R, K, UD, kSmallSliceTable>(slices, n, keep, s);
 }
 
 template <class R, int K>
 flagcxResult_t launchSlicesTable(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n, uint32_t grid,
-                                 hipStream_t s) {
+                                 uint32_t keep, hipStream_t s) {
   constexpr int U = unrollFor(K);
   if (grid == 0) return flagcxSuccess;
-  return launchKernel(reduceSlicesTable<R, K, U>, grid, s, d, tileStart, n);
+  return launchKernel(reduceSlicesTable<R, K, U>, grid, s, d, tileStart, n, keep);
 }
 
 inline uint64_t bcastTiles(const BcastDescDev &d, int k, int es, int U) {
@@ -139,7 +187,7 @@ inline uint64_t bcastTiles(const BcastDescDev &d, int k, int es, int U) {
 }
 
 template <class R, int K, int U>
-flagcxResult_t launchBcastOne(const BcastDescDev &d, hipStream_t s) {  // the one-slot table
+flagcxResult_t launchBcastOne(const BcastDescDev &d, uint32_t keep, hipStream_t s) {  // the one-slot table
   const uint64_t tiles = bcastTiles(d, K, R::ES, U);
   if (tiles > 0x7ffffff0ull) return flagcxInvalidArgument;
   InlineBcastTable<1> t;
@@ -147,13 +195,15 @@ flagcxResult_t launchBcastOne(const BcastDescDev &d, hipStream_t s) {  // the on
   t.tileStart[0] = 0;
   t.tileStart[1] = (uint32_t)tiles;
   t.n = 1;
-  return launchKernel(reduceBcastInline<R, K, U, 1>, (uint32_t)tiles, s, t);
+  t.keep = keep;
+  return launchKernel(reduceBcastInline<R, K, U, 1, kChain>, (uint32_t)tiles, s, t);
 }
 
-template <class R, int K, int U>
-flagcxResult_t launchBcastMany(const BcastDescDev *d, size_t n, hipStream_t s) {  // the sixteen-slot table
+template <class R, int K, int U, int SCHED>
+flagcxResult_t launchBcastMany(const BcastDescDev *d, size_t n, uint32_t keep, hipStream_t s) {  // the eight-slot table
   InlineBcastTable<kInlineBcast> t;
   t.n = 0;
+  t.keep = keep;
   t.tileStart[0] = 0;
   for (size_t i = 0; i <= n; i++) {
     uint64_t tiles = 0;
@@ -163,7 +213,7 @@ flagcxResult_t launchBcastMany(const BcastDescDev *d, size_t n, hipStream_t s) {
     }
     const bool full = t.n == (uint32_t)kInlineBcast || (i < n && (uint64_t)t.tileStart[t.n] + tiles > 0x7ffffff0ull);
     if ((i == n || full) && t.n > 0) {
-      const flagcxResult_t rc = launchKernel(reduceBcastInline<R, K, U, kInlineBcast>, t.tileStart[t.n], s, t);
+      const flagcxResult_t rc = launchKernel(reduceBcastInline<R, K, U, kInlineBcast, SCHED>, t.tileStart[t.n], s, t);
       if (rc != flagcxSuccess) return rc;
       t.n = 0;
     }
@@ -175,13 +225,32 @@ flagcxResult_t launchBcastMany(const BcastDescDev *d, size_t n, hipStream_t s) {
   return flagcxSuccess;
 }
 
-template <class R, int K>
+inline uint32_t bcastPolicy(const BcastDescDev *d, size_t n, int es, int k, uint64_t *vecsPerOutput) {
+  uint64_t vecs = 0, bytes = 0;
+  for (size_t i = 0; i < n; i++) {
+    vecs += vectorsOf(d[i].count, es);
+    bytes += touchedBytes(d[i].count, es, k, (int)d[i].nout);
+  }
+  *vecsPerOutput = vecs;
+  return cachePolicyFor(bytes);
+}
+
+template <class R, int K, bool LEAN>
 flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s) {
+  constexpr int US = smallBcastUnroll(LEAN), UD = kBcastUnroll;
   uint64_t vecs = 0;   // per output buffer, all descriptors together
-  for (size_t i = 0; i < n; i++) vecs += vectorsOf(d[i].count, R::ES);
+  const uint32_t keep = bcastPolicy(d, n, R::ES, K, &vecs);
+  if constexpr (LEAN) return launchBcastMany<R, K, UD, kChain>(d, n, keep, s);
   const bool small = vecs < kSmallLaunchVecs;
-  if (n == 1) return small ? launchBcastOne<R, K, kSmallBcastUnroll>(d[0], s) : launchBcastOne<R, K, kBcastUnroll>(d[0], s);
-  return small ? launchBcastMany<R, K, kSmallBcastUnroll>(d, n, s) : launchBcastMany<R, K, kBcastUnroll>(d, n, s);
+  if (n == 1) return small ? launchBcastOne<R, K, US>(d[0], keep, s) : launchBcastOne<R, K, UD>(d[0], keep, s);
+  return small ? launchBcastMany<R, K, US, kChain>(d, n, keep, s) : launchBcastMany<R, K, UD, kChain>(d, n, keep, s);
+}
+
+template <class R, int K, int SCHED>
+flagcxResult_t launchOrdered(const BcastDescDev *d, size_t n, hipStream_t s) {
+  uint64_t vecs = 0;
+  const uint32_t keep = bcastPolicy(d, n, R::ES, K, &vecs);
+  return launchBcastMany<R, K, kOrderedUnroll, SCHED>(d, n, keep, s);
 }
 
 template <class R, int U>
@@ -193,6 +262,7 @@ flagcxResult_t launchBcastRuntimeU(void *const *out, int nout, const void *const
   a.count = count;
   a.k = k;
   a.nout = nout;
+  a.keep = cachePolicyFor(touchedBytes(count, R::ES, k, nout));
   if (count == 0) return flagcxSuccess;
   a.co = coAlignedHost(out[0], in, k, out + 1, nout - 1) ? 1 : 0;
   const uint64_t ntiles = planTiles((uint64_t)(uintptr_t)out[0], count, R::ES, U, handOutFor(a.co != 0, k)).tiles();
@@ -202,32 +272,37 @@ flagcxResult_t launchBcastRuntimeU(void *const *out, int nout, const void *const
 }
 
 // One vector per lane while a launch writes less than 4 MiB per buffer, as for the fixed-k kernels.
-template <class R>
+template <class R, bool LEAN>
 flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const *in, int k, uint64_t count,
                                   hipStream_t s) {
-  if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchBcastRuntimeU<R, 1>(out, nout, in, k, count, s);
+  if constexpr (!LEAN)
+    if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchBcastRuntimeU<R, 1>(out, nout, in, k, count, s);
   return launchBcastRuntimeU<R, unrollFor(0)>(out, nout, in, k, count, s);
 }
 
 template <class R, int U>
 flagcxResult_t launchChunksRuntimeU(ChunkedArgs *a, hipStream_t s) {
-  uint64_t total = 0;
+  uint64_t total = 0, bytes = 0;
   a->tileStart[0] = 0;
   for (int c = 0; c < a->nchunks; c++) {
     a->co[c] = chunkCoAligned(*a, c) ? 1 : 0;
     total += a->cnt[c] ? chunkPlan<R::ES, U>(*a, c).tiles() : 0;
     if (total > 0x7ffffff0ull) return flagcxInvalidArgument;
     a->tileStart[c + 1] = (uint32_t)total;
+    bytes += touchedBytes(a->cnt[c], R::ES, a->only[c] >= 0 ? 1 : a->k, a->outSel[c] >= 0 ? 1 : a->nout);
   }
   if (total == 0) return flagcxSuccess;
+  a->keep = cachePolicyFor(bytes);
   return launchKernel(reduceChunksRuntime<R, U>, (uint32_t)total, s, *a);
 }
 
-template <class R>
+template <class R, bool LEAN>
 flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
-  uint64_t vecs = 0;
-  for (int c = 0; c < a->nchunks; c++) vecs += vectorsOf(a->cnt[c], R::ES);
-  if (vecs < kSmallLaunchVecs) return launchChunksRuntimeU<R, 1>(a, s);
+  if constexpr (!LEAN) {
+    uint64_t vecs = 0;
+    for (int c = 0; c < a->nchunks; c++) vecs += vectorsOf(a->cnt[c], R::ES);
+    if (vecs < kSmallLaunchVecs) return launchChunksRuntimeU<R, 1>(a, s);
+  }
   return launchChunksRuntimeU<R, unrollFor(0)>(a, s);
 }
 
@@ -242,6 +317,7 @@ flagcxResult_t launchAllToAllU(void *const *recv, const void *const *send, int n
   }
   a.blockElems = blockElems;
   a.n = n;
+  a.keep = cachePolicyFor(touchedBytes(blockElems * (uint64_t)n * (uint64_t)n, R::ES, 1, 1));
   const uint64_t V = (uint64_t)U * kBlock, nv = vectorsOf(blockElems, R::ES) + 1;   // + 1: a block off 16-byte alignment spans one vector more
   const uint64_t striped = blockElems * (uint64_t)R::ES >= kStripeMinBytes ? 2 : 0;   // shorter blocks have no regions
   const uint64_t per = (nv + V - 1) / V + striped, total = per * (uint64_t)n * (uint64_t)n;
@@ -256,14 +332,35 @@ flagcxResult_t launchAllToAll(void *const *recv, const void *const *send, int n,
   return launchAllToAllU<R, unrollFor(1)>(recv, send, n, blockElems, s);
 }
 
-template <class R, int K, bool BCAST = true>
+// Which associations other than the input-order fold a reducer is built for:
+// the tree for every floating type and sum / prod / max / min (integers give the
+// same bits in any association; a mean is not a tree of two-input means), the
+// keep-local chain for floating max / min (sums and products commute bit for
+// bit in each step, so the input-order fold over suitably ordered inputs
+// already is that chain).
+template <class R>
+struct OrderedFolds {
+  static constexpr bool tree = false, keepLocal = false;
+};
+template <int DT, int OP>
+struct OrderedFolds<Red<DT, OP>> {
+  static constexpr bool floating = DT == flagcxFloat16 || DT == flagcxBfloat16 || DT == flagcxFloat32 || DT == flagcxFloat64;
+  static constexpr bool tree = floating && OP != flagcxAvg;
+  static constexpr bool keepLocal = floating && (OP == flagcxMax || OP == flagcxMin);
+};
+
+template <class R, int K, bool LEAN>
 void fillSet(KernelSet &ks) {
-  ks.direct[K] = &launchDirect<R, K>;
-  if (K > 0) {
-    ks.slicesInline[K] = &launchSlicesInline<R, (K > 0 ? K : 1)>;
-    ks.slicesTable[K] = &launchSlicesTable<R, (K > 0 ? K : 1)>;
-    if constexpr (BCAST) ks.bcastInline[K] = &launchBcastInline<R, (K > 0 ? K : 1)>;
-    else ks.bcastInline[K] = nullptr;
+  ks.direct[K] = &launchDirect<R, K, LEAN>;
+  ks.ordered[0][K] = ks.ordered[1][K] = nullptr;
+  if constexpr (K > 0) {
+    ks.slicesInline[K] = &launchSlicesInline<R, K, LEAN>;
+    ks.slicesTable[K] = &launchSlicesTable<R, K>;
+    ks.bcastInline[K] = &launchBcastInline<R, K, LEAN>;
+    if constexpr (K >= 3) {   // one and two inputs: every association is the input-order fold of suitably ordered inputs
+      if constexpr (OrderedFolds<R>::tree) ks.ordered[0][K] = &launchOrdered<R, K, kTree>;
+      if constexpr (OrderedFolds<R>::keepLocal) ks.ordered[1][K] = &launchOrdered<R, K, kKeepLocal>;
+    }
   } else {
     ks.slicesInline[0] = nullptr;
     ks.slicesTable[0] = nullptr;
@@ -271,20 +368,20 @@ void fillSet(KernelSet &ks) {
   }
 }
 
-template <class R>
+template <class R, bool LEAN>
 KernelSet makeSet() {
-  KernelSet ks;
-  fillSet<R, 0>(ks);
-  fillSet<R, 1>(ks);
-  fillSet<R, 2>(ks);
-  fillSet<R, 3>(ks);
-  fillSet<R, 4>(ks);
-  fillSet<R, 5>(ks);
-  fillSet<R, 6>(ks);
-  fillSet<R, 7>(ks);
-  fillSet<R, 8>(ks);
-  ks.bcastRuntime = &launchBcastRuntime<R>;
-  ks.chunksRuntime = &launchChunksRuntime<R>;
+  KernelSet ks = {};
+  fillSet<R, 0, LEAN>(ks);
+  fillSet<R, 1, LEAN>(ks);
+  fillSet<R, 2, LEAN>(ks);
+  fillSet<R, 3, LEAN>(ks);
+  fillSet<R, 4, LEAN>(ks);
+  fillSet<R, 5, LEAN>(ks);
+  fillSet<R, 6, LEAN>(ks);
+  fillSet<R, 7, LEAN>(ks);
+  fillSet<R, 8, LEAN>(ks);
+  ks.bcastRuntime = &launchBcastRuntime<R, LEAN>;
+  ks.chunksRuntime = &launchChunksRuntime<R, LEAN>;
   ks.elemSize = R::ES;
   return ks;
 }
@@ -293,19 +390,21 @@ KernelSet makeSet() {
 template <int ES>
 KernelSet makeCopySet() {
   KernelSet ks = {};
-  fillSet<CopyRed<ES>, 1, true>(ks);
-  ks.bcastRuntime = &launchBcastRuntime<CopyRed<ES>>;
-  ks.chunksRuntime = &launchChunksRuntime<CopyRed<ES>>;
+  fillSet<CopyRed<ES>, 1, false>(ks);
+  ks.bcastRuntime = &launchBcastRuntime<CopyRed<ES>, false>;
+  ks.chunksRuntime = &launchChunksRuntime<CopyRed<ES>, false>;
   ks.allToAll = &launchAllToAll<CopyRed<ES>>;
   ks.elemSize = ES;
   return ks;
 }
 
-template <int DT>
+// The four types of the device path (fp32, fp16, bf16, int32) get the full set
+// of variants; the types only the reference's host loops carry get the lean one.
+template <int DT, bool LEAN>
 const KernelSet *makeSets() {
-  static const KernelSet sets[5] = {makeSet<Red<DT, flagcxSum>>(), makeSet<Red<DT, flagcxProd>>(),
-                                    makeSet<Red<DT, flagcxMax>>(), makeSet<Red<DT, flagcxMin>>(),
-                                    makeSet<Red<DT, flagcxAvg>>()};  // indexed by flagcxRedOp_t
+  static const KernelSet sets[5] = {makeSet<Red<DT, flagcxSum>, LEAN>(), makeSet<Red<DT, flagcxProd>, LEAN>(),
+                                    makeSet<Red<DT, flagcxMax>, LEAN>(), makeSet<Red<DT, flagcxMin>, LEAN>(),
+                                    makeSet<Red<DT, flagcxAvg>, LEAN>()};  // indexed by flagcxRedOp_t
   return sets;
 }
 

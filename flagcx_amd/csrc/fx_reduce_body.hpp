@@ -458,27 +458,12 @@ struct CopyRed {
 // fetched); grouped columns and temporal loads 6.3-6.4 (1.11 x).  Aligned
 // streams keep column i and nontemporal loads (grouped columns cost 1-2 % for
 // 8 inputs of 512 MiB, temporal loads 4 % for large aligned streams).
-#ifndef FX_PIECE_VECS
-#define FX_PIECE_VECS 32      // 512 bytes; other values are for experiments (a divisor of the workgroup size)
-#endif
-#ifndef FX_STRIPE_TILES
-#define FX_STRIPE_TILES 64    // tiles per region; other values are for experiments (a multiple of 8)
-#endif
-constexpr uint32_t kPieceVecs = FX_PIECE_VECS;
-constexpr uint32_t kStripeTiles = FX_STRIPE_TILES;
-constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;      // 32 KiB
-#ifndef FX_STRIPE_MIN_BYTES
-#define FX_STRIPE_MIN_BYTES (1ull << 19)
-#endif
+constexpr uint32_t kPieceVecs = 32;                         // 512 bytes (a divisor of the workgroup size)
+constexpr uint32_t kStripeTiles = 64;                       // tiles per region (a multiple of 8)
+constexpr uint32_t kRowVecs = kPieceVecs * kStripeTiles;    // 32 KiB
 // Segments shorter than this (output bytes) stay contiguous: the smallest region
-// (two vectors per lane) is 512 KiB.  (It was 4 MiB at first; the chunks of a
-// collective over eight ranks of 16 MiB are 2 MiB each, and striping them takes
-// the ring-order all-reduce from 57 to 47 us and the reduce-scatter from 28 to
-// 25 us; from 1 MiB down to 512 KiB the 512 KiB blocks of an all-gather over
-// sixteen ranks of 8 MiB gain, 29.4 -> 24.5 us, and those of the eight-rank
-// all-to-all of 4 MiB, 12.8 -> 12.0 us; single segments of 0.5-4 MiB measure
-// the same either way, and 256 KiB the same as 512 KiB.)
-constexpr uint64_t kStripeMinBytes = FX_STRIPE_MIN_BYTES;
+// (two vectors per lane) is 512 KiB.
+constexpr uint64_t kStripeMinBytes = 1ull << 19;
 
 // Streams a and b sit at the same offset within a cache line.
 constexpr uint64_t kLineBytes = 128;
@@ -547,6 +532,7 @@ struct Seg {
   const char *in[K];
   char *out;
   uint64_t lead, end;
+  uint32_t keep;   // cache policy of the launch (kKeepAllLoads / kKeepStores bits), wave-uniform
   __device__ __forceinline__ const char *inp(int p) const { return in[p]; }
   __device__ __forceinline__ int inputs() const { return K; }
 };
@@ -559,6 +545,7 @@ struct Seg<0> {
   uint64_t mis;
   char *out;
   uint64_t lead, end;
+  uint32_t keep;
   int k;
   __device__ __forceinline__ const char *inp(int p) const { return asGlobal(raw[p]) - mis; }
   __device__ __forceinline__ int inputs() const { return k; }
@@ -617,16 +604,22 @@ struct SegB : Seg<K> {
   int nmore;
 };
 
+// One result vector to memory, streaming or ordinary as the launch's policy says
+// (the choice is the same for every lane of the launch).
+__device__ __forceinline__ void stg_as(uint32_t keep, void *p, u32x4 v) {
+  if (keep & kKeepStores) stg_keep(p, v);
+  else stg_stream(p, v);
+}
 template <int K>
 __device__ __forceinline__ void storeVector(const Seg<K> &sg, uint64_t byteOff, u32x4 v) {
-  stg_stream(sg.out + byteOff, v);
+  stg_as(sg.keep, sg.out + byteOff, v);
 }
 template <int K>
 __device__ __forceinline__ void storeVector(const SegB<K> &sg, uint64_t byteOff, u32x4 v) {
-  stg_stream(sg.out + byteOff, v);
+  stg_as(sg.keep, sg.out + byteOff, v);
 #pragma unroll
   for (int o = 0; o < kMaxFixedK - 1; o++)   // constant indices keep the pointers in scalar registers
-    if (o < sg.nmore) stg_stream(sg.more[o] + byteOff, v);
+    if (o < sg.nmore) stg_as(sg.keep, sg.more[o] + byteOff, v);
 }
 template <int ES, int K>
 __device__ __forceinline__ void storeElems(const Seg<K> &sg, uint64_t e0, int lo, int hi, u32x4 v) {
@@ -704,11 +697,11 @@ __device__ __forceinline__ void storeToMore(const SG &sg, uint64_t byteOff, u32x
     for (int i = 0; i < 4; i++) q[i] = sg.outp(o + i < sg.nmore ? o + i : o);
 #pragma unroll
     for (int i = 0; i < 4; i++)
-      if (o + i < sg.nmore) stg_stream(q[i] + byteOff, v);
+      if (o + i < sg.nmore) stg_as(sg.keep, q[i] + byteOff, v);
   }
 }
 __device__ __forceinline__ void storeVector(const SegMany &sg, uint64_t byteOff, u32x4 v) {
-  stg_stream(sg.out + byteOff, v);
+  stg_as(sg.keep, sg.out + byteOff, v);
   storeToMore(sg, byteOff, v);
 }
 template <int ES>
@@ -727,6 +720,7 @@ struct SegChunk {
   uint64_t outAdj;       // the same for the extra outputs
   char *out;
   uint64_t lead, end;
+  uint32_t keep;
   int k, first, only, nmore;
   __device__ __forceinline__ int inputs() const { return only >= 0 ? 1 : k; }
   __device__ __forceinline__ const char *inp(int p) const {
@@ -740,7 +734,7 @@ struct SegChunk {
   __device__ __forceinline__ char *outp(int o) const { return asGlobal(rawOut[o]) + outAdj; }
 };
 __device__ __forceinline__ void storeVector(const SegChunk &sg, uint64_t byteOff, u32x4 v) {
-  stg_stream(sg.out + byteOff, v);
+  stg_as(sg.keep, sg.out + byteOff, v);
   storeToMore(sg, byteOff, v);
 }
 template <int ES>
@@ -749,8 +743,79 @@ __device__ __forceinline__ void storeElems(const SegChunk &sg, uint64_t e0, int 
   for (int o = 0; o < sg.nmore; o++) scatterElems<ES>(sg.outp(o), e0, lo, hi, v);
 }
 
+// ------------------------------------------------------- fold associations
+//
+// How the K input vectors of one output vector are combined.
+//   kChain      acc = in[0]; acc = acc (op) in[p], p = 1..K-1: the peer loop of
+//               flagcx/adaptor/kernel/nvidia/custom_allreduce.cu:345-359.
+//   kTree       the binomial tree of the reference's flagcxReduce
+//               (flagcx/runner/uni_runner_impl.cc:1314-1326,1372-1477), in[a] being
+//               tree rank a (rank (a + root) % n): in round i every tree rank a with
+//               more than i receive steps computes
+//               partial(a) = partial(a + 2^i) (op) partial(a), the received operand
+//               first; the result is partial(0).
+//   kKeepLocal  the host ring's chain (flagcx/service/bootstrap.cc:853-871 with the
+//               std::max / std::min of flagcx/service/include/utils.h:707-725):
+//               res = in[0]; res = in[j] (op) res, j = 1..K-1 -- the operand that is
+//               local to the rank of that step comes FIRST, so it is the one kept
+//               when the comparison is false (a NaN on either side), and a NaN met
+//               on the way hides what was folded before it exactly as on the ring.
+// In the tree and in the keep-local chain every step is a complete two-input
+// reduction in the element type (16-bit sums and products are rounded after
+// every step), as when each step is a launch of its own writing a buffer.
+enum Sched { kChain = 0, kTree = 1, kKeepLocal = 2 };
+
+// Receive steps of tree rank a among n (uni_runner_impl.cc:1314-1326): the root
+// takes ceil(log2 n); others the number of trailing zero bits of a, clipped so
+// that a + 2^i stays below n.
+__host__ __device__ constexpr int treeStepsOf(int a, int n) {
+  int total = 0;
+  while ((1 << total) < n) total++;
+  if (a == 0) return total;
+  int st = 0;
+  while (((a >> st) & 1) == 0) st++;
+  if (st && n - a <= (1 << (st - 1))) {
+    int rest = n - a - 1;
+    for (st = 0; rest; rest >>= 1) st++;
+  }
+  return st;
+}
+
+template <class R>
+__device__ __forceinline__ u32x4 combineTwo(u32x4 x, u32x4 y) {
+  typename R::Acc acc;
+  R::init(acc, x);
+  R::fold(acc, y);
+  return R::finish(acc, 2u);
+}
+
+template <class R, int K, int SCHED>
+__device__ __forceinline__ u32x4 foldVectors(u32x4 (&v)[K]) {
+  if constexpr (SCHED == kChain) {
+    typename R::Acc acc;
+    R::init(acc, v[0]);
+#pragma unroll
+    for (int p = 1; p < K; p++) R::fold(acc, v[p]);
+    return R::finish(acc, (uint32_t)K);
+  } else if constexpr (SCHED == kTree) {
+    constexpr int total = treeStepsOf(0, K);
+#pragma unroll
+    for (int i = 0; i < total; i++) {
+#pragma unroll
+      for (int a = 0; a < K; a++)   // a + 2^i takes no step in round i, so the order of a within a round is free
+        if (treeStepsOf(a, K) > i) v[a] = combineTwo<R>(v[a + (1 << i)], v[a]);
+    }
+    return v[0];
+  } else {
+    u32x4 r = v[0];
+#pragma unroll
+    for (int j = 1; j < K; j++) r = combineTwo<R>(v[j], r);
+    return r;
+  }
+}
+
 // Reduce vector j of the segment with full bounds / alignment handling.
-template <class R, int K, class SG>
+template <class R, int K, int SCHED, class SG>
 __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
   constexpr int VE = 16 / R::ES;
   const uint64_t e0 = j * VE;
@@ -758,26 +823,35 @@ __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
   const int lo = (sg.lead > e0) ? (int)(sg.lead - e0) : 0;
   const int hi = (sg.end - e0 < (uint64_t)VE) ? (int)(sg.end - e0) : VE;
   const bool full = (lo == 0 && hi == VE);
-  typename R::Acc acc;
-  const int k = sg.inputs();
   auto fetch = [&](int p) -> u32x4 {
     if (!full) return gatherElems<R::ES>(sg.inp(p), e0, lo, hi);
     return ldg_stream(sg.inp(p) + j * 16);
   };
-  R::init(acc, fetch(0));
-  // Sixteen inputs in flight at a time, folded in their order: a launch smaller than one full tile comes through
-  // here, and with a run-time k nothing else overlaps the loads -- one after the other they cost 0.3 us per input.
-  constexpr int kGroup = 16;
-  int p = 1;
-  for (; p + kGroup <= k; p += kGroup) {
-    u32x4 v[kGroup];
+  u32x4 r;
+  if constexpr (SCHED != kChain) {
+    static_assert(K > 0, "the tree and keep-local associations need a compile-time input count");
+    u32x4 v[K > 0 ? K : 1];
 #pragma unroll
-    for (int q = 0; q < kGroup; q++) v[q] = fetch(p + q);
+    for (int p = 0; p < K; p++) v[p] = fetch(p);
+    r = foldVectors<R, (K > 0 ? K : 1), SCHED>(v);
+  } else {
+    typename R::Acc acc;
+    const int k = sg.inputs();
+    R::init(acc, fetch(0));
+    // Sixteen inputs in flight at a time, folded in their order: a launch smaller than one full tile comes through
+    // here, and with a run-time k nothing else overlaps the loads -- one after the other they cost 0.3 us per input.
+    constexpr int kGroup = 16;
+    int p = 1;
+    for (; p + kGroup <= k; p += kGroup) {
+      u32x4 v[kGroup];
 #pragma unroll
-    for (int q = 0; q < kGroup; q++) R::fold(acc, v[q]);
+      for (int q = 0; q < kGroup; q++) v[q] = fetch(p + q);
+#pragma unroll
+      for (int q = 0; q < kGroup; q++) R::fold(acc, v[q]);
+    }
+    for (; p < k; p++) R::fold(acc, fetch(p));
+    r = R::finish(acc, (uint32_t)k);
   }
-  for (; p < k; p++) R::fold(acc, fetch(p));
-  u32x4 r = R::finish(acc, (uint32_t)k);
   if (full)
     storeVector(sg, j * 16, r);
   else
@@ -785,67 +859,79 @@ __device__ __forceinline__ void reduceVectorChecked(const SG &sg, uint64_t j) {
 }
 
 // Branch-free body: lane handles U whole vectors at byte offsets off + u*ustride
-// of every stream, all K*U loads in flight before the first use.  TEMPORAL picks
-// ordinary loads instead of nontemporal ones (the grouped flavour of the striped
-// zone); it is a template parameter so that the nontemporal body is compiled,
-// and scheduled, exactly as it is without it.
-template <bool TEMPORAL>
-__device__ __forceinline__ u32x4 ldg_as(const void *p) {
-  return TEMPORAL ? ldg_keep(p) : ldg_stream(p);
+// of every stream, all K*U loads in flight before the first use.  `keep` is the
+// launch's cache policy: input p is read with ordinary loads when bit p is set,
+// with nontemporal ones otherwise (the same for every lane, so the choice is a
+// scalar branch around the U loads of that input).
+template <class R, int K, int U, int SCHED, class SG>
+__device__ __forceinline__ void reduceVectorsFixed(const SG &sg, uint64_t off, uint64_t ustride, uint32_t keep) {
+  u32x4 v[U][K];
+#pragma unroll
+  for (int p = 0; p < K; p++) {
+    const char *ip = sg.inp(p) + off;
+    if ((keep >> p) & 1u) {
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u][p] = ldg_keep(ip + u * ustride);
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u][p] = ldg_stream(ip + u * ustride);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) storeVector(sg, off + u * ustride, foldVectors<R, K, SCHED>(v[u]));
 }
 
-#ifndef FX_RUNTIME_GROUP
-#define FX_RUNTIME_GROUP 4
-#endif
-constexpr int kRuntimeGroup = FX_RUNTIME_GROUP;   // inputs a lane of a run-time-k kernel keeps in flight
+constexpr int kRuntimeGroup = 4;   // inputs a lane of a run-time-k kernel keeps in flight
 
-template <class R, int K, int U, bool TEMPORAL, class SG>
-__device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, uint64_t ustride) {
-  if (K > 0) {
-    u32x4 v[U][K > 0 ? K : 1];
+template <bool KEEP>
+__device__ __forceinline__ u32x4 ldg_as(const void *p) {
+  return KEEP ? ldg_keep(p) : ldg_stream(p);
+}
+
+// The same for a run-time number of inputs, folded in their order.  The load
+// flavour is a template parameter here and the caller branches once.
+template <class R, int U, bool KEEP, class SG>
+__device__ __forceinline__ void reduceVectorsRuntime(const SG &sg, uint64_t off, uint64_t ustride) {
+  typename R::Acc acc[U];
 #pragma unroll
-    for (int u = 0; u < U; u++)
+  for (int u = 0; u < U; u++) R::init(acc[u], ldg_as<KEEP>(sg.inp(0) + off + u * ustride));
+  // kRuntimeGroup inputs in flight at a time (folded in their order): a lane that waits for
+  // every input in turn is what a small launch of many inputs spends its time on
+  const int k = sg.inputs();
+  int p = 1;
+  for (; p + kRuntimeGroup <= k; p += kRuntimeGroup) {
+    u32x4 v[kRuntimeGroup][U];
 #pragma unroll
-      for (int p = 0; p < K; p++) v[u][p] = ldg_as<TEMPORAL>(sg.inp(p) + off + u * ustride);
+    for (int q = 0; q < kRuntimeGroup; q++) {
+      const char *ip = sg.inp(p + q);
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-      typename R::Acc acc;
-      R::init(acc, v[u][0]);
-#pragma unroll
-      for (int p = 1; p < K; p++) R::fold(acc, v[u][p]);
-      storeVector(sg, off + u * ustride, R::finish(acc, (uint32_t)K));
+      for (int u = 0; u < U; u++) v[q][u] = ldg_as<KEEP>(ip + off + u * ustride);
     }
+#pragma unroll
+    for (int q = 0; q < kRuntimeGroup; q++)
+#pragma unroll
+      for (int u = 0; u < U; u++) R::fold(acc[u], v[q][u]);
+  }
+  for (; p < k; p++) {
+    const char *ip = sg.inp(p);
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = ldg_as<KEEP>(ip + off + u * ustride);
+#pragma unroll
+    for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) storeVector(sg, off + u * ustride, R::finish(acc[u], (uint32_t)sg.inputs()));
+}
+
+template <class R, int K, int U, int SCHED, class SG>
+__device__ __forceinline__ void reduceVectorsFast(const SG &sg, uint64_t off, uint64_t ustride, uint32_t keep) {
+  if constexpr (K > 0) {
+    reduceVectorsFixed<R, K, U, SCHED>(sg, off, ustride, keep);
   } else {
-    typename R::Acc acc[U];
-#pragma unroll
-    for (int u = 0; u < U; u++) R::init(acc[u], ldg_as<TEMPORAL>(sg.inp(0) + off + u * ustride));
-    // kRuntimeGroup inputs in flight at a time (folded in their order): a lane that waits for
-    // every input in turn is what a small launch of many inputs spends its time on
-    const int k = sg.inputs();
-    int p = 1;
-    for (; p + kRuntimeGroup <= k; p += kRuntimeGroup) {
-      u32x4 v[kRuntimeGroup][U];
-#pragma unroll
-      for (int q = 0; q < kRuntimeGroup; q++) {
-        const char *ip = sg.inp(p + q);
-#pragma unroll
-        for (int u = 0; u < U; u++) v[q][u] = ldg_as<TEMPORAL>(ip + off + u * ustride);
-      }
-#pragma unroll
-      for (int q = 0; q < kRuntimeGroup; q++)
-#pragma unroll
-        for (int u = 0; u < U; u++) R::fold(acc[u], v[q][u]);
-    }
-    for (; p < k; p++) {
-      const char *ip = sg.inp(p);
-      u32x4 v[U];
-#pragma unroll
-      for (int u = 0; u < U; u++) v[u] = ldg_as<TEMPORAL>(ip + off + u * ustride);
-#pragma unroll
-      for (int u = 0; u < U; u++) R::fold(acc[u], v[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < U; u++) storeVector(sg, off + u * ustride, R::finish(acc[u], (uint32_t)sg.inputs()));
+    static_assert(SCHED == kChain, "run-time input counts fold in input order only");
+    if (keep & kKeepAllLoads) reduceVectorsRuntime<R, U, true>(sg, off, ustride);
+    else reduceVectorsRuntime<R, U, false>(sg, off, ustride);
   }
 }
 
@@ -899,20 +985,19 @@ __host__ __device__ inline TileLane laneOfTile(const TilePlan &tp, uint32_t tile
 // column a tile owns in the grouped flavour): a launch whose workgroup b runs
 // tile b - first passes (b - tile) mod 8 = first mod 8, so that the grouping
 // follows the dies; a kernel that hands tiles out differently passes 0.
-template <class R, int K, int U, class SG>
+template <class R, int K, int U, class SG, int SCHED = kChain>
 __device__ __forceinline__ void reduceTile(const SG &sg, const TilePlan &tp, uint32_t tile, uint32_t xcdShift) {
   const TileLane tl = laneOfTile(tp, tile, threadIdx.x, U, xcdShift);
   if (tl.fast) {
-    // The grouped flavour only occurs for one-input segments (handOutFor).
-    if (K == 1 && tp.grouped && tile < tp.zoneTiles)
-      reduceVectorsFast<R, K, U, true>(sg, tl.j * 16, tl.stride * 16);
-    else
-      reduceVectorsFast<R, K, U, false>(sg, tl.j * 16, tl.stride * 16);
+    // The grouped flavour only occurs for one-input segments (handOutFor): its
+    // loads are ordinary ones whatever the launch's policy says.
+    const uint32_t keep = sg.keep | ((K == 1 && tp.grouped && tile < tp.zoneTiles) ? 1u : 0u);
+    reduceVectorsFast<R, K, U, SCHED>(sg, tl.j * 16, tl.stride * 16, keep);
   } else {
 #pragma unroll 1
     for (int u = 0; u < U; u++) {
       const uint64_t j = tl.j + (uint64_t)u * tl.stride;
-      if (j < tl.limit) reduceVectorChecked<R, K>(sg, j);
+      if (j < tl.limit) reduceVectorChecked<R, K, SCHED>(sg, j);
     }
   }
 }
@@ -966,6 +1051,7 @@ struct DirectArgs {
   void *out;
   uint64_t count;
   int k;
+  uint32_t keep;   // cache policy, see kKeepAllLoads
 };
 
 struct ManyArgs {
@@ -973,6 +1059,7 @@ struct ManyArgs {
   void *out[kMaxK];
   uint64_t count;
   int k, nout;
+  uint32_t keep;
   int co;   // every stream sits at out[0]'s offset within a cache line (the host has looked at all k + nout pointers)
 };
 
@@ -987,6 +1074,7 @@ __global__ void __launch_bounds__(kBlock) reduceBcastRuntime(ManyArgs a) {
   sg.lead = mis / R::ES;
   sg.end = sg.lead + a.count;
   sg.k = a.k;
+  sg.keep = a.keep;
   sg.rawOut = a.out + 1;
   sg.nmore = a.nout - 1;
   const TilePlan tp = planTiles((uint64_t)(uintptr_t)a.out[0], a.count, R::ES, U, handOutFor(a.co != 0, a.k));
@@ -1007,6 +1095,7 @@ struct ChunkedArgs {
   int8_t outSel[kMaxK];                   // >= 0: this output alone; -1: all nout
   int8_t co[kMaxK];                       // chunkCoAligned of the chunk, worked out once on the host
   int k, nout, nchunks;
+  uint32_t keep;
 };
 
 // Whether every stream of a chunk sits at the primary output's offset within a
@@ -1048,6 +1137,7 @@ __global__ void __launch_bounds__(kBlock) reduceChunksRuntime(ChunkedArgs a) {
   sg.lead = mis / R::ES;
   sg.end = sg.lead + a.cnt[c];
   sg.k = a.k;
+  sg.keep = a.keep;
   sg.first = a.first[c];
   sg.only = a.only[c];
   sg.nmore = a.outSel[c] >= 0 ? 0 : a.nout - 1;
@@ -1058,6 +1148,7 @@ __global__ void __launch_bounds__(kBlock) reduceChunksRuntime(ChunkedArgs a) {
 template <class R, int K, int U>
 __global__ void __launch_bounds__(kBlock) reduceCopyDirect(DirectArgs<K> a) {
   Seg<K> sg;
+  sg.keep = a.keep;
   const TilePlan tp = makeSeg<R::ES, U>(sg, a.in, a.out, a.count, a.k);
   reduceTile<R, K, U>(sg, tp, blockIdx.x, 0u);
 }
@@ -1083,7 +1174,7 @@ struct SliceDescK {
 
 template <int K>
 constexpr int inlineSlicesFor() {
-  return (4000 - 8) / (int)(sizeof(SliceDescK<K>) + sizeof(uint32_t));
+  return (4000 - 12) / (int)(sizeof(SliceDescK<K>) + sizeof(uint32_t));
 }
 
 // NS = 0 means as many slots as fit under 4 KiB.  A second, small size exists
@@ -1098,6 +1189,7 @@ struct InlineSliceTable {
   SliceDescK<K> d[kSlots];
   uint32_t tileStart[kSlots + 1];
   uint32_t n;
+  uint32_t keep;
 };
 
 __device__ __forceinline__ uint32_t findSlice(const uint32_t *tileStart, uint32_t n, uint32_t b) {
@@ -1110,23 +1202,24 @@ __device__ __forceinline__ uint32_t findSlice(const uint32_t *tileStart, uint32_
 }
 
 template <class R, int K, int U, class D>
-__device__ __forceinline__ void reduceSlicesBody(const D *d, const uint32_t *tileStart, uint32_t n) {
+__device__ __forceinline__ void reduceSlicesBody(const D *d, const uint32_t *tileStart, uint32_t n, uint32_t keep) {
   const uint32_t b = blockIdx.x;
   const uint32_t i = findSlice(tileStart, n, b);
   Seg<K> sg;
+  sg.keep = keep;
   const TilePlan tp = makeSeg<R::ES, U>(sg, d[i].in, d[i].out, d[i].count, K);
   reduceTile<R, K, U>(sg, tp, b - tileStart[i], tileStart[i] & 7u);
 }
 
 template <class R, int K, int U, int NS>
 __global__ void __launch_bounds__(kBlock) reduceSlicesInline(InlineSliceTable<K, NS> t) {
-  reduceSlicesBody<R, K, U>(t.d, t.tileStart, t.n);
+  reduceSlicesBody<R, K, U>(t.d, t.tileStart, t.n, t.keep);
 }
 
 template <class R, int K, int U>
 __global__ void __launch_bounds__(kBlock)
-reduceSlicesTable(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n) {
-  reduceSlicesBody<R, K, U>(d, tileStart, n);
+reduceSlicesTable(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n, uint32_t keep) {
+  reduceSlicesBody<R, K, U>(d, tileStart, n, keep);
 }
 
 // All-to-all of equal blocks over up to kMaxK ranks in one launch: block (r, i)
@@ -1142,6 +1235,7 @@ struct AllToAllArgs {
   uint64_t blockElems;      // elements of the kernel's copy type per block
   uint32_t tilesPerBlock;
   int n;
+  uint32_t keep;
 };
 
 template <class R, int U>
@@ -1152,6 +1246,7 @@ __global__ void __launch_bounds__(kBlock) allToAllBlocks(AllToAllArgs a) {
   const void *in = (const char *)a.send[r] + (uint64_t)i * bytes;
   void *out = (char *)a.recv[i] + (uint64_t)r * bytes;
   Seg<1> sg;
+  sg.keep = a.keep;
   const TilePlan tp = makeSeg<R::ES, U>(sg, &in, out, a.blockElems, 1);
   if (tile >= tp.tiles()) return;
   reduceTile<R, 1, U>(sg, tp, tile, (blockIdx.x - tile) & 7u);
@@ -1168,22 +1263,27 @@ struct BcastDescDev {
 
 // Two table sizes: the kernel-argument block is copied at every launch (about
 // 0.3 us per KiB), and the common case -- a whole all-reduce merged into one
-// descriptor -- should not carry fifteen empty slots.
-constexpr int kInlineBcast = 16;
+// descriptor -- should not carry seven empty slots.  Eight slots hold one
+// descriptor per chunk of a collective over eight ranks.
+constexpr int kInlineBcast = 8;
 
 template <int NS>
 struct InlineBcastTable {
   BcastDescDev d[NS];
   uint32_t tileStart[NS + 1];
   uint32_t n;
+  uint32_t keep;
 };
 
-template <class R, int K, int U, int NS>
+// SCHED other than kChain: the same launch with the inputs combined in the
+// reference's tree or host-ring association (see Sched).
+template <class R, int K, int U, int NS, int SCHED = kChain>
 __global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable<NS> t) {
   const uint32_t b = blockIdx.x;
   const uint32_t i = findSlice(t.tileStart, t.n, b);
   const BcastDescDev &d = t.d[i];
   SegB<K> sg;
+  sg.keep = t.keep;
   const uint64_t mis = (uint64_t)(uintptr_t)d.out[0] & 15u;
   sg.nmore = (int)d.nout - 1;
   bool co = true;   // every output at the same place in its cache line, or the striped pieces would split lines
@@ -1193,7 +1293,7 @@ __global__ void __launch_bounds__(kBlock) reduceBcastInline(InlineBcastTable<NS>
     if (o < sg.nmore) co = co && sameLinePhase((uint64_t)(uintptr_t)d.out[o + 1], (uint64_t)(uintptr_t)d.out[0]);
   }
   const TilePlan tp = makeSeg<R::ES, U>(static_cast<Seg<K> &>(sg), d.in, d.out[0], d.count, K, co);
-  reduceTile<R, K, U>(sg, tp, b - t.tileStart[i], t.tileStart[i] & 7u);
+  reduceTile<R, K, U, SegB<K>, SCHED>(sg, tp, b - t.tileStart[i], t.tileStart[i] & 7u);
 }
 
 }  // namespace fx

@@ -3,9 +3,9 @@
 #include "fx_launch.hpp"
 namespace fx {
 const KernelSet *kernelSetsElem() {
-  static const KernelSet sets[6] = {makeSet<RedElem<flagcxFloat16, flagcxSum>>(),  makeSet<RedElem<flagcxFloat16, flagcxMax>>(),
-                                    makeSet<RedElem<flagcxFloat16, flagcxMin>>(),  makeSet<RedElem<flagcxBfloat16, flagcxSum>>(),
-                                    makeSet<RedElem<flagcxBfloat16, flagcxMax>>(), makeSet<RedElem<flagcxBfloat16, flagcxMin>>()};
+  static const KernelSet sets[6] = {makeSet<RedElem<flagcxFloat16, flagcxSum>, true>(),  makeSet<RedElem<flagcxFloat16, flagcxMax>, true>(),
+                                    makeSet<RedElem<flagcxFloat16, flagcxMin>, true>(),  makeSet<RedElem<flagcxBfloat16, flagcxSum>, true>(),
+                                    makeSet<RedElem<flagcxBfloat16, flagcxMax>, true>(), makeSet<RedElem<flagcxBfloat16, flagcxMin>, true>()};
   return sets;
 }
 }  // namespace fx

@@ -301,6 +301,31 @@ struct HostPiece {
 flagcxResult_t chainHostPieces(const Ctx &c, const std::vector<HostPiece> &pieces) {
   Group *g = c.g;
   const int n = c.n;
+  // Up to eight ranks: the whole chain of a piece in registers, one launch for
+  // all pieces, every input read once (in[0] = rank c+1's data, in[j] = the
+  // local operand of step j).  Outputs that do not share their offset within 16
+  // bytes fall through to the step-by-step form below.
+  if (n <= FX_MAX_SLICE_INPUTS) {
+    BcastList bd;
+    bool alike = true;
+    int nout = 1;
+    for (const HostPiece &p : pieces) {
+      if (p.cnt == 0) continue;
+      nout = (int)p.outs.size();
+      if (nout > FX_MAX_SLICE_INPUTS) alike = false;
+      fxBcastDesc d;
+      memset(&d, 0, sizeof(d));
+      for (int j = 0; j < n; j++) d.in[j] = cadd(c.send(mod(p.chunk + 1 + j, n)), p.off * c.ts);
+      for (int o = 0; o < nout && o < FX_MAX_SLICE_INPUTS; o++) {
+        d.out[o] = p.outs[o];
+        alike = alike && ((((uintptr_t)p.outs[o] ^ (uintptr_t)p.outs[0]) & 15u) == 0);
+      }
+      d.count = p.cnt;
+      bd.push_back(d);
+    }
+    if (bd.empty()) return flagcxSuccess;
+    if (alike) return R(fx_reduce_ordered(bd.data(), bd.size(), n, nout, g->dtype, g->op, FX_FOLD_KEEP_LOCAL, c.s));
+  }
   std::vector<size_t> soff(pieces.size(), 0);
   size_t total = 0;
   for (size_t i = 0; i < pieces.size(); i++) {
@@ -556,8 +581,18 @@ flagcxResult_t runReduce(const Ctx &c) {
     return R(fx_reduce_copy(c.recv(root), in.data(), n, count, g->dtype, g->op, 0, c.s));
   }
   // Tree order: round i, every tree rank a with more than i receive steps
-  // computes partial(a) = partial(a + 2^i) (op) partial(a).  Partials live in a
-  // per-rank scratch row; the root's last round writes recvbuff.
+  // computes partial(a) = partial(a + 2^i) (op) partial(a).  Up to eight ranks
+  // that is one launch that keeps the partials in registers (in[a] = tree rank
+  // a's data); beyond, partials live in a per-rank scratch row, one launch per
+  // round, and the root's last round writes recvbuff.
+  if (n <= FX_MAX_SLICE_INPUTS) {
+    fxBcastDesc d;
+    memset(&d, 0, sizeof(d));
+    for (int a = 0; a < n; a++) d.in[a] = c.send(mod(a + root, n));
+    d.out[0] = c.recv(root);
+    d.count = count;
+    return R(fx_reduce_ordered(&d, 1, n, 1, g->dtype, g->op, FX_FOLD_TREE, c.s));
+  }
   flagcxResult_t rc = ensureScratch(g, (size_t)n * count * ts, c.s);
   if (rc != flagcxSuccess) return rc;
   const int total = treeSteps(0, n);

@@ -50,6 +50,23 @@ def reduce_bcast_slices(descs, k, nout, dtype, op, stream=None):
     return lib.fx_reduce_bcast_slices(arr, len(descs), k, nout, dtype, op, stream)
 
 
+FOLD_CHAIN, FOLD_TREE, FOLD_KEEP_LOCAL = 0, 1, 2   # include/flagcx_amd/fx_kernels.h
+
+
+def reduce_ordered(descs, k, nout, dtype, op, order, stream=None):
+    """descs as for reduce_bcast_slices; the k inputs of every slice are combined in the given
+    association (FOLD_TREE: ins[a] = tree rank a; FOLD_KEEP_LOCAL: ins[0] first, then ins[j] (op) res)."""
+    descs = list(descs)
+    arr = (N.BcastDesc * max(len(descs), 1))()
+    for i, (ins, outs, count) in enumerate(descs):
+        for p, ptr in enumerate(ins):
+            arr[i].inp[p] = ptr
+        for o, ptr in enumerate(outs):
+            arr[i].out[o] = ptr
+        arr[i].count = count
+    return lib.fx_reduce_ordered(arr, len(descs), k, nout, dtype, op, order, stream)
+
+
 def reduce_bcast(outs, ins, count, dtype, op, first=0, stream=None):
     """One segment, up to 64 inputs folded once into up to 64 outputs; op = -1 copies ins[0] (count in bytes)."""
     return lib.fx_reduce_bcast(_ptr_array(outs), len(outs), _ptr_array(ins), len(ins), count, dtype, op, first, stream)

@@ -7,6 +7,14 @@ algBw = bytes / 1e9 / t).  Usage:
     python -m flagcx_amd.perf pack              # BASELINE.json configs[3]: alltoallv pack / unpack
     python -m flagcx_amd.perf allreduce -n 8 -d bf16 -b 1M -e 64M [--graph]
     python -m flagcx_amd.perf fifo -b 4K -e 256M -f 8   # round trips through the reduce FIFO
+    python -m flagcx_amd.perf coldstart         # library sizes and the first call's latency (code-object load)
+
+Warm and cold.  Every figure is "warm" unless --cold is given: the same buffers
+are used launch after launch, so whatever of them fits MI355X's 256 MiB
+memory-side cache is served from it.  With --cold (reduce, slices, pack) every
+timed launch is preceded by a 1 GiB fill with ordinary stores that pushes the
+operands out of that cache, and is timed by its own pair of events; both
+columns are printed.
 """
 import argparse
 import sys
@@ -55,9 +63,43 @@ class Timer:
             d.event_destroy(e1)
         return sorted(rounds)[1]
 
+    SCRUB_BYTES = 1 << 30
+
+    def ms_cold(self, fn, launches=9):
+        """Milliseconds per call when the caches hold nothing of the operands: before
+        every timed call a 1 GiB fill with ordinary stores (the runtime's memset
+        kernel, four times the memory-side cache) runs on the same stream; each call
+        is timed by its own pair of events; the median of `launches` calls."""
+        d = self.dev
+        if not hasattr(self, "scrub"):
+            self.scrub = d.malloc(self.SCRUB_BYTES)
+        fn()
+        d.stream_sync(self.stream)
+        each = []
+        for i in range(launches):
+            d.memset(self.scrub, i & 0xff, self.SCRUB_BYTES, self.stream)
+            e0, e1 = d.event_create(), d.event_create()
+            d.event_record(e0, self.stream)
+            fn()
+            d.event_record(e1, self.stream)
+            d.event_sync(e1)
+            each.append(d.event_ms(e0, e1))
+            d.event_destroy(e0)
+            d.event_destroy(e1)
+        return sorted(each)[len(each) // 2]
+
+    def both(self, fn, cold):
+        """(warm ms, cold ms or None)."""
+        return self.ms(fn), (self.ms_cold(fn) if cold else None)
+
 
 def row(label, nbytes, ms, algo_bytes):
-    print(f"{label:<44s} size {nbytes:>12d} B   {ms * 1e3:10.2f} us   {algo_bytes / ms / 1e6:9.1f} GB/s", flush=True)
+    """ms: milliseconds, or (warm ms, cold ms or None) from Timer.both."""
+    warm, cold = ms if isinstance(ms, tuple) else (ms, None)
+    line = f"{label:<44s} size {nbytes:>12d} B   {warm * 1e3:10.2f} us   {algo_bytes / warm / 1e6:9.1f} GB/s"
+    if cold is not None:
+        line += f"   | cold {cold * 1e3:10.2f} us   {algo_bytes / cold / 1e6:9.1f} GB/s"
+    print(line, flush=True)
 
 
 def run_reduce(dev, a):
@@ -83,7 +125,7 @@ def run_reduce(dev, a):
         fn = lambda: N.check(K.reduce_copy(out + (0 if a.inplace else a.misalign * es),
                                            [p + (a.misalign * es if not a.mixed else s) for p, s in zip(ins, shift)]
                                            if not a.inplace else ins, n, dtype, op, 0, t.raw))
-        row(f"reduce k={k} {a.dtype} {a.op}{' inplace' if a.inplace else ''}", nbytes, t.ms(fn), (k + 1) * nbytes)
+        row(f"reduce k={k} {a.dtype} {a.op}{' inplace' if a.inplace else ''}", nbytes, t.both(fn, a.cold), (k + 1) * nbytes)
         nbytes *= a.factor
 
 
@@ -120,13 +162,13 @@ def run_slices(dev, a):
         arr, cnt = K.make_slices(([s], d, b) for s, d, b in descs)
         return lambda: N.check(N.lib.fx_copy_slices(arr, cnt, t.raw))
 
-    row("one rank share: 16 x 512 KiB, 8-way", share_bytes, t.ms(reducer(one)), 9 * share_bytes)
+    row("one rank share: 16 x 512 KiB, 8-way", share_bytes, t.both(reducer(one), a.cold), 9 * share_bytes)
     allr = [d for r in per_rank for d in r]
-    row("all 8 shares: 128 x 512 KiB, 8-way", n * es, t.ms(reducer(allr)), 9 * n * es)
+    row("all 8 shares: 128 x 512 KiB, 8-way", n * es, t.both(reducer(allr), a.cold), 9 * n * es)
     plan = K.Plan(allr, k, N.DT_BF16, N.OP_SUM)
-    row("all 8 shares as a device-resident plan", n * es, t.ms(lambda: N.check(plan.launch(t.raw))), 9 * n * es)
+    row("all 8 shares as a device-resident plan", n * es, t.both(lambda: N.check(plan.launch(t.raw)), a.cold), 9 * n * es)
     onechunk = [([p for p in ds], dr[0], n // k)]
-    row("one share as ONE contiguous slice", share_bytes, t.ms(reducer(onechunk)), 9 * share_bytes)
+    row("one share as ONE contiguous slice", share_bytes, t.both(reducer(onechunk), a.cold), 9 * share_bytes)
     # ring-faithful: 7 successive 2-input steps over the share (reported, not the target)
     steps = [[([ds[0] + o, ds[1] + o], dr[0] + o, c) for (ins_, _, c), o in
               zip(one, [d[1] - dr[-1 % k] for d in one])]]
@@ -134,8 +176,8 @@ def run_slices(dev, a):
     step = reducer(two, 2)
     row("ring-faithful: 7 x (16 x 512 KiB, 2-input)", share_bytes, t.ms(lambda: [step() for _ in range(7)]), 7 * 3 * share_bytes)
     one_rank_ag = [c for c in copies if c[1] - dr[0] >= 0 and c[1] - dr[0] < n * es]
-    row("all-gather copy, one rank: 7 x 8 MiB", 7 * share_bytes, t.ms(copier(one_rank_ag)), 2 * 7 * share_bytes)
-    row("all-gather copy, all ranks: 56 x 8 MiB", 56 * share_bytes, t.ms(copier(copies)), 2 * 56 * share_bytes)
+    row("all-gather copy, one rank: 7 x 8 MiB", 7 * share_bytes, t.both(copier(one_rank_ag), a.cold), 2 * 7 * share_bytes)
+    row("all-gather copy, all ranks: 56 x 8 MiB", 56 * share_bytes, t.both(copier(copies), a.cold), 2 * 56 * share_bytes)
     with S.SimGroup(k, nslices=8, redslicesize=262144) as g:
         row("flagcxAllReduce, 8 simulated ranks, 64 MiB", n * es,
             t.ms(lambda: N.check(g.all_reduce(ds, dr, n, N.DT_BF16, N.OP_SUM, t.stream))), 9 * n * es + 2 * 56 * share_bytes)
@@ -149,8 +191,8 @@ def run_pack(dev, a):
     dsend, dpacked, drecv = dev.malloc(slen * 4), dev.malloc(total * 4), dev.malloc(rlen * 4)
     dev.memset(dsend, 1, slen * 4)
     print("counts", counts, "sdispls % 4 el:", [d % 4 for d in sd], "slots % 4:", [int(x) % 4 for x in np.cumsum([0] + counts[:-1])])
-    row("pack   (config 4 layout)", total * 4, t.ms(lambda: N.check(K.pack(dpacked, dsend, counts, sd, N.DT_FP32, t.raw))), 2 * total * 4)
-    row("unpack (config 4 layout)", total * 4, t.ms(lambda: N.check(K.unpack(drecv, dpacked, counts, rd, N.DT_FP32, t.raw))), 2 * total * 4)
+    row("pack   (config 4 layout)", total * 4, t.both(lambda: N.check(K.pack(dpacked, dsend, counts, sd, N.DT_FP32, t.raw)), a.cold), 2 * total * 4)
+    row("unpack (config 4 layout)", total * 4, t.both(lambda: N.check(K.unpack(drecv, dpacked, counts, rd, N.DT_FP32, t.raw)), a.cold), 2 * total * 4)
     c4 = [c // 4 * 4 for c in counts]
     s4 = [d // 4 * 4 for d in sd]
     row("pack, counts/displs multiples of 16 B", sum(c4) * 4, t.ms(lambda: N.check(K.pack(dpacked, dsend, c4, s4, N.DT_FP32, t.raw))), 2 * sum(c4) * 4)
@@ -158,7 +200,7 @@ def run_pack(dev, a):
     bd = [i * 4_194_304 + 0 for i in range(8)]
     dbig, dpk = dev.malloc(8 * 4_194_304 * 4 + 64), dev.malloc(8 * 4_194_304 * 4)
     dev.memset(dbig, 2, 8 * 4_194_304 * 4 + 64)
-    row("pack, 8 x 4,194,304 el aligned", sum(big) * 4, t.ms(lambda: N.check(K.pack(dpk, dbig, big, bd, N.DT_FP32, t.raw))), 2 * sum(big) * 4)
+    row("pack, 8 x 4,194,304 el aligned", sum(big) * 4, t.both(lambda: N.check(K.pack(dpk, dbig, big, bd, N.DT_FP32, t.raw)), a.cold), 2 * sum(big) * 4)
     row("pack, 8 x 4,194,304 el, source off by 1 el", sum(big) * 4,
         t.ms(lambda: N.check(K.pack(dpk, dbig + 4, big, bd, N.DT_FP32, t.raw))), 2 * sum(big) * 4)
 
@@ -372,9 +414,60 @@ def run_torchref():
     row("torch.sum(stacked [8, n] bf16, 0, out=)", 512 << 20, ms_of(lambda: torch.sum(st, 0, out=out), 10), 9 * (512 << 20))
 
 
+COLDSTART_CHILD = r"""
+import ctypes as C, json, os, sys, time
+t0 = time.perf_counter()
+from flagcx_amd import _native as N
+from flagcx_amd import kernels as K
+from flagcx_amd.adaptor import Device
+t_import = time.perf_counter() - t0
+dev = Device(0)
+n = 1 << 20
+out = {"import_and_dlopen_ms": round(t_import * 1e3, 2), "first_calls": []}
+t0 = time.perf_counter()
+bufs = [dev.malloc(n * 8) for _ in range(3)]
+dev.sync()
+out["runtime_init_and_3_mallocs_ms"] = round((time.perf_counter() - t0) * 1e3, 2)
+for name, dt in (("bf16", N.DT_BF16), ("bf16 again", N.DT_BF16), ("fp32", N.DT_FP32), ("uint8", N.DT_UINT8), ("copy", None)):
+    t0 = time.perf_counter()
+    if dt is None:
+        N.check(K.copy_slices([(bufs[0], bufs[2], n)]))
+    else:
+        N.check(K.reduce_copy(bufs[2], bufs[:2], n, dt, N.OP_SUM))
+    dev.sync()
+    out["first_calls"].append({"what": name, "ms": round((time.perf_counter() - t0) * 1e3, 3)})
+print(json.dumps(out))
+"""
+
+
+def run_coldstart():
+    """Sizes of the libraries and what the first call of a kind costs in a fresh
+    process: every element type is a code object of its own inside
+    libflagcx-kernels-mi355x.so, loaded (and decompressed) by the HIP runtime at the
+    first launch of one of its kernels."""
+    import json
+    import os
+    import subprocess
+    for f in sorted(os.listdir(N.LIB_DIR)):
+        print(f"{f:<36s} {os.path.getsize(os.path.join(N.LIB_DIR, f)) / (1 << 20):8.2f} MiB")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for run in range(3):
+        r = subprocess.run([sys.executable, "-c", COLDSTART_CHILD], capture_output=True, text=True, cwd=root)
+        if r.returncode != 0:
+            print(r.stdout + r.stderr)
+            return 1
+        o = json.loads(r.stdout.strip().splitlines()[-1])
+        calls = "  ".join(f"{c['what']} {c['ms']:.2f}" for c in o["first_calls"])
+        print(f"fresh process {run}: import+dlopen {o['import_and_dlopen_ms']:.1f} ms, runtime init + 3 mallocs "
+              f"{o['runtime_init_and_3_mallocs_ms']:.1f} ms, first calls (ms incl. sync): {calls}", flush=True)
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo", "collectives", "torchref"])
+    ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo", "collectives", "torchref", "coldstart"])
+    ap.add_argument("--cold", action="store_true",
+                    help="reduce / slices / pack: also time every launch after a 1 GiB fill that empties the caches")
     ap.add_argument("-k", type=int, default=4)
     ap.add_argument("-n", "--nranks", type=int, default=8)
     ap.add_argument("-d", "--dtype", default="fp32", choices=list(DT))
@@ -394,6 +487,8 @@ def main(argv=None):
     a = ap.parse_args(argv)
     if a.what == "torchref":         # torch brings its own HIP runtime: nothing of this library is loaded beside it
         return run_torchref()
+    if a.what == "coldstart":
+        return run_coldstart()
     dev = Device(0)
     {"reduce": run_reduce, "slices": run_slices, "pack": run_pack, "allreduce": run_allreduce,
      "fifo": run_fifo, "collectives": run_collectives}[a.what](dev, a)

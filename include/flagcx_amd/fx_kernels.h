@@ -204,6 +204,38 @@ int fx_reduce_bcast_slices(const fxBcastDesc *slices, size_t n, int k, int nout,
                            int dtype, int op, void *stream);
 
 /*
+ * The same with the k inputs of every slice combined in another association
+ * than the input-order fold -- the two the reference's own multi-step paths
+ * produce -- in ONE launch, every input read once:
+ *   FX_FOLD_CHAIN       in[0] (op) in[1] (op) ... left to right (what
+ *                       fx_reduce_bcast_slices does).
+ *   FX_FOLD_TREE        the binomial tree of flagcxReduce through the uniRunner
+ *                       (flagcx/runner/uni_runner_impl.cc:1314-1326,1372-1477):
+ *                       in[a] is tree rank a, i.e. rank (a + root) % n; in round i
+ *                       every tree rank a with more than i receive steps computes
+ *                       partial(a) = partial(a + 2^i) (op) partial(a), received
+ *                       operand first; the result is partial(0).
+ *   FX_FOLD_KEEP_LOCAL  the host ring's chain (flagcx/service/bootstrap.cc:853-871
+ *                       with std::max / std::min, flagcx/service/include/utils.h:
+ *                       707-725): res = in[0]; res = in[j] (op) res for j = 1..k-1,
+ *                       the step's local operand first, so that a NaN hides what
+ *                       was folded before it exactly as on the ring.
+ * Every step of the tree and of the keep-local chain is a complete two-input
+ * reduction in the element type (16-bit sums and products are rounded after
+ * every step), as when each step is a launch of its own.  flagcxAvg with an
+ * order other than FX_FOLD_CHAIN is flagcxNotSupported (a mean is not a tree of
+ * two-input means), as are FX_OP_ELEMENT_FOLD and FX_FOLD_KEEP_LOCAL sums or
+ * products of three or more fp16 / bf16 inputs (types the host ring does not
+ * carry, flagcx/service/include/utils.h:690-694).  With FX_FOLD_TREE or
+ * FX_FOLD_KEEP_LOCAL and three or more floating-point inputs, all outputs of a
+ * slice must share out[0]'s alignment within 16 bytes (flagcxInvalidArgument
+ * otherwise).
+ */
+enum { FX_FOLD_CHAIN = 0, FX_FOLD_TREE = 1, FX_FOLD_KEEP_LOCAL = 2 };
+int fx_reduce_ordered(const fxBcastDesc *slices, size_t n, int k, int nout,
+                      int dtype, int op, int order, void *stream);
+
+/*
  * The same for ONE segment with up to FX_MAX_INPUTS inputs and FX_MAX_INPUTS
  * outputs: outs[0..nout) all receive the fold of ins[first], ins[first+1], ...
  * (wrapping), in one launch and with (k + nout) * size bytes of traffic.  This
@@ -318,5 +350,25 @@ const char *fx_version(void);
 
 #ifdef __cplusplus
 }
+
+/*
+ * The reference's own launcher of the trigger-ring consumer, under its own
+ * name, signature and C++ linkage (declared in
+ * flagcx/include/flagcx_kernel_internal.h:56, defined in
+ * flagcx/adaptor/kernel/nvidia/flagcx_reduce_kernel_device.cu:188-192, called
+ * by runUniRunner, flagcx/runner/uni_runner_impl.cc:1872-1874), so that the
+ * reference's scheduler links against libflagcx-kernels-mi355x.so and runs
+ * without a source change.  fifoBuffer is hostGetDevicePointer() of the pinned
+ * ring; the capacity is read from word 0 of the ring.  nthreads and nblocks
+ * are accepted and ignored (this consumer sizes itself to the device, see
+ * fx_fifo_consumer_create).  The kernel ends when the ring's terminate word is
+ * set and the ring is drained; the bound every wait in it carries is
+ * FX_FIFO_MAX_IDLE_POLLS polls of an idle ring (environment; default 2^36).
+ * FX_FIFO_IN_ORDER, FX_FIFO_WGS and FX_FIFO_WGS_PER_CU apply as for
+ * fx_fifo_consumer_create.  The device memory one launch needs comes from a
+ * per-device pool and goes back to it when the kernel has ended.  Failures are
+ * reported on stderr (the signature has no result).
+ */
+void flagcxLaunchCollectiveKernel(void *fifoBuffer, size_t nthreads, size_t nblocks, flagcxStream_t stream);
 #endif
 #endif /* FLAGCX_AMD_FX_KERNELS_H_ */

@@ -29,11 +29,15 @@ def _declared_functions():
     return names
 
 
+# Declared with C++ linkage, as the reference declares it (flagcx_kernel_internal.h:56): exported under its mangled name.
+CXX_LINKAGE = {"flagcxLaunchCollectiveKernel": "_Z28flagcxLaunchCollectiveKernelPvmmP12flagcxStream"}
+
+
 def test_kernel_library_exports_every_declared_symbol():
     declared = _declared_functions()
     assert {"fx_reduce_copy", "fx_reduce_slices", "fx_pack", "flagcxAllReduce", "flagcxCustomAllReduceImpl",
-            "fx_synth_fill", "fx_part_ring_ar"} <= declared
-    missing = [n for n in sorted(declared) if not hasattr(N.lib, n)]
+            "fx_synth_fill", "fx_part_ring_ar", "fx_reduce_ordered", "flagcxLaunchCollectiveKernel"} <= declared
+    missing = [n for n in sorted(declared) if not hasattr(N.lib, CXX_LINKAGE.get(n, n))]
     assert not missing, f"declared in include/ but not exported: {missing}"
     assert set(N.exported_symbols()) <= declared          # the binding uses nothing undeclared
 
@@ -41,12 +45,15 @@ def test_kernel_library_exports_every_declared_symbol():
 def test_kernels_only_library_exports_fx_and_nothing_flagcx():
     """The library a FlagCX build links into libflagcx.so must not bring a second
     flagcxAllReduce: it exports every fx_* function of the kernel header and of
-    the partition API, and no other dynamic symbol."""
+    the partition API, the reference-named consumer launcher, and no other
+    dynamic symbol."""
     import subprocess
     path = os.path.join(N.LIB_DIR, "libflagcx-kernels-mi355x.so")
     out = subprocess.run(["nm", "-D", "--defined-only", path], check=True, capture_output=True, text=True).stdout
     exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
-    assert exported and all(s.startswith("fx_") for s in exported), sorted(exported)[:10]
+    launcher = CXX_LINKAGE["flagcxLaunchCollectiveKernel"]   # the one symbol FlagCX's scheduler calls by name
+    assert launcher in exported
+    assert all(s.startswith("fx_") for s in exported - {launcher}), sorted(exported)[:10]
     wanted = {n for n in _declared_functions() if n.startswith("fx_") and n != "fx_synth_fill"}
     assert wanted <= exported, sorted(wanted - exported)
     lib = C.CDLL(path)
@@ -293,6 +300,33 @@ def test_reduce_fifo_producer_loop_against_a_host_side_consumer():
     assert N.lib.fx_fifo_run_batch(buf, trig, 0, 1000) == N.SUCCESS
 
 
+def test_scheduler_stand_in_takes_one_symbol_from_the_kernel_library(tmp_path):
+    """tests/unirunner_client.cc declares flagcxLaunchCollectiveKernel exactly as
+    the reference's header does and carries its own host side of the ring, as
+    libflagcx.so does: linked against libflagcx-kernels-mi355x.so alone it must
+    leave no symbol undefined, and the launcher must be the only symbol it takes
+    from that library.  (The GPU tests run the copy of it that the build made.)"""
+    import shutil
+    import subprocess
+    if not shutil.which("g++"):
+        pytest.skip("no g++")
+    exe = tmp_path / "unirunner_client"
+    subprocess.run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-Werror", f"-I{ROOT}/include",
+                    f"{ROOT}/tests/unirunner_client.cc", "-o", str(exe), f"-L{N.LIB_DIR}", "-lflagcx-kernels-mi355x",
+                    "-ldl", "-Wl,--no-undefined", f"-Wl,-rpath,{N.LIB_DIR}", "-Wl,-rpath-link,/opt/rocm/lib"], check=True)
+    out = subprocess.run(["nm", "-D", "--undefined-only", str(exe)], check=True, capture_output=True, text=True).stdout
+    undefined = {line.split()[-1].split("@")[0] for line in out.splitlines() if line.strip()}
+    ours = {u for u in undefined if u.startswith("fx_") or "flagcx" in u}
+    assert ours == {CXX_LINKAGE["flagcxLaunchCollectiveKernel"]}, sorted(ours)
+    src = open(f"{ROOT}/tests/unirunner_client.cc").read()
+    ref = "/root/reference/flagcx/include/flagcx_kernel_internal.h"
+    if os.path.exists(ref):          # the prototype is the reference's, token for token
+        want = re.search(r"void flagcxLaunchCollectiveKernel\([^;]*;", open(ref).read(), flags=re.S).group(0)
+        assert " ".join(want.split()) in " ".join(src.split())
+    built = os.path.join(N.LIB_DIR, "unirunner_client")
+    assert os.path.exists(built), "the build did not leave flagcx_amd/lib/unirunner_client for the GPU tests"
+
+
 def test_headers_are_plain_c_and_a_c_client_links(tmp_path):
     """The boundary is a C ABI: every header compiles as strict C11, a C program
     links against the kernel library and the host-only entry points answer."""
@@ -358,8 +392,8 @@ int main(void) {
     exe = tmp_path / "client"
     libdir = os.path.join(root, "flagcx_amd", "lib")
     subprocess.run(["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{root}/include", str(src), "-o",
-                    str(exe), f"-L{libdir}", "-lflagcx_amd", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"],
-                   check=True)
+                    str(exe), f"-L{libdir}", "-lflagcx_amd", "-lflagcx-kernels-mi355x", f"-Wl,-rpath,{libdir}",
+                    "-Wl,-rpath,/opt/rocm/lib"], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
     assert "flagcx_amd" in out
 

@@ -120,26 +120,32 @@ def test_reduce_reducescatter_allgather(dev, stream):
             assert np.array_equal(dev.to_host(dg[r], n * rc, np.float32), want)
 
 
-@pytest.mark.parametrize("n", [2, 3, 5, 6, 8])
-def test_reduce_in_tree_order_matches_the_reference_tree(dev, stream, n):
+@pytest.mark.parametrize("dname", ["fp32", "bf16"])
+@pytest.mark.parametrize("n", [2, 3, 5, 6, 8, 11])
+def test_reduce_in_tree_order_matches_the_reference_tree(dev, stream, n, dname):
     """flagcxReduce through the reference's uniRunner is a binomial tree
-    (uni_runner_impl.cc:1266-1557); fp32 sums must match it bit for bit when that
-    order is asked for, for every root, in place and out of place."""
+    (uni_runner_impl.cc:1266-1557); sums must match it bit for bit when that
+    order is asked for, for every root, in place and out of place -- fp32, and
+    bf16 where every step of the tree rounds to the element type.  Up to eight
+    ranks run as one launch, eleven as one launch per round."""
     count = 70003
-    sends = seeded_inputs(N.DT_FP32, n, count, seed=n)
+    dtype = DTYPES[dname]
+    es, npdt = N.DTYPE_SIZE[dtype], N.NP_DTYPE[dtype]
+    bits = np.uint32 if es == 4 else np.uint16
+    sends = seeded_inputs(dtype, n, count, seed=n)
     for root in sorted({0, 1 % n, n - 1}):
         for op in (N.OP_SUM, N.OP_PROD):
-            want = O.tree_reduce(sends, root, N.DT_FP32, op)
+            want = O.tree_reduce(sends, root, dtype, op)
             with DevBufs(dev) as b, S.SimGroup(n, order=2) as g:      # FX_ORDER_TREE
                 ds = [b.put(a) for a in sends]
-                dout = b.alloc(count * 4)
-                N.check(g.reduce(ds, [dout if r == root else None for r in range(n)], count, N.DT_FP32, op, root, stream))
+                dout = b.alloc(count * es)
+                N.check(g.reduce(ds, [dout if r == root else None for r in range(n)], count, dtype, op, root, stream))
                 dev.stream_sync(stream)
-                assert_parity(dev.to_host(dout, count, np.float32), want, N.DT_FP32, op, f"tree n={n} root={root}")
-                N.check(g.reduce(ds, [ds[r] if r == root else None for r in range(n)], count, N.DT_FP32, op, root, stream))
+                assert np.array_equal(dev.to_host(dout, count, npdt).view(bits), want.view(bits)), f"tree n={n} root={root}"
+                N.check(g.reduce(ds, [ds[r] if r == root else None for r in range(n)], count, dtype, op, root, stream))
                 dev.stream_sync(stream)
-                assert_parity(dev.to_host(ds[root], count, np.float32), want, N.DT_FP32, op, "tree in place")
-    if n > 3:   # and it is a different association from the rank-order fold
+                assert np.array_equal(dev.to_host(ds[root], count, npdt).view(bits), want.view(bits)), "tree in place"
+    if n > 3 and dname == "fp32":   # and it is a different association from the rank-order fold
         a = O.tree_reduce(sends, 0, N.DT_FP32, N.OP_SUM)
         assert not np.array_equal(a.view(np.uint32), O.reduce_copy(sends, N.DT_FP32, N.OP_SUM).view(np.uint32))
 

@@ -114,7 +114,8 @@ def test_simulated_rank_allreduce_replays_correctly_in_a_graph(dev):
 
 
 def test_scratch_users_capture_cold_after_a_reservation(dev):
-    """Tree-order reduce, ring reduce-scatter and in-place all-to-all need scratch.
+    """Ring reduce-scatter, in-place all-to-all and the tree-order reduce of more
+    than eight ranks need scratch.
     With the scratch reserved at set-up (fxSimCommConfig FX_SIM_SCRATCH_BYTES) their
     very first call may be inside a capture -- no eager call beforehand -- and the
     graph replays correctly on new data; without a reservation the same call is
@@ -131,16 +132,19 @@ def test_scratch_users_capture_cold_after_a_reservation(dev):
         dp = [b.alloc(count // n * 4) for _ in range(n)]
         da = [b.put(a) for a in sends]                       # all-to-all runs in place on these
         graph, gexec = C.c_void_p(), C.c_void_p()
-        # no reservation: refused under capture (nothing is enqueued), fine eagerly
-        with S.SimGroup(n, order=S.ORDER_TREE) as g:
+        # no reservation: a call that needs scratch is refused under capture (nothing is enqueued), fine eagerly;
+        # the tree-order reduce of up to eight ranks keeps its partials in registers and needs none
+        with S.SimGroup(n, order=S.ORDER_TREE, algo=S.ALGO_RING) as g:
             assert hip.hipStreamBeginCapture(raw, 0) == 0
             try:
-                rc = g.reduce(ds, [droot] * n, count, dtype, N.OP_SUM, 2, stream)
+                rc = g.reduce_scatter(ds, dp, count // n, dtype, N.OP_SUM, stream)
+                rc_tree = g.reduce(ds, [droot] * n, count, dtype, N.OP_SUM, 2, stream)
             finally:
                 assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
-            assert rc == N.INVALID_USAGE
+            assert rc == N.INVALID_USAGE and rc_tree == N.SUCCESS
             hip.hipGraphDestroy(graph)
             N.check(g.reduce(ds, [droot] * n, count, dtype, N.OP_SUM, 2, stream))
+            N.check(g.reduce_scatter(ds, dp, count // n, dtype, N.OP_SUM, stream))
             dev.stream_sync(stream)
             assert_parity(dev.to_host(droot, count, np.float32), O.tree_reduce(sends, 2, dtype, N.OP_SUM), dtype,
                           N.OP_SUM, "eager tree reduce")

@@ -118,7 +118,7 @@ flagcxResult_t launchSliceBatches(const KernelSet *ks, const fxSliceDesc *slices
   // A single segment needs no table: the direct kernel's argument block is 100
   // bytes instead of the eight-slot table's 700.
   if (merged.size() == 1) return ks->direct[k](merged[0].out, merged[0].in, k, merged[0].count, s);
-  return ks->slicesInline[k](merged.data(), merged.size(), s);
+  return ks->slicesInline[k](merged.data(), merged.size(), rereadHint(merged.data(), merged.size(), k, (size_t)ks->elemSize), s);
 }
 
 // Largest power-of-two granularity (4, 2 or 1 bytes) shared by all copy slices.
@@ -685,7 +685,8 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
     pl->k = k;
     pl->n = (uint32_t)desc.size();
     pl->grid = start.back();
-    pl->keep = cachePolicyFor(touchedBytes(elems, ks->elemSize, k, 1));
+    pl->keep = cachePolicyFor(touchedBytes(elems, ks->elemSize, k, 1),
+                              rereadHint(merged.data(), merged.size(), k, (size_t)ks->elemSize));
     pl->dDesc = nullptr;
     pl->dTileStart = nullptr;
     if (pl->n) {

@@ -33,23 +33,31 @@ inline uint64_t vectorsOf(uint64_t count, int es) { return (count * (uint64_t)es
 
 // ---- cache policy of a launch ----
 //
-// MI355X has 256 MiB of memory-side cache behind the 4 MiB L2 of each die.
-// Nontemporal accesses stream past it, which is what a launch wants whose
-// operands could never fit: they would only push out what could.  A launch
-// whose operands do fit wants the opposite -- its inputs were usually written
-// by the kernel just before it and its output is read by the one just after --
-// so a launch that touches no more than temporalMaxBytes() uses ordinary loads
-// and stores.  FX_TEMPORAL_MAX_BYTES (environment, read once) moves the
-// threshold; FX_CACHE_POLICY = stream | keep | keep-loads | keep-stores forces
-// one policy for every launch (measurements).
+// Every byte of a reduction is used once, so by default loads and stores are
+// nontemporal: they stream past the 4 MiB L2 of each die and the 256 MiB
+// memory-side cache behind them.  Measured on MI355X with every launch preceded
+// by a 1 GiB fill (nothing of the operands cached), ordinary loads are 40-70 %
+// SLOWER than nontemporal ones from 4 MiB to 256 MiB per input (two fp32
+// inputs of 64 MiB: 57 against 34 us; eight bf16 inputs of 16 MiB: 51 against
+// 30 us), and with the operands cached they are within +-10 % of them, better
+// at some sizes and worse at others.  Ordinary stores are never better.  So the
+// operands' size alone does not choose ordinary accesses.  What does:
+//  * a launch that reads the same bytes more than once -- the all-gather copy
+//    phase hands one source chunk to every other rank, seven copies of it --
+//    reads with ordinary loads, so that the later readers find the chunk in a
+//    cache (56 copies of 8 MiB: 75 against 118 us, and 97 against 126 us from
+//    cold); the batch entry points detect that (rereadHint);
+//  * FX_TEMPORAL_MAX_BYTES (environment, read once; default 0 = never) makes
+//    every launch that touches no more than that many bytes use ordinary loads,
+//    for a caller who knows that its operands are cache-resident;
+//  * FX_CACHE_POLICY = stream | keep | keep-loads | keep-stores forces one
+//    policy for every launch (measurements).
 struct CachePolicyConfig {
   uint64_t maxBytes;
-  int forced;        // -1: by size; otherwise the policy bits for every launch
+  int forced;        // -1: by the rules above; otherwise the policy bits for every launch
 };
-constexpr uint64_t kTemporalMaxBytesDefault = 256ull << 20;
-constexpr uint32_t kAutoKeepBits = kKeepAllLoads | kKeepStores;
 inline CachePolicyConfig readCachePolicyConfig() {
-  CachePolicyConfig c = {kTemporalMaxBytesDefault, -1};
+  CachePolicyConfig c = {0, -1};
   if (const char *e = getenv("FX_TEMPORAL_MAX_BYTES")) {
     char *end = nullptr;
     const unsigned long long v = strtoull(e, &end, 0);
@@ -63,21 +71,52 @@ inline CachePolicyConfig readCachePolicyConfig() {
   }
   return c;
 }
-inline uint32_t cachePolicyFor(uint64_t bytesTouched) {
+// `hint`: policy bits the caller has a reason for (rereadHint).
+inline uint32_t cachePolicyFor(uint64_t bytesTouched, uint32_t hint = 0) {
   static const CachePolicyConfig cfg = readCachePolicyConfig();
   if (cfg.forced >= 0) return (uint32_t)cfg.forced;
-  return bytesTouched <= cfg.maxBytes ? kAutoKeepBits : 0u;
+  return hint | (bytesTouched <= cfg.maxBytes ? kKeepAllLoads : 0u);
 }
 // Bytes a reduction of `count` elements of `es` bytes touches: k inputs, nout outputs.
 inline uint64_t touchedBytes(uint64_t count, int es, int k, int nout) {
   return count * (uint64_t)es * (uint64_t)(k + nout);
 }
 
+// kKeepAllLoads when at least half of the input bytes of a batch of one-input
+// slices are read by more than one slice (same address and length), else 0.
+// Batches of 2..kRereadMaxSlices slices are looked at; the cost is a sort of
+// that many pointers.
+constexpr size_t kRereadMaxSlices = 128;
+inline uint32_t rereadHint(const fxSliceDesc *slices, size_t n, int k, size_t es) {
+  if (k != 1 || n < 2 || n > kRereadMaxSlices) return 0;
+  struct Src {
+    uintptr_t p;
+    uint64_t bytes;
+  };
+  Src src[kRereadMaxSlices];
+  uint64_t total = 0;
+  for (size_t i = 0; i < n; i++) {
+    src[i].p = (uintptr_t)slices[i].in[0];
+    src[i].bytes = slices[i].count * (uint64_t)es;
+    total += src[i].bytes;
+  }
+  for (size_t i = 1; i < n; i++) {   // insertion sort: the lists are short and mostly grouped already
+    const Src v = src[i];
+    size_t j = i;
+    for (; j > 0 && (src[j - 1].p > v.p || (src[j - 1].p == v.p && src[j - 1].bytes > v.bytes)); j--) src[j] = src[j - 1];
+    src[j] = v;
+  }
+  uint64_t again = 0;
+  for (size_t i = 1; i < n; i++)
+    if (src[i].p == src[i - 1].p && src[i].bytes == src[i - 1].bytes) again += src[i].bytes;
+  return again * 2 >= total ? kKeepAllLoads : 0u;
+}
+
 struct KernelSet {
   // index = compile-time input count, 0 = runtime-k kernel
   flagcxResult_t (*direct[kMaxFixedK + 1])(void *out, const void *const *in, int k, uint64_t count, hipStream_t s);
   // n validated, non-empty slices; as many launches as their kernel-argument tables need
-  flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const fxSliceDesc *slices, size_t n, hipStream_t s);
+  flagcxResult_t (*slicesInline[kMaxFixedK + 1])(const fxSliceDesc *slices, size_t n, uint32_t hint, hipStream_t s);
   // device-resident tables, tile counts made with unrollFor(k)
   flagcxResult_t (*slicesTable[kMaxFixedK + 1])(const SliceDescDev *d, const uint32_t *tileStart, uint32_t n,
                                                 uint32_t grid, uint32_t keep, hipStream_t s);
@@ -159,14 +198,14 @@ flagcxResult_t launchSlicesInlineSized(const fxSliceDesc *slices, size_t n, uint
 // The policy follows what the whole call touches (a batch that spreads over
 // several launches still shares the caches).
 template <class R, int K, bool LEAN>
-flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, size_t n, hipStream_t s) {
+flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, size_t n, uint32_t hint, hipStream_t s) {
   constexpr int US = smallUnrollFor(K, LEAN), UD = unrollFor(K);
   uint64_t vecs = 0, elems = 0;
   for (size_t i = 0; i < n; i++) {
     vecs += vectorsOf(slices[i].count, R::ES);
     elems += slices[i].count;
   }
-  const uint32_t keep = cachePolicyFor(touchedBytes(elems, R::ES, K, 1));
+  const uint32_t keep = cachePolicyFor(touchedBytes(elems, R::ES, K, 1), hint);
   if constexpr (LEAN) return launchSlicesInlineSized<R, K, UD, kSmallSliceTable>(slices, n, keep, s);
   if (n > (size_t)kSmallSliceTable) return launchSlicesInlineSized<R, K, UD, 0>(slices, n, keep, s);
   if constexpr (US != UD)

@@ -64,7 +64,14 @@ __device__ __forceinline__ uint32_t roundBf16Top(float f) {
 __device__ __forceinline__ float halfToF32(uint32_t bits16) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
 }
+// fp32 -> fp16, round to nearest even, as a step of its own: the empty asm hides
+// where f came from.  Without it the compiler fuses a multiplication that feeds
+// the conversion into one mixed-precision instruction that rounds the exact
+// product to 16 bits once, and a product whose fp32 rounding lands on a tie
+// between two fp16 values then comes out one ulp off the accumulate-in-fp32,
+// round-once definition (7 of 131,072 four-input products of N(0,1) values).
 __device__ __forceinline__ uint32_t f32ToHalf(float f) {
+  asm("" : "+v"(f));
   return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
 }
 

@@ -60,7 +60,9 @@ struct PendingP2p {
   hipStream_t stream;
   uint64_t id;             // names this half for a sleeping poster (rendezvous mode)
   int owner;               // the rank that posted it
-  bool idle, marked;       // rendezvous mode: its stream had nothing left to do / carries the owner's mark (ready[owner])
+  bool idle, marked;       // rendezvous mode: its stream had nothing left to do / carries a mark of its own
+  hipEvent_t mark;         // that mark: an event of this half alone (two halves of one bracket may sit on two streams,
+                           // and a collective of the same rank re-records ready[owner]); from and back to Group::markPool
 };
 
 // What a sleeping poster finds when its partner has come (rendezvous mode).
@@ -82,6 +84,7 @@ struct Group {
   uint64_t nextP2pId = 1;
   std::map<uint64_t, P2pOutcome> p2pMatched;      // rendezvous mode: results awaiting their sleeping poster
   std::vector<hipEvent_t> after;                  // rendezvous mode: after[r] follows the latest copy rank r enqueued for a partner
+  std::vector<hipEvent_t> markPool;               // rendezvous mode: events for the marks of pending halves, not in use
   // pending collective
   Kind kind = kNone;
   size_t count = 0;
@@ -144,6 +147,17 @@ flagcxResult_t ensureScratch(Group *g, size_t bytes, hipStream_t s) {
   g->scratch = blk;
   g->scratchBytes = want;
   return flagcxSuccess;
+}
+
+// Rendezvous mode asks a rank's stream whether it is idle and marks it with an
+// event that another rank's stream then waits for.  Neither is possible on a
+// stream that is being captured (a query is illegal there and invalidates the
+// capture; the wait would pull a second stream into it), so a call in that mode
+// on such a stream is refused with flagcxInvalidUsage and enqueues nothing.
+// Captures are for the single-thread mode, where every rank posts from one thread.
+inline bool isCapturing(hipStream_t s) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  return s && hipStreamIsCapturing(s, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
 }
 
 // Descriptor lists of one collective: a handful of entries in the common case
@@ -868,15 +882,22 @@ flagcxResult_t runBroadcast(const Ctx &c) {
   return R(fx_copy_slices(d.data(), d.size(), c.s));
 }
 
-// Block i of rank r's sendbuff becomes block r of rank i's recvbuff.  If any
-// rank runs in place the blocks go through staging first.
+// Block i of rank r's sendbuff becomes block r of rank i's recvbuff.  The
+// one-launch kernel reads and writes concurrently, so if ANY rank's send buffer
+// meets ANY rank's receive buffer (a rank in place, rank a receiving into what
+// rank b sends, a partial overlap) the blocks go through staging first.
 flagcxResult_t runAlltoAll(const Ctx &c) {
   Group *g = c.g;
   const int n = c.n;
   const size_t bytes = g->count * c.ts;
   if (bytes == 0) return flagcxSuccess;
   bool inplace = false;
-  for (int r = 0; r < n; r++) inplace = inplace || (c.send(r) == c.recv(r));
+  const size_t span = (size_t)n * bytes;
+  for (int r = 0; r < n && !inplace; r++)
+    for (int i = 0; i < n && !inplace; i++) {
+      const uintptr_t s = (uintptr_t)c.send(r), d = (uintptr_t)c.recv(i);
+      inplace = s < d + span && d < s + span;
+    }
   SliceList d;
   if (!inplace) {   // every block straight from its sender to its receiver, one launch
     PtrList sends;
@@ -985,6 +1006,7 @@ flagcxResult_t postAndMaybeRunImpl(flagcxComm_t comm, Kind kind, const void *sen
   // to it while its rank's thread is in here.
   bool marked = false, idle = false;
   if (g->n > 1 && g->sync.load(std::memory_order_relaxed) == FX_SYNC_RENDEZVOUS) {
+    if (isCapturing(stream->base)) return flagcxInvalidUsage;   // see isCapturing
     idle = hipStreamQuery(stream->base) == hipSuccess;
     if (!idle) {
       (void)hipGetLastError();   // "not ready" is an answer, not an error to leave behind for the caller's next check
@@ -1127,6 +1149,9 @@ void freeGroupResources(Group *g) {
   if (g->done) (void)hipEventDestroy(g->done);
   for (auto e : g->after)
     if (e) (void)hipEventDestroy(e);
+  for (auto e : g->markPool) (void)hipEventDestroy(e);
+  for (const PendingP2p &o : g->p2p)
+    if (o.mark) (void)hipEventDestroy(o.mark);
   if (g->p2pBefore) (void)hipEventDestroy(g->p2pBefore);
   if (g->p2pAfter) (void)hipEventDestroy(g->p2pAfter);
   if (g->scratch) (void)hipFree(g->scratch);
@@ -1246,6 +1271,7 @@ flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64
   if (!matched) {  // the partner never came: withdraw this half
     for (size_t i = 0; i < g->p2p.size(); i++)
       if (g->p2p[i].id == id) {
+        if (g->p2p[i].mark) g->markPool.push_back(g->p2p[i].mark);
         g->p2p.erase(g->p2p.begin() + (long)i);
         break;
       }
@@ -1287,6 +1313,7 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
   if (ts == 0 || peer < 0 || peer >= g->n) return flagcxInvalidArgument;
   if (count && !(isSend ? sbuf : (const void *)rbuf)) return flagcxInvalidArgument;
   const bool rendezvous = g->sync.load(std::memory_order_relaxed) == FX_SYNC_RENDEZVOUS;
+  if (rendezvous && isCapturing(stream->base)) return flagcxInvalidUsage;   // see isCapturing
   if (rendezvous && tGroupDepth > 0 && !tClosingBracket) {
     tQueued.push_back(QueuedP2p{comm, isSend, sbuf, rbuf, count, dtype, peer, stream});
     return flagcxSuccess;
@@ -1318,7 +1345,7 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
         if (g->after.empty()) g->after.assign((size_t)g->n, nullptr);
         hipEvent_t &mine = g->after[(size_t)comm->rank];
         if (o.marked) {
-          if (hipStreamWaitEvent(s, g->ready[(size_t)o.owner], 0) != hipSuccess) res = flagcxUnhandledDeviceError;
+          if (hipStreamWaitEvent(s, o.mark, 0) != hipSuccess) res = flagcxUnhandledDeviceError;
         } else if (!o.idle) {   // posted before the group was switched to this mode: mark its stream from here
           if ((!g->p2pBefore && hipEventCreateWithFlags(&g->p2pBefore, hipEventDisableTiming) != hipSuccess) ||
               hipEventRecord(g->p2pBefore, o.stream) != hipSuccess || hipStreamWaitEvent(s, g->p2pBefore, 0) != hipSuccess)
@@ -1345,21 +1372,32 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
       g->p2pMatched[o.id] = P2pOutcome{res, enqueued ? comm->rank : -1, s};
       g->cv.notify_all();
     }
+    if (o.mark) g->markPool.push_back(o.mark);   // the wait on it is enqueued: the event may be recorded anew
     g->p2p.erase(g->p2p.begin() + (long)i);
     return res;
   }
   // No partner yet.  In rendezvous mode this thread now stays inside the library until one comes, so the stream's
   // state is final: idle, or marked here for the partner to wait on.
   bool idle = false, marked = false;
+  hipEvent_t mark = nullptr;
   if (rendezvous && bytes) {
     idle = hipStreamQuery(s) == hipSuccess;
     if (!idle) {
       (void)hipGetLastError();   // "not ready" is an answer, not an error
-      marked = hipEventRecord(g->ready[(size_t)comm->rank], s) == hipSuccess;
-      if (!marked) return flagcxUnhandledDeviceError;
+      if (!g->markPool.empty()) {
+        mark = g->markPool.back();
+        g->markPool.pop_back();
+      } else if (hipEventCreateWithFlags(&mark, hipEventDisableTiming) != hipSuccess) {
+        return flagcxUnhandledDeviceError;
+      }
+      marked = hipEventRecord(mark, s) == hipSuccess;
+      if (!marked) {
+        g->markPool.push_back(mark);
+        return flagcxUnhandledDeviceError;
+      }
     }
   }
-  g->p2p.push_back(PendingP2p{isSend, src, dst, sbuf, rbuf, bytes, s, g->nextP2pId++, comm->rank, idle, marked});
+  g->p2p.push_back(PendingP2p{isSend, src, dst, sbuf, rbuf, bytes, s, g->nextP2pId++, comm->rank, idle, marked, mark});
   if (!rendezvous) return flagcxSuccess;
   const uint64_t id = g->p2p.back().id;
   if (tClosingBracket) {  // flagcxGroupEnd posts all of the bracket's halves before it waits for any

@@ -213,13 +213,19 @@ class FxBackend : public c10d::Backend {
  public:
   FxBackend(const c10::intrusive_ptr<c10d::Store> &store, int rank, int size) : Backend(rank, size) {
     TORCH_CHECK(size >= 1 && rank >= 0 && rank < size, "bad rank ", rank, " of ", size);
-    // rank 0 makes the id; the others read it from the store (blocking until it is there)
-    const std::string key = "flagcx_amd/unique_id";
+    // rank 0 makes the id; the others read it from the store (blocking until it is there).  The key names the
+    // group: a store may be shared by several groups one after the other (simulated ranks over one HashStore
+    // without torch's per-group prefix), and the id of an earlier group must not be found by a later one's ranks.
+    // Every rank counts the groups it has joined through this store; ranks join their groups in the same order,
+    // so the count is the same number for all ranks of one group.
+    const int64_t generation = store->add("flagcx_amd/groups_joined/" + std::to_string(rank), 1);
+    const std::string key = "flagcx_amd/unique_id/" + std::to_string(generation);
     flagcxUniqueId id;
     if (rank == 0) {
       ok(flagcxGetUniqueId(&id), "flagcxGetUniqueId");
       store->set(key, std::vector<uint8_t>(id.internal, id.internal + sizeof(id.internal)));
     } else {
+      store->wait({key});
       const std::vector<uint8_t> bytes = store->get(key);
       TORCH_CHECK(bytes.size() == sizeof(id.internal), "unique id in the store has ", bytes.size(), " bytes");
       std::memcpy(id.internal, bytes.data(), sizeof(id.internal));
@@ -594,7 +600,10 @@ c10::intrusive_ptr<c10d::Backend> createBackend(const c10::intrusive_ptr<c10d::S
 
 PYBIND11_MODULE(fx_c10d, m) {
   m.doc() = "torch.distributed backend over libflagcx_amd.so";
-  m.def("create_backend", &createBackend, py::arg("store"), py::arg("rank"), py::arg("size"));
+  // without the interpreter lock: a rank other than 0 waits in here for rank 0's id, and rank 0 may be
+  // another thread of this process
+  m.def("create_backend", &createBackend, py::arg("store"), py::arg("rank"), py::arg("size"),
+        py::call_guard<py::gil_scoped_release>());
   // torch binds these two on ProcessGroup only; a backend object on its own reaches them here
   m.def("allgather_into_tensor_coalesced", [](const c10::intrusive_ptr<c10d::Backend> &b, Tensors outs, Tensors ins) {
     return b->allgather_into_tensor_coalesced(outs, ins);

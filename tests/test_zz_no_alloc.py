@@ -3,6 +3,8 @@ entry point it is a variant of (fx_plan_create + fx_plan_launch) and against
 the CPU oracle: two calls in a row on the same GPU, the second with a smaller
 input, so that what the first call left in the static table must not leak into
 the second."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -100,3 +102,67 @@ def test_static_table_copy_and_limits(dev):
     assert K.reduce_slices_static([([0, 0], 0, 5)], 2, N.DT_FP32, N.OP_SUM) == N.INVALID_ARGUMENT
     assert K.reduce_slices_static([([16, 16], 16, 5)], 9, N.DT_FP32, N.OP_SUM) == N.INVALID_ARGUMENT
     assert K.reduce_slices_static([([16, 16], 16, 5)], 2, 99, N.OP_SUM) == N.INVALID_ARGUMENT
+
+
+def test_static_table_in_a_captured_graph_two_dependent_calls(dev):
+    """What the entry point is for: one eager call first (it looks the table's
+    address up), then TWO calls captured on one stream -- different descriptors,
+    the second reading what the first wrote, so the second's table overwrites the
+    first's while both are in the graph -- replayed on new data; every replay
+    against the oracle."""
+    hip = C.CDLL("libamdhip64.so.7")          # the runtime the library itself is linked against (same mapping)
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    dtype, op, k, total = N.DT_FP32, N.OP_SUM, 3, 200_003
+    rng = np.random.default_rng(11)
+    first_sl, second_sl = _pieces(rng, total, 40), _pieces(rng, total, 9)      # 40 descriptors: two table-writer launches
+    stream = dev.stream_create()
+    raw = dev.raw_stream(stream)
+    with DevBufs(dev) as b:
+        ins = seeded_inputs(dtype, k, total, seed=3)
+        dins = [b.put(a) for a in ins]
+        dmid, dout = b.alloc(total * 4), b.alloc(total * 4)
+        # the eager call: any call on this GPU outside a capture
+        N.check(K.reduce_slices_static([(dins, dmid, 16)], k, dtype, op, raw))
+        dev.stream_sync(stream)
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(raw, 0) == 0
+        try:
+            # mid = in0 + in1 + in2 on the first pieces; out = mid + in0 (two inputs) on the second pieces
+            N.check(K.reduce_slices_static([([p + o * 4 for p in dins], dmid + o * 4, c) for o, c in first_sl], k, dtype, op, raw))
+            N.check(K.reduce_slices_static([([dmid + o * 4, dins[0] + o * 4], dout + o * 4, c) for o, c in second_sl], 2, dtype,
+                                           op, raw))
+        finally:
+            assert hip.hipStreamEndCapture(raw, C.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for rep in range(3):
+            if rep:
+                ins = seeded_inputs(dtype, k, total, seed=3 + rep)
+                for d, a in zip(dins, ins):
+                    dev.upload(d, a)
+            dev.memset(dmid, FILL, total * 4)
+            dev.memset(dout, FILL, total * 4)
+            # eager work of the program's own between the replays, through the same table
+            N.check(K.reduce_slices_static([(dins, dout, 1000)], k, dtype, op, raw))
+            dev.stream_sync(stream)
+            dev.memset(dout, FILL, total * 4)
+            dev.sync()
+            assert hip.hipGraphLaunch(gexec, raw) == 0
+            dev.stream_sync(stream)
+            mid = np.frombuffer(bytes([FILL]) * (total * 4), dtype=np.float32).copy()
+            for o, c in first_sl:
+                if c:
+                    mid[o:o + c] = O.reduce_copy([a[o:o + c] for a in ins], dtype, op)
+            want = np.frombuffer(bytes([FILL]) * (total * 4), dtype=np.float32).copy()
+            for o, c in second_sl:
+                if c:
+                    want[o:o + c] = O.reduce2(mid[o:o + c], ins[0][o:o + c], dtype, op)
+            assert_parity(dev.to_host(dmid, total, np.float32), mid, dtype, op, f"replay {rep}: first captured call")
+            assert_parity(dev.to_host(dout, total, np.float32), want, dtype, op, f"replay {rep}: second captured call")
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+    dev.stream_destroy(stream)

@@ -242,6 +242,31 @@ def simulated(n, gen):
     del ranks
 
 
+def two_groups_over_one_store(gen):
+    """A second group built over the store of a first one must not pick up the
+    first one's unique id -- not even when its rank 1 is built before its rank 0."""
+    import threading
+    import time
+    store = dist.HashStore()
+    first = [fxb.new_backend(store, r, 2) for r in range(2)]
+    box = {}
+    th = threading.Thread(target=lambda: box.__setitem__(1, fxb.new_backend(store, 1, 2)))
+    th.start()
+    time.sleep(0.3)                      # rank 1 of the second group is now waiting for ITS rank 0
+    assert 1 not in box, "rank 1 of the second group did not wait for its own rank 0"
+    box[0] = fxb.new_backend(store, 0, 2)
+    th.join(30)
+    assert not th.is_alive() and 1 in box
+    second = [box[0], box[1]]
+    for name, ranks in (("first", first), ("second", second)):
+        ts = [make(torch.float32, (1000,), gen) for _ in range(2)]
+        want = O.reduce_copy([words(t) for t in ts], comm.dtype_code(torch.float32), comm.op_code(ReduceOp.SUM))
+        wait_all([b.allreduce([t], dist.AllreduceOptions()) for b, t in zip(ranks, ts)])
+        for r, t in enumerate(ts):
+            same(words(t).ravel(), want, f"{name} group over a shared store, rank {r}")
+    print("ok  two successive groups over one HashStore", flush=True)
+
+
 def one_rank(gen):
     fxb.register()
     dist.init_process_group("flagcx", store=dist.HashStore(), rank=0, world_size=1)
@@ -301,6 +326,7 @@ def main():
         print("HIP runtime in this process:", sorted({ln.split()[-1] for ln in f if "libamdhip64" in ln}), flush=True)
     simulated(4, gen)
     simulated(8, gen)
+    two_groups_over_one_store(gen)
     one_rank(gen)
     print("torch backend ok", flush=True)
 

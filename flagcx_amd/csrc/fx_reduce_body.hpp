@@ -502,25 +502,38 @@ __host__ __device__ inline HandOut handOutFor(bool samePhase, int k) {
   return samePhase ? kStriped : (k == 1 ? kGrouped : kContiguous);
 }
 
+// Element sizes, vectors per tile and tiles per region are powers of two, so
+// the plan is shifts and masks only: a persistent kernel works it out once per
+// trigger in every workgroup, with an element size it only knows at run time,
+// and a 64-bit division there is a hundred instructions.
+__host__ __device__ constexpr uint32_t log2Of(uint32_t x) {   // x a power of two
+  uint32_t l = 0;
+  while ((1u << l) < x) l++;
+  return l;
+}
 __host__ __device__ inline TilePlan planTiles(uint64_t outAddr, uint64_t count, int es, int U, HandOut how) {
   TilePlan tp;
-  const uint64_t V = (uint64_t)U * kBlock, RV = V * kStripeTiles, ve = 16u / (uint32_t)es;
-  const uint64_t mis = outAddr & 15u, lead = mis / (uint32_t)es, end = lead + count;
-  tp.nv = (end + ve - 1) / ve;
-  tp.firstFull = (lead + ve - 1) / ve;
-  tp.endFull = end / ve;
+  const uint32_t esShift = (es == 1) ? 0u : (es == 2) ? 1u : (es == 4) ? 2u : 3u;
+  const uint32_t veShift = 4u - esShift;                                     // elements per vector
+  const uint32_t vShift = log2Of(kBlock) + ((U == 1) ? 0u : (U == 2) ? 1u : (U == 4) ? 2u : 3u);   // vectors per tile
+  const uint32_t rvShift = vShift + log2Of(kStripeTiles);                    // vectors per region
+  const uint64_t V = 1ull << vShift, RV = 1ull << rvShift, ve = 1ull << veShift;
+  const uint64_t mis = outAddr & 15u, lead = mis >> esShift, end = lead + count;
+  tp.nv = (end + ve - 1) >> veShift;
+  tp.firstFull = (lead + ve - 1) >> veShift;
+  tp.endFull = end >> veShift;
   const uint64_t a0 = (outAddr - mis) >> 4;  // absolute vector number of vector 0
-  uint64_t zs = (a0 + tp.firstFull + RV - 1) / RV * RV, ze = (a0 + tp.endFull) / RV * RV;
+  const uint64_t zs = ((a0 + tp.firstFull + RV - 1) >> rvShift) << rvShift, ze = ((a0 + tp.endFull) >> rvShift) << rvShift;
   tp.grouped = (how == kGrouped);
-  if (how == kContiguous || ze <= zs || count * (uint64_t)es < kStripeMinBytes) {
+  if (how == kContiguous || ze <= zs || (count << esShift) < kStripeMinBytes) {
     tp.zs = tp.ze = 0;
   } else {
     tp.zs = zs - a0;
     tp.ze = ze - a0;
   }
-  tp.zoneTiles = (uint32_t)((tp.ze - tp.zs) / V);
-  tp.headTiles = (uint32_t)((tp.zs + V - 1) / V);
-  tp.tailTiles = (uint32_t)((tp.nv - tp.ze + V - 1) / V);
+  tp.zoneTiles = (uint32_t)((tp.ze - tp.zs) >> vShift);
+  tp.headTiles = (uint32_t)((tp.zs + V - 1) >> vShift);
+  tp.tailTiles = (uint32_t)((tp.nv - tp.ze + V - 1) >> vShift);
   return tp;
 }
 

@@ -46,6 +46,16 @@ int main() {
             if (owner[i] == -1) { printf("FAIL index %u has no workgroup (grid %u seq %llu tiles %llu)\n", i, grid, (unsigned long long)seq, (unsigned long long)tiles); return 1; }
           cases++;
         }
+  // the rotation carried from trigger to trigger is the one worked out from the trigger's number
+  for (uint32_t pool : {1u, 2u, 3u, 60u, 61u, 62u, 122u, 255u, 256u, 512u})
+    for (uint64_t start : {0ull, 5ull, 1000003ull, (1ull << 40) + 7}) {
+      uint32_t rot = rotOf(start, pool);
+      const uint32_t step = rotStep(pool);
+      for (uint64_t seq = start; seq < start + 2000; seq++, rot = nextRot(rot, step, pool)) {
+        if (rot != rotOf(seq, pool) || rot >= pool) { printf("FAIL rotation drifts: pool %u seq %llu\n", pool, (unsigned long long)seq); return 1; }
+        cases++;
+      }
+    }
   printf("ok %ld cases\n", cases);
   return 0;
 }

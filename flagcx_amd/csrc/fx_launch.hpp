@@ -8,15 +8,14 @@
 namespace fx {
 
 // Vectors per lane per input, measured on MI355X.
-//  * Launches that write less than 4 MiB (per output buffer): 1 for three inputs
-//    and more, and for the multi-output kernels.  With 4, such a launch has fewer
-//    workgroups than the device has compute units and each lane waits for 32
-//    loads: an eight-input reduction of 1 MiB per input takes 4.8 us against
-//    2.9 us, the eight-rank all-reduce of 64 KiB per rank 6.2 against 4.3 us.
-//    The run-time-k kernels (nine inputs and more, 2 otherwise) likewise.
-//  * Larger launches: 4 (2 for one and two inputs).  Between 1, 2, 4 and 8 the
-//    difference at these sizes is within 1 % and changes sign with where the
-//    buffers sit.
+//  * One, for three inputs and more, while a launch writes less than 32 MiB (4 MiB per output buffer for the
+//    multi-output kernels; the run-time-k kernels likewise).  With four, such a launch has few workgroups per compute
+//    unit and every lane waits for 32 loads before its first store: an eight-input bf16 reduction of 4 MiB per input
+//    takes 6.9 us against 4.8 us (12.1 against 10.2 from cold), 16 MiB 25.2 against 23.8 (29.4 against 28.0), a
+//    four-input fp32 one of 4 MiB 4.4 against 3.9; the eight-rank all-reduce of 64 KiB per rank 6.2 against 4.3 us,
+//    but at 8 MiB per rank 20.0 us with four against 22.7 with one, hence its lower limit.
+//  * Above that: four (two for one and two inputs).  From 32 MiB of output up the difference between one and four
+//    is within 1 % either way (eight inputs of 512 MiB: 747 us with four, 751 with one).
 // LEAN kernel sets (the types only the host path of the reference carries, and
 // the element-type fold) have one variant per input count: no separate
 // small-launch kernels and one table size.
@@ -24,7 +23,8 @@ constexpr int unrollFor(int K) { return K <= 2 ? 2 : 4; }
 constexpr int smallUnrollFor(int K, bool lean) {
   return (!lean && (K >= 3 || K == 0)) ? 1 : unrollFor(K);   // K = 0: run-time k, nine inputs and more
 }
-constexpr uint64_t kSmallLaunchVecs = 256 * 1024;  // fewer 16-byte vectors of output than this: one vector per lane
+constexpr uint64_t kSmallLaunchVecs = 2048 * 1024;      // single-output kernels: fewer 16-byte vectors of output than this (32 MiB) -> one vector per lane
+constexpr uint64_t kSmallBcastVecs = 256 * 1024;        // multi-output and many-rank kernels: 4 MiB per output buffer
 constexpr int kBcastUnroll = 4;
 constexpr int smallBcastUnroll(bool lean) { return lean ? kBcastUnroll : 1; }   // the multi-output kernels, any number of inputs
 constexpr int kOrderedUnroll = 2;   // the tree / keep-local kernels: one variant for every size
@@ -280,7 +280,7 @@ flagcxResult_t launchBcastInline(const BcastDescDev *d, size_t n, hipStream_t s)
   uint64_t vecs = 0;   // per output buffer, all descriptors together
   const uint32_t keep = bcastPolicy(d, n, R::ES, K, &vecs);
   if constexpr (LEAN) return launchBcastMany<R, K, UD, kChain>(d, n, keep, s);
-  const bool small = vecs < kSmallLaunchVecs;
+  const bool small = vecs < kSmallBcastVecs;
   if (n == 1) return small ? launchBcastOne<R, K, US>(d[0], keep, s) : launchBcastOne<R, K, UD>(d[0], keep, s);
   return small ? launchBcastMany<R, K, US, kChain>(d, n, keep, s) : launchBcastMany<R, K, UD, kChain>(d, n, keep, s);
 }
@@ -315,7 +315,7 @@ template <class R, bool LEAN>
 flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const *in, int k, uint64_t count,
                                   hipStream_t s) {
   if constexpr (!LEAN)
-    if (vectorsOf(count, R::ES) < kSmallLaunchVecs) return launchBcastRuntimeU<R, 1>(out, nout, in, k, count, s);
+    if (vectorsOf(count, R::ES) < kSmallBcastVecs) return launchBcastRuntimeU<R, 1>(out, nout, in, k, count, s);
   return launchBcastRuntimeU<R, unrollFor(0)>(out, nout, in, k, count, s);
 }
 
@@ -340,7 +340,7 @@ flagcxResult_t launchChunksRuntime(ChunkedArgs *a, hipStream_t s) {
   if constexpr (!LEAN) {
     uint64_t vecs = 0;
     for (int c = 0; c < a->nchunks; c++) vecs += vectorsOf(a->cnt[c], R::ES);
-    if (vecs < kSmallLaunchVecs) return launchChunksRuntimeU<R, 1>(a, s);
+    if (vecs < kSmallBcastVecs) return launchChunksRuntimeU<R, 1>(a, s);
   }
   return launchChunksRuntimeU<R, unrollFor(0)>(a, s);
 }

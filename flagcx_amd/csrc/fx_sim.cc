@@ -68,8 +68,9 @@ struct PendingP2p {
 // What a sleeping poster finds when its partner has come (rendezvous mode).
 struct P2pOutcome {
   flagcxResult_t res;
-  int by;                  // the rank whose call enqueued the copy, -1 if nothing was enqueued
-  hipStream_t where;       // on this stream
+  hipStream_t where;       // the stream the copy was enqueued on
+  hipEvent_t after;        // recorded behind that copy, an event of this copy alone (a rank may enqueue copies for two
+                           // partners on two streams); nullptr if nothing was enqueued; back to Group::markPool when used
 };
 
 struct Group {
@@ -83,8 +84,8 @@ struct Group {
   hipEvent_t p2pBefore = nullptr, p2pAfter = nullptr;   // made at the first pair whose halves sit on two streams
   uint64_t nextP2pId = 1;
   std::map<uint64_t, P2pOutcome> p2pMatched;      // rendezvous mode: results awaiting their sleeping poster
-  std::vector<hipEvent_t> after;                  // rendezvous mode: after[r] follows the latest copy rank r enqueued for a partner
-  std::vector<hipEvent_t> markPool;               // rendezvous mode: events for the marks of pending halves, not in use
+  std::vector<hipEvent_t> markPool;               // rendezvous mode: events for the marks of pending halves and for the
+                                                  // copies made for a sleeping partner, not in use
   // pending collective
   Kind kind = kNone;
   size_t count = 0;
@@ -1147,9 +1148,9 @@ void freeGroupResources(Group *g) {
   for (auto e : g->ready)
     if (e) (void)hipEventDestroy(e);
   if (g->done) (void)hipEventDestroy(g->done);
-  for (auto e : g->after)
-    if (e) (void)hipEventDestroy(e);
   for (auto e : g->markPool) (void)hipEventDestroy(e);
+  for (auto &m : g->p2pMatched)
+    if (m.second.after) (void)hipEventDestroy(m.second.after);
   for (const PendingP2p &o : g->p2p)
     if (o.mark) (void)hipEventDestroy(o.mark);
   if (g->p2pBefore) (void)hipEventDestroy(g->p2pBefore);
@@ -1280,15 +1281,20 @@ flagcxResult_t awaitPartner(Group *g, std::unique_lock<std::mutex> &lock, uint64
   }
   const P2pOutcome out = g->p2pMatched[id];
   g->p2pMatched.erase(id);
-  hipEvent_t follows = (out.by >= 0 && out.where != own) ? g->after[(size_t)out.by] : nullptr;
   lock.unlock();
-  if (out.res == flagcxSuccess && follows) {
-    // the partner may have moved its event on to a later copy of its own by now: later on the same stream, so still after ours
-    if (hipEventQuery(follows) == hipSuccess) return out.res;
-    (void)hipGetLastError();   // "not ready" is an answer, not an error
-    if (hipStreamWaitEvent(own, follows, 0) != hipSuccess) return flagcxUnhandledDeviceError;
+  flagcxResult_t res = out.res;
+  if (out.after) {
+    if (res == flagcxSuccess && out.where != own) {
+      if (hipEventQuery(out.after) != hipSuccess) {   // not over yet: what this rank enqueues next comes after the copy
+        (void)hipGetLastError();                      // "not ready" is an answer, not an error
+        if (hipStreamWaitEvent(own, out.after, 0) != hipSuccess) res = flagcxUnhandledDeviceError;
+      }
+    }
+    lock.lock();
+    g->markPool.push_back(out.after);   // the wait on it is enqueued (or not needed): the event may be recorded anew
+    lock.unlock();
   }
-  return out.res;
+  return res;
 }
 
 // send / recv between simulated ranks: the later of the two calls performs the
@@ -1326,7 +1332,7 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
     PendingP2p &o = g->p2p[i];
     if (o.isSend == isSend || o.src != src || o.dst != dst) continue;
     flagcxResult_t res = flagcxSuccess;
-    bool enqueued = false;
+    hipEvent_t behind = nullptr;   // rendezvous mode, two streams: recorded behind the copy for the sleeping partner
     if (o.bytes != bytes) {
       res = flagcxInvalidArgument;  // the two sides disagree on the message size
     } else if (bytes) {
@@ -1341,9 +1347,7 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
       } else if (rendezvous) {
         // The other half's thread is inside its call (or its flagcxGroupEnd) until we are done: its stream stands
         // still.  An idle one needs no waiting for, a busy one carries its owner's mark; and the owner makes
-        // its own stream wait for the copy when it wakes, through after[this rank].
-        if (g->after.empty()) g->after.assign((size_t)g->n, nullptr);
-        hipEvent_t &mine = g->after[(size_t)comm->rank];
+        // its own stream wait for the copy when it wakes, through the event recorded behind the copy (`behind`).
         if (o.marked) {
           if (hipStreamWaitEvent(s, o.mark, 0) != hipSuccess) res = flagcxUnhandledDeviceError;
         } else if (!o.idle) {   // posted before the group was switched to this mode: mark its stream from here
@@ -1352,11 +1356,20 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
             res = flagcxUnhandledDeviceError;
         }
         if (res == flagcxSuccess) res = R(fx_copy_slices(&d, 1, s));
-        if (res == flagcxSuccess &&
-            ((!mine && hipEventCreateWithFlags(&mine, hipEventDisableTiming) != hipSuccess) ||
-             hipEventRecord(mine, s) != hipSuccess))
-          res = flagcxUnhandledDeviceError;
-        enqueued = res == flagcxSuccess;
+        if (res == flagcxSuccess) {
+          if (!g->markPool.empty()) {
+            behind = g->markPool.back();
+            g->markPool.pop_back();
+          } else if (hipEventCreateWithFlags(&behind, hipEventDisableTiming) != hipSuccess) {
+            behind = nullptr;
+            res = flagcxUnhandledDeviceError;
+          }
+          if (behind && hipEventRecord(behind, s) != hipSuccess) {
+            g->markPool.push_back(behind);
+            behind = nullptr;
+            res = flagcxUnhandledDeviceError;
+          }
+        }
       } else {
         if ((!g->p2pBefore && hipEventCreateWithFlags(&g->p2pBefore, hipEventDisableTiming) != hipSuccess) ||
             (!g->p2pAfter && hipEventCreateWithFlags(&g->p2pAfter, hipEventDisableTiming) != hipSuccess) ||
@@ -1369,7 +1382,7 @@ flagcxResult_t postP2pImpl(flagcxComm_t comm, bool isSend, const void *sbuf, voi
       }
     }
     if (rendezvous) {
-      g->p2pMatched[o.id] = P2pOutcome{res, enqueued ? comm->rank : -1, s};
+      g->p2pMatched[o.id] = P2pOutcome{res, s, behind};
       g->cv.notify_all();
     }
     if (o.mark) g->markPool.push_back(o.mark);   // the wait on it is enqueued: the event may be recorded anew

@@ -481,6 +481,87 @@ def test_rendezvous_ring_exchange_inside_a_group_bracket(dev, monkeypatch):
     assert N.lib.flagcxGroupEnd(None) == N.INVALID_USAGE            # no bracket open on this thread
 
 
+def test_rendezvous_bracket_with_two_streams_per_rank(dev, monkeypatch):
+    """One bracket whose two halves sit on two streams of the same rank, both busy:
+    each pending half carries a mark of its own, so the partner of the first half
+    waits for THAT stream's earlier work, not for wherever the rank's last mark
+    went.  Every rank sends on stream A data that a long-running fill on A writes
+    just before, and receives on stream B."""
+    import threading
+    monkeypatch.setenv("FX_SIM_RENDEZVOUS_TIMEOUT_MS", "15000")
+    n, count, rounds = 4, 2_000_003, 6
+    errors = []
+    with DevBufs(dev) as b, S.SimGroup(n, sync=S.SYNC_RENDEZVOUS) as g:
+        dsend = [b.alloc(count * 4) for _ in range(n)]
+        drecv = [b.alloc(count * 4) for _ in range(n)]
+        busy = [b.alloc(64 << 20) for _ in range(n)]
+
+        def rank_main(r):
+            try:
+                dev.set_device()
+                sa, sb = dev.stream_create(), dev.stream_create()
+                host = np.empty(count, np.float32)
+                for it in range(rounds):
+                    src = np.full(count, r * 100 + it, np.float32)
+                    dev.memset(busy[r], it, 64 << 20, sa)          # keeps stream A busy ahead of the upload
+                    dev.upload(dsend[r], src, sa)
+                    dev.memset(busy[r], it + 1, 64 << 20, sb)      # and stream B busy too, so both halves get marks
+                    N.check(N.lib.flagcxGroupStart(g.comms[r]))
+                    N.check(N.lib.flagcxSend(dsend[r], count, N.DT_FP32, (r + 1) % n, g.comms[r], sa))
+                    N.check(N.lib.flagcxRecv(drecv[r], count, N.DT_FP32, (r - 1) % n, g.comms[r], sb))
+                    N.check(N.lib.flagcxGroupEnd(g.comms[r]))
+                    dev.download(host, drecv[r], sb)
+                    dev.stream_sync(sb)
+                    dev.stream_sync(sa)
+                    if not (host == ((r - 1) % n) * 100 + it).all():
+                        errors.append((r, it, host[:4].tolist(), host[-2:].tolist()))
+                    N.check(N.lib.flagcxBarrier(g.comms[r], sa))
+                    dev.stream_sync(sa)
+                dev.stream_destroy(sa)
+                dev.stream_destroy(sb)
+            except Exception as e:                      # noqa: BLE001 - reported below
+                errors.append((r, repr(e)))
+
+        threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=100)
+        assert not any(t.is_alive() for t in threads)
+        assert not errors, errors[:4]
+
+
+def test_alltoall_stages_whenever_a_send_buffer_meets_a_receive_buffer(dev, stream):
+    """Not only a rank in place: rank 0 receives into what rank 1 sends, and rank 2's
+    receive buffer overlaps rank 0's send buffer partly.  The one-launch kernel reads
+    and writes concurrently, so such calls must go through staging; the result is
+    what the original send contents say."""
+    n, blk = 3, 50_001
+    rng = np.random.default_rng(12)
+    sends = [rng.integers(-1000, 1000, n * blk, dtype=np.int32) for _ in range(n)]
+    with DevBufs(dev) as b, S.SimGroup(n) as g:
+        arena = b.alloc(4 * n * blk * 4 + 4096)
+        ds = [arena, arena + n * blk * 4, arena + 2 * n * blk * 4]
+        own = b.alloc(n * blk * 4)
+        dr = [ds[1],                      # rank 0 receives into rank 1's send buffer
+              own,
+              ds[0] + 1000 * 4]           # rank 2's receive buffer overlaps rank 0's send buffer (and runs into rank 1's)
+        for d, a in zip(ds, sends):
+            dev.upload(d, a)
+        for r in range(n):
+            N.check(N.lib.flagcxAlltoAll(ds[r], dr[r], blk, N.DT_INT32, g.comms[r], stream))
+        dev.stream_sync(stream)
+        # rank 1's own buffer is touched by nobody else: it must hold block 1 of every rank's ORIGINAL send data
+        want1 = np.concatenate([sends[r][blk:2 * blk] for r in range(n)])
+        assert np.array_equal(dev.to_host(own, n * blk, np.int32), want1)
+        # rank 0 and rank 2 overlap each other's results where dr[2] runs into ds[1] = dr[0]; what lies outside that
+        # overlap is checked: the first part of rank 2's buffer (inside ds[0]) and the tail of rank 0's
+        want2 = np.concatenate([sends[r][2 * blk:3 * blk] for r in range(n)])
+        got2 = dev.to_host(dr[2], n * blk, np.int32)
+        free2 = n * blk - 1000            # elements of dr[2] that lie before ds[1] starts
+        assert np.array_equal(got2[:free2], want2[:free2])
+
+
 def test_rendezvous_times_out_when_a_rank_never_arrives(dev, stream, monkeypatch):
     import threading
     monkeypatch.setenv("FX_SIM_RENDEZVOUS_TIMEOUT_MS", "200")

@@ -283,7 +283,7 @@ int fxHostStagedCreate(fxHostStaged_t *h, int nranks, fxDeviceMemcpyFn memcpyFn)
 }
 
 namespace {
-int runStaged(fxHostStaged_t h, Kind kind, int root, const void *const *sendbuffs, void *const *recvbuffs, size_t count,
+static int runStaged(fxHostStaged_t h, Kind kind, int root, const void *const *sendbuffs, void *const *recvbuffs, size_t count,
               int dtype, int op, uint64_t *timers) {
   if (!h || !sendbuffs || !recvbuffs) return flagcxInvalidArgument;
   if (!carried(dtype, op)) return flagcxInvalidArgument;   // as the reference's host loops

@@ -327,6 +327,16 @@ def test_scheduler_stand_in_takes_one_symbol_from_the_kernel_library(tmp_path):
     assert os.path.exists(built), "the build did not leave flagcx_amd/lib/unirunner_client for the GPU tests"
 
 
+def test_reference_named_launcher_refuses_a_missing_ring_without_touching_the_device(capfd):
+    """flagcxLaunchCollectiveKernel has no result to return (the reference's signature is void): a call it cannot
+    serve says so on stderr and enqueues nothing.  No GPU needed for the first check it makes."""
+    lib = C.CDLL(os.path.join(N.LIB_DIR, "libflagcx-kernels-mi355x.so"))
+    fn = getattr(lib, CXX_LINKAGE["flagcxLaunchCollectiveKernel"])
+    fn.restype, fn.argtypes = None, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+    fn(None, 32, 1, None)
+    assert "flagcxLaunchCollectiveKernel: no ring" in capfd.readouterr().err
+
+
 def test_headers_are_plain_c_and_a_c_client_links(tmp_path):
     """The boundary is a C ABI: every header compiles as strict C11, a C program
     links against the kernel library and the host-only entry points answer."""

@@ -82,6 +82,63 @@ def test_kernel_layer_random_cases(dev):
         _kernel_case(dev, rng, no)
 
 
+def _ordered_case(dev, rng, no):
+    """fx_reduce_ordered: tree or keep-local association, any type, 2..8 inputs, one to eight outputs, the inputs
+    each at their own offset, one or two slices; NaNs and signed zeros planted for max / min."""
+    names = ["fp32", "fp64", "bf16", "fp16", "int32", "uint8", "int64"]
+    dname = names[rng.integers(len(names))]
+    dtype = DTYPES[dname]
+    es = N.DTYPE_SIZE[dtype]
+    order = int(rng.choice([K.FOLD_TREE, K.FOLD_KEEP_LOCAL]))
+    op = int(rng.choice([N.OP_SUM, N.OP_PROD, N.OP_MAX, N.OP_MIN]))
+    k = int(rng.integers(2, 9))
+    if order == K.FOLD_KEEP_LOCAL and dname in ("bf16", "fp16") and op in (N.OP_SUM, N.OP_PROD) and k >= 3:
+        op = N.OP_MAX                 # the one combination the entry point refuses (no such host path)
+    n = int(rng.integers(1, 3_000_000 // es)) if rng.random() < 0.1 else int(rng.integers(1, 40000))
+    nout = int(rng.integers(1, 9))
+    ve = 16 // es
+    o0 = int(rng.integers(0, ve * 40))
+    offs = [o0 if rng.random() < 0.5 else int(rng.integers(0, ve * 40)) for _ in range(k)]
+    cut = int(rng.integers(0, n + 1))
+    seed = int(rng.integers(1 << 30))
+    desc = f"ordered case {no}: {dname} order={order} op={op} k={k} n={n} nout={nout} out+{o0} in+{offs} cut={cut} seed={seed}"
+    print(desc, flush=True)
+    ins = seeded_inputs(dtype, k, n, seed=seed)
+    if op in (N.OP_MAX, N.OP_MIN) and dname in ("fp32", "fp64", "bf16", "fp16") and n > 64:
+        for a in ins:
+            idx = rng.choice(n, size=min(32, n), replace=False)
+            if dname in ("bf16", "fp16"):
+                nan = 0x7fc0 if dname == "bf16" else 0x7e00
+                a[idx[:8]], a[idx[8:16]], a[idx[16:24]], a[idx[24:]] = nan, nan | 0x8000, 0x0000, 0x8000
+            else:
+                a[idx[:8]], a[idx[8:16]], a[idx[16:24]], a[idx[24:]] = np.nan, -np.nan, 0.0, -0.0
+    if order == K.FOLD_TREE:
+        want = O.tree_reduce(ins, 0, dtype, op)
+    else:
+        want = ins[0].copy()
+        for j in range(1, k):
+            want = O.reduce2(ins[j], want, dtype, op)
+    with DevBufs(dev) as b:
+        dins = [b.put(a, pad_before=o * es, pad_after=64) for a, o in zip(ins, offs)]
+        outs = [_fresh_out(b, dev, o0 * es, n * es) for _ in range(nout)]
+        descs = [([p + lo * es for p in dins], [q + lo * es for q in outs], hi - lo) for lo, hi in ((0, cut), (cut, n))]
+        N.check(K.reduce_ordered(descs, k, nout, dtype, op, order), desc)
+        dev.sync()
+        for d in outs:
+            got = dev.to_host(d, n, N.NP_DTYPE[dtype])
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), desc
+            assert (dev.to_host(d + n * es, 32, np.uint8) == PAD).all(), "wrote past the end: " + desc
+            if d % 16:
+                lead = d % 16
+                assert (dev.to_host(d - lead, lead, np.uint8) == PAD).all(), "wrote before the start: " + desc
+
+
+def test_ordered_folds_random_cases(dev):
+    rng = np.random.default_rng(20241125)
+    for no in range(1200):
+        _ordered_case(dev, rng, no)
+
+
 def _collective_case(dev, stream, rng, no):
     names = ["fp32", "int32", "fp64", "uint8", "int64", "bf16", "fp16"]
     dname = names[rng.integers(len(names))]

@@ -17,9 +17,16 @@
 //   (truncating toward zero, on the wrapped sum) for signed integers, unsigned
 //   division for unsigned ones.  FlagCX itself only forwards avg to vendor
 //   libraries, so this definition is this path's own.
+//   Two further associations of the same k inputs (enum Sched) exist for the
+//   callers that must reproduce a multi-step schedule of the reference's in one
+//   launch: its binomial tree and its host ring's "local operand first" chain.
+//   They round to the element type after every step, as those schedules do.
 //
 // Data movement: one 16-byte vector per lane per input, U vectors per lane in
-// flight per input, all K*U loads issued before the first use.  The index
+// flight per input, all K*U loads issued before the first use.  Loads and
+// stores bypass the caches (nontemporal) unless the launch's policy word
+// (`keep` in every argument block) asks for ordinary accesses: one bit per
+// input plus one for the stores, uniform over the launch.  The index
 // space is anchored at the output pointer rounded down to 16 bytes, so stores
 // are always whole aligned vectors except in the first and last vector of a
 // segment, which fall back to element accesses.  An input need not share the

@@ -110,6 +110,34 @@ int main() {
     }
     cases += 8;
   }
+  // Which batches of one-input slices read with ordinary loads: those that read at least half of their bytes twice.
+  {
+    char *src = (char *)0x7f0000100000ull, *dst = (char *)0x7f4000000000ull;
+    const uint64_t chunk = 1 << 20;
+    std::vector<fxSliceDesc> ag;                 // the all-gather copy phase of 8 ranks: chunk r to the 7 other ranks
+    for (int r = 0; r < 8; r++)
+      for (int q = 0; q < 8; q++)
+        if (q != r) ag.push_back(fxSliceDesc{{src + r * chunk}, dst + (q * 8 + r) * chunk, chunk});
+    std::vector<fxSliceDesc> pack;               // a pack: every slice another source
+    for (int i = 0; i < 64; i++) pack.push_back(fxSliceDesc{{src + i * chunk}, dst + i * chunk, chunk});
+    std::vector<fxSliceDesc> half = pack, less = pack, lens = pack, many;
+    for (int i = 0; i < 32; i++) half[2 * i + 1].in[0] = half[2 * i].in[0];      // 32 of 64 slices read again: exactly half
+    for (int i = 0; i < 31; i++) less[2 * i + 1].in[0] = less[2 * i].in[0];      // 31 of 64
+    for (int i = 0; i < 64; i++) lens[i].in[0] = src, lens[i].count = chunk - i; // one address, 64 different lengths
+    for (int i = 0; i < (int)kRereadMaxSlices + 1; i++) many.push_back(fxSliceDesc{{src}, dst + i * chunk, chunk});
+    std::vector<fxSliceDesc> shuffled = ag;      // the order of the slices does not matter
+    for (size_t i = 0; i < shuffled.size(); i++) std::swap(shuffled[i], shuffled[(i * 37 + 11) % shuffled.size()]);
+    if (rereadHint(ag.data(), ag.size(), 1, 1) != kKeepAllLoads || rereadHint(shuffled.data(), shuffled.size(), 1, 2) != kKeepAllLoads ||
+        rereadHint(pack.data(), pack.size(), 1, 1) != 0 || rereadHint(half.data(), half.size(), 1, 4) != kKeepAllLoads ||
+        rereadHint(less.data(), less.size(), 1, 4) != 0 || rereadHint(lens.data(), lens.size(), 1, 1) != 0 ||
+        rereadHint(ag.data(), 1, 1, 1) != 0 || rereadHint(ag.data(), ag.size(), 2, 1) != 0 ||
+        rereadHint(many.data(), many.size(), 1, 1) != 0 || rereadHint(many.data(), kRereadMaxSlices, 1, 1) != kKeepAllLoads ||
+        touchedBytes(1000, 2, 8, 1) != 18000 || touchedBytes(3ull << 30, 8, 8, 8) != (3ull << 37)) {
+      printf("FAIL re-read detection\n");
+      return 1;
+    }
+    cases += 12;
+  }
   printf("ok %ld cases\n", cases);
   return 0;
 }

@@ -413,7 +413,9 @@ def test_kernel_index_arithmetic_on_the_host(tmp_path):
     functions the kernels themselves call -- over 14,168 (address, length, element
     size, unroll, hand-out, die shift) cases and checks that every vector of a segment
     is handled exactly once, the unchecked path only ever sees whole in-segment
-    vectors, and nothing outside the segment is touched."""
+    vectors, and nothing outside the segment is touched; then the host's decisions
+    around them: which segments are striped, and which batches of copies count as
+    reading their sources more than once (fx::rereadHint)."""
     import shutil
     import subprocess
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"

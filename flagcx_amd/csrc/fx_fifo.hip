@@ -405,65 +405,65 @@ fifoConsumer(uint64_t *host, FifoMirror *m, uint32_t cap, uint32_t inOrder, uint
     }
     const uint32_t batch = (uint32_t)sh[1];
     for (uint64_t takes = sh[2]; takes != 0; takes &= takes - 1) {
-    const uint32_t bi = (uint32_t)__builtin_ctzll(takes);
-    const void *in1 = (const void *)(uintptr_t)shTrig[bi][0], *in2 = (const void *)(uintptr_t)shTrig[bi][1];
-    void *out = (void *)(uintptr_t)shTrig[bi][2];
-    const uint64_t w3 = shTrig[bi][3] & ~kBulkBit;
-    const uint64_t count = w3 & 0xffffffffull;
-    const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
-    Share share;
-    share.idx = shIdx[bi];
-    share.takers = shTakers[bi];
-    // The trigger's buffers may have been written by other agents since this
-    // kernel last looked: drop stale cache lines before reading them.  Only a
-    // workgroup that takes tiles does so (every workgroup doing it for every batch
-    // it inspects costs more than a microsecond per round trip), and one wavefront
-    // does it for the workgroup: the caches are the compute unit's and the die's,
-    // and the barrier orders the other wavefronts' loads behind it.
-    if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-    __syncthreads();
-    bool ok = true;
-    if (count) {
-      switch (dtype) {
-        case flagcxFloat32: ok = runShareOp<flagcxFloat32>(op, in1, in2, out, count, share); break;
-        case flagcxInt32: ok = runShareOp<flagcxInt32>(op, in1, in2, out, count, share); break;
-        case flagcxBfloat16: ok = runShareOp<flagcxBfloat16>(op, in1, in2, out, count, share); break;
-        case flagcxFloat16: ok = runShareOp<flagcxFloat16>(op, in1, in2, out, count, share); break;
-        case flagcxUint32: ok = runShareOp<flagcxUint32>(op, in1, in2, out, count, share); break;
-        case flagcxInt8: ok = runShareOp<flagcxInt8>(op, in1, in2, out, count, share); break;
-        case flagcxUint8: ok = runShareOp<flagcxUint8>(op, in1, in2, out, count, share); break;
-        case flagcxInt64: ok = runShareOp<flagcxInt64>(op, in1, in2, out, count, share); break;
-        case flagcxUint64: ok = runShareOp<flagcxUint64>(op, in1, in2, out, count, share); break;
-        case flagcxFloat64: ok = runShareOp<flagcxFloat64>(op, in1, in2, out, count, share); break;
-        default: ok = false;
+      const uint32_t bi = (uint32_t)__builtin_ctzll(takes);
+      const void *in1 = (const void *)(uintptr_t)shTrig[bi][0], *in2 = (const void *)(uintptr_t)shTrig[bi][1];
+      void *out = (void *)(uintptr_t)shTrig[bi][2];
+      const uint64_t w3 = shTrig[bi][3] & ~kBulkBit;
+      const uint64_t count = w3 & 0xffffffffull;
+      const int dtype = (int)((w3 >> 48) & 0xf), op = (int)((w3 >> 52) & 0xf);
+      Share share;
+      share.idx = shIdx[bi];
+      share.takers = shTakers[bi];
+      // The trigger's buffers may have been written by other agents since this
+      // kernel last looked: drop stale cache lines before reading them.  Only a
+      // workgroup that takes tiles does so (every workgroup doing it for every batch
+      // it inspects costs more than a microsecond per round trip), and one wavefront
+      // does it for the workgroup: the caches are the compute unit's and the die's,
+      // and the barrier orders the other wavefronts' loads behind it.
+      if (threadIdx.x < 64) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+      __syncthreads();
+      bool ok = true;
+      if (count) {
+        switch (dtype) {
+          case flagcxFloat32: ok = runShareOp<flagcxFloat32>(op, in1, in2, out, count, share); break;
+          case flagcxInt32: ok = runShareOp<flagcxInt32>(op, in1, in2, out, count, share); break;
+          case flagcxBfloat16: ok = runShareOp<flagcxBfloat16>(op, in1, in2, out, count, share); break;
+          case flagcxFloat16: ok = runShareOp<flagcxFloat16>(op, in1, in2, out, count, share); break;
+          case flagcxUint32: ok = runShareOp<flagcxUint32>(op, in1, in2, out, count, share); break;
+          case flagcxInt8: ok = runShareOp<flagcxInt8>(op, in1, in2, out, count, share); break;
+          case flagcxUint8: ok = runShareOp<flagcxUint8>(op, in1, in2, out, count, share); break;
+          case flagcxInt64: ok = runShareOp<flagcxInt64>(op, in1, in2, out, count, share); break;
+          case flagcxUint64: ok = runShareOp<flagcxUint64>(op, in1, in2, out, count, share); break;
+          case flagcxFloat64: ok = runShareOp<flagcxFloat64>(op, in1, in2, out, count, share); break;
+          default: ok = false;
+        }
       }
-    }
-    // Every wavefront waits until its own stores are acknowledged (s_waitcnt
-    // vmcnt(0); a workgroup barrier alone does not make a wavefront wait for
-    // its vector stores), then the barrier collects the four of them.
-    waitVectorMemory();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      const uint32_t slot = (slotNow + bi) % cap;
-      // The results were stored through the caches (SegWT) and every wavefront
-      // waited for its stores before the barrier above, so they are in memory
-      // before this workgroup reports in: no cache write-back here (one per
-      // workgroup and trigger cost 7 us on a 16 MiB trigger).
-      const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (prev == share.takers - 1) {  // last one out completes the trigger
-        // Everybody else has counted in, so everybody's results are in memory; this
-        // thread reads none of them, and the counter is put back to zero by workgroup
-        // 0 when it next fills the slot: Complete can go out at once.  No cache-wide
-        // write-back or invalidate here -- either would stall every workgroup of this
-        // die that is busy with another trigger (0.78 against 1.3 us per 256 KiB
-        // trigger with the ring kept full).
-        if (!ok) __hip_atomic_fetch_add(&m->badTriggers, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(hostTrig + 4 * slot + 3, w3 | ((uint64_t)fxTriggerComplete << 56), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_SYSTEM);
-        __hip_atomic_fetch_add(&m->completed, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // Every wavefront waits until its own stores are acknowledged (s_waitcnt
+      // vmcnt(0); a workgroup barrier alone does not make a wavefront wait for
+      // its vector stores), then the barrier collects the four of them.
+      waitVectorMemory();
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        const uint32_t slot = (slotNow + bi) % cap;
+        // The results were stored through the caches (SegWT) and every wavefront
+        // waited for its stores before the barrier above, so they are in memory
+        // before this workgroup reports in: no cache write-back here (one per
+        // workgroup and trigger cost 7 us on a 16 MiB trigger).
+        const uint32_t prev = __hip_atomic_fetch_add(&m->done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (prev == share.takers - 1) {  // last one out completes the trigger
+          // Everybody else has counted in, so everybody's results are in memory; this
+          // thread reads none of them, and the counter is put back to zero by workgroup
+          // 0 when it next fills the slot: Complete can go out at once.  No cache-wide
+          // write-back or invalidate here -- either would stall every workgroup of this
+          // die that is busy with another trigger (0.78 against 1.3 us per 256 KiB
+          // trigger with the ring kept full).
+          if (!ok) __hip_atomic_fetch_add(&m->badTriggers, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(hostTrig + 4 * slot + 3, w3 | ((uint64_t)fxTriggerComplete << 56), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_SYSTEM);
+          __hip_atomic_fetch_add(&m->completed, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
-    }
-    }  // batch
+    }  // the triggers of this batch that this workgroup takes part in
     seq += batch;
     slotNow = (slotNow + batch) % cap;
     rot = (rot + batch * rotBy) % pool;

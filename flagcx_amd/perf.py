@@ -14,7 +14,9 @@ are used launch after launch, so whatever of them fits MI355X's 256 MiB
 memory-side cache is served from it.  With --cold (reduce, slices, pack) every
 timed launch is preceded by a 1 GiB fill with ordinary stores that pushes the
 operands out of that cache, and is timed by its own pair of events; both
-columns are printed.
+columns are printed.  reduce --fresh adds the case a reduction meets when it
+follows the kernel that made its operands: the inputs rewritten just before
+the timed launch, with the caches otherwise warm and after the 1 GiB fill.
 """
 import argparse
 import sys
@@ -65,19 +67,26 @@ class Timer:
 
     SCRUB_BYTES = 1 << 30
 
-    def ms_cold(self, fn, launches=9):
+    def ms_cold(self, fn, launches=9, scrub=True, produce=None):
         """Milliseconds per call when the caches hold nothing of the operands: before
         every timed call a 1 GiB fill with ordinary stores (the runtime's memset
         kernel, four times the memory-side cache) runs on the same stream; each call
-        is timed by its own pair of events; the median of `launches` calls."""
+        is timed by its own pair of events; the median of `launches` calls.
+        `produce` (a function that rewrites the inputs on the stream) runs after the
+        fill and before the timed call: the inputs are then what a kernel has just
+        written, as when a reduction follows the kernel that made its operands;
+        `scrub=False` leaves the fill out."""
         d = self.dev
-        if not hasattr(self, "scrub"):
+        if scrub and not hasattr(self, "scrub"):
             self.scrub = d.malloc(self.SCRUB_BYTES)
         fn()
         d.stream_sync(self.stream)
         each = []
         for i in range(launches):
-            d.memset(self.scrub, i & 0xff, self.SCRUB_BYTES, self.stream)
+            if scrub:
+                d.memset(self.scrub, i & 0xff, self.SCRUB_BYTES, self.stream)
+            if produce:
+                produce()
             e0, e1 = d.event_create(), d.event_create()
             d.event_record(e0, self.stream)
             fn()
@@ -88,17 +97,23 @@ class Timer:
             d.event_destroy(e1)
         return sorted(each)[len(each) // 2]
 
-    def both(self, fn, cold):
-        """(warm ms, cold ms or None)."""
-        return self.ms(fn), (self.ms_cold(fn) if cold else None)
+    def both(self, fn, cold, produce=None):
+        """(warm ms, cold ms or None), and with `produce` two more: (.., inputs just
+        written, 1 GiB fill and then the inputs written)."""
+        res = (self.ms(fn), (self.ms_cold(fn) if cold else None))
+        if produce:
+            res += (self.ms_cold(fn, scrub=False, produce=produce), self.ms_cold(fn, produce=produce))
+        return res
 
 
 def row(label, nbytes, ms, algo_bytes):
-    """ms: milliseconds, or (warm ms, cold ms or None) from Timer.both."""
-    warm, cold = ms if isinstance(ms, tuple) else (ms, None)
+    """ms: milliseconds, or the tuple from Timer.both."""
+    warm, cold = ms[:2] if isinstance(ms, tuple) else (ms, None)
     line = f"{label:<44s} size {nbytes:>12d} B   {warm * 1e3:10.2f} us   {algo_bytes / warm / 1e6:9.1f} GB/s"
     if cold is not None:
         line += f"   | cold {cold * 1e3:10.2f} us   {algo_bytes / cold / 1e6:9.1f} GB/s"
+    if isinstance(ms, tuple) and len(ms) == 4:
+        line += f"   | inputs fresh {ms[2] * 1e3:8.2f} us   | fill, then inputs fresh {ms[3] * 1e3:8.2f} us"
     print(line, flush=True)
 
 
@@ -125,7 +140,11 @@ def run_reduce(dev, a):
         fn = lambda: N.check(K.reduce_copy(out + (0 if a.inplace else a.misalign * es),
                                            [p + (a.misalign * es if not a.mixed else s) for p, s in zip(ins, shift)]
                                            if not a.inplace else ins, n, dtype, op, 0, t.raw))
-        row(f"reduce k={k} {a.dtype} {a.op}{' inplace' if a.inplace else ''}", nbytes, t.both(fn, a.cold), (k + 1) * nbytes)
+        produce = None
+        if a.fresh and not a.inplace:      # the inputs rewritten by a fill of their own before every timed launch
+            produce = lambda: [dev.memset(p, 0x3c + i, nbytes + a.misalign * es, t.stream) for i, p in enumerate(ins)]
+        row(f"reduce k={k} {a.dtype} {a.op}{' inplace' if a.inplace else ''}", nbytes, t.both(fn, a.cold, produce),
+            (k + 1) * nbytes)
         nbytes *= a.factor
 
 
@@ -468,6 +487,9 @@ def main(argv=None):
     ap.add_argument("what", choices=["reduce", "slices", "pack", "allreduce", "fifo", "collectives", "torchref", "coldstart"])
     ap.add_argument("--cold", action="store_true",
                     help="reduce / slices / pack: also time every launch after a 1 GiB fill that empties the caches")
+    ap.add_argument("--fresh", action="store_true",
+                    help="reduce: two more columns, every launch timed right after its inputs were rewritten on the "
+                         "same stream -- without and with the 1 GiB fill before that")
     ap.add_argument("-k", type=int, default=4)
     ap.add_argument("-n", "--nranks", type=int, default=8)
     ap.add_argument("-d", "--dtype", default="fp32", choices=list(DT))

@@ -412,13 +412,29 @@ def run_torchref():
             best = min(best, e0.elapsed_time(e1) / iters)
         return best
 
+    scrub = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+
+    def cold_ms_of(fn, launches=9):
+        """As Timer.ms_cold: every launch behind a 1 GiB fill, timed by its own pair of events; the median."""
+        each = []
+        for i in range(launches):
+            scrub.fill_(i)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            e1.synchronize()
+            each.append(e0.elapsed_time(e1))
+        return sorted(each)[len(each) // 2]
+
     for dt, es in ((torch.float32, 4), (torch.bfloat16, 2)):
-        for mib in (64, 256, 512):
+        for mib in (16, 64, 256, 512):
             n = (mib << 20) // es
             a, b = torch.randn(n, device="cuda").to(dt), torch.randn(n, device="cuda").to(dt)
             c = torch.empty_like(a)
-            row(f"torch.add(a, b, out=c) {str(dt)[6:]}", mib << 20, ms_of(lambda: torch.add(a, b, out=c), 50), 3 * (mib << 20))
-            row(f"c.copy_(a) {str(dt)[6:]}", mib << 20, ms_of(lambda: c.copy_(a), 50), 2 * (mib << 20))
+            add, copy = (lambda: torch.add(a, b, out=c)), (lambda: c.copy_(a))
+            row(f"torch.add(a, b, out=c) {str(dt)[6:]}", mib << 20, (ms_of(add, 50), cold_ms_of(add)), 3 * (mib << 20))
+            row(f"c.copy_(a) {str(dt)[6:]}", mib << 20, (ms_of(copy, 50), cold_ms_of(copy)), 2 * (mib << 20))
             del a, b, c
     n = (512 << 20) // 2
     xs = [torch.randn(n, device="cuda").to(torch.bfloat16) for _ in range(8)]

@@ -40,8 +40,14 @@ inline uint64_t vectorsOf(uint64_t count, int es) { return (count * (uint64_t)es
 // SLOWER than nontemporal ones from 4 MiB to 256 MiB per input (two fp32
 // inputs of 64 MiB: 57 against 34 us; eight bf16 inputs of 16 MiB: 51 against
 // 30 us), and with the operands cached they are within +-10 % of them, better
-// at some sizes and worse at others.  Ordinary stores are never better.  So the
-// operands' size alone does not choose ordinary accesses.  What does:
+// at some sizes and worse at others.  (The fill leaves the caches full of dirty
+// lines, and a load that allocates a line evicts one: a write to memory per
+// line read.  Behind caches full of clean lines the two kinds of load take the
+// same time, and inputs that were written just before the launch and fit the
+// memory-side cache are read 8-10 % faster with ordinary loads.)  Ordinary
+// stores are never better.  The loss is several times the gain, and a launch
+// cannot know what the caches hold, so the operands' size alone does not choose
+// ordinary accesses.  What does:
 //  * a launch that reads the same bytes more than once -- the all-gather copy
 //    phase hands one source chunk to every other rank, seven copies of it --
 //    reads with ordinary loads, so that the later readers find the chunk in a

@@ -217,6 +217,12 @@ def run_pack(dev, a):
     print("counts", counts, "sdispls % 4 el:", [d % 4 for d in sd], "slots % 4:", [int(x) % 4 for x in np.cumsum([0] + counts[:-1])])
     row("pack   (config 4 layout)", total * 4, t.both(lambda: N.check(K.pack(dpacked, dsend, counts, sd, N.DT_FP32, t.raw)), a.cold), 2 * total * 4)
     row("unpack (config 4 layout)", total * 4, t.both(lambda: N.check(K.unpack(drecv, dpacked, counts, rd, N.DT_FP32, t.raw)), a.cold), 2 * total * 4)
+    # the two phases as one step: two dependent launches, eagerly and as one replayed graph of two kernel nodes
+    both = lambda: (N.check(K.pack(dpacked, dsend, counts, sd, N.DT_FP32, t.raw)),
+                    N.check(K.unpack(drecv, dpacked, counts, rd, N.DT_FP32, t.raw)))
+    row("pack + unpack, two launches", 2 * total * 4, t.ms(both), 4 * total * 4)
+    row("pack + unpack, one graph of two nodes", 2 * total * 4, t.ms(_replay_of(t, both)), 4 * total * 4)
+    row("4 x (pack + unpack), one graph", 8 * total * 4, t.ms(_replay_of(t, both, 4)), 16 * total * 4)
     c4 = [c // 4 * 4 for c in counts]
     s4 = [d // 4 * 4 for d in sd]
     row("pack, counts/displs multiples of 16 B", sum(c4) * 4, t.ms(lambda: N.check(K.pack(dpacked, dsend, c4, s4, N.DT_FP32, t.raw))), 2 * sum(c4) * 4)

@@ -685,7 +685,7 @@ int fx_plan_create(fxPlan_t *plan, const fxSliceDesc *slices, size_t n, int k, i
     pl->k = k;
     pl->n = (uint32_t)desc.size();
     pl->grid = start.back();
-    pl->keep = cachePolicyFor(touchedBytes(elems, ks->elemSize, k, 1),
+    pl->keep = cachePolicyFor(touchedBytes(elems, ks->elemSize, k, 0), touchedBytes(elems, ks->elemSize, 0, 1),
                               rereadHint(merged.data(), merged.size(), k, (size_t)ks->elemSize));
     pl->dDesc = nullptr;
     pl->dTileStart = nullptr;
@@ -796,7 +796,8 @@ int fx_reduce_slices_static(const fxSliceDesc *slices, size_t n, int k, int dtyp
   if (rc) return rc;
   rc = flush();
   if (rc) return rc;
-  return ks->slicesTable[k](dDesc, dTileStart, (uint32_t)entries, next, cachePolicyFor(touchedBytes(elems, (int)es, k, 1)), s);
+  const uint32_t keep = cachePolicyFor(touchedBytes(elems, (int)es, k, 0), touchedBytes(elems, (int)es, 0, 1));
+  return ks->slicesTable[k](dDesc, dTileStart, (uint32_t)entries, next, keep, s);
 }
 
 static int packOrUnpack(bool pack, void *a, const void *b, const size_t *counts, const size_t *displs, int npeers,

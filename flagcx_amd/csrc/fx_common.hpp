@@ -146,21 +146,24 @@ __device__ __forceinline__ u32x4 ldg_keep(const void *p) {
 __device__ __forceinline__ void stg_stream(void *p, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
 }
-// A store without the streaming hint, for results that the next kernel reads
-// while they still fit the caches.  A buffer store for the same reason as
-// ldg_keep is a buffer load.
+// A write-back store at agent scope (sc1, no streaming hint): the line stays in
+// the caches for whoever reads the result next.  For launches whose results fit
+// the memory-side cache these are faster than the streaming ones (and than
+// stores without a scope, which a plain assignment would give).  A buffer store:
+// the instruction carries the scope bit.
 __device__ __forceinline__ void stg_keep(void *p, u32x4 v) {
   const uint64_t a = (uint64_t)(uintptr_t)p;
   const uint64_t base = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
                         ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
   __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)base, 0, 0x7fffffff, 0x00020000);
-  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4_raw, v), rsrc, (int)(uint32_t)(a - base), 0, 0);
+  constexpr int kSc1 = 16;   // agent scope
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4_raw, v), rsrc, (int)(uint32_t)(a - base), 0, kSc1);
 }
 
 // Cache policy of one launch, decided on the host from the bytes the launch
-// touches (see cachePolicyFor in fx_launch.hpp) and carried in the kernel
-// arguments: bit p (p < 8) = input p is read with ordinary loads, kKeepStores =
-// results are written with ordinary stores.  Zero = everything streams.
+// reads and writes (see cachePolicyFor in fx_launch.hpp) and carried in the
+// kernel arguments: bit p (p < 8) = input p is read with ordinary loads,
+// kKeepStores = results are written with stg_keep.  Zero = everything streams.
 constexpr uint32_t kKeepAllLoads = 0xffu;
 constexpr uint32_t kKeepStores = 0x100u;
 

@@ -33,21 +33,20 @@ inline uint64_t vectorsOf(uint64_t count, int es) { return (count * (uint64_t)es
 
 // ---- cache policy of a launch ----
 //
-// Every byte of a reduction is used once, so by default loads and stores are
-// nontemporal: they stream past the 4 MiB L2 of each die and the 256 MiB
-// memory-side cache behind them.  Measured on MI355X with every launch preceded
-// by a 1 GiB fill (nothing of the operands cached), ordinary loads are 40-70 %
-// SLOWER than nontemporal ones from 4 MiB to 256 MiB per input (two fp32
-// inputs of 64 MiB: 57 against 34 us; eight bf16 inputs of 16 MiB: 51 against
-// 30 us), and with the operands cached they are within +-10 % of them, better
-// at some sizes and worse at others.  (The fill leaves the caches full of dirty
-// lines, and a load that allocates a line evicts one: a write to memory per
-// line read.  Behind caches full of clean lines the two kinds of load take the
-// same time, and inputs that were written just before the launch and fit the
-// memory-side cache are read 8-10 % faster with ordinary loads.)  Ordinary
-// stores are never better.  The loss is several times the gain, and a launch
-// cannot know what the caches hold, so the operands' size alone does not choose
-// ordinary accesses.  What does:
+// Loads.  Every byte of a reduction is used once, so loads are nontemporal:
+// they stream past the 4 MiB L2 of each die and the 256 MiB memory-side cache
+// behind them.  Measured on MI355X with every launch preceded by a 1 GiB fill
+// (nothing of the operands cached), ordinary loads are 40-70 % SLOWER than
+// nontemporal ones from 4 MiB to 256 MiB per input (two fp32 inputs of 64 MiB:
+// 57 against 34 us; eight bf16 inputs of 16 MiB: 51 against 30 us), and with the
+// operands cached they are within +-10 % of them, better at some sizes and worse
+// at others.  (The fill leaves the caches full of dirty lines, and a load that
+// allocates a line evicts one: a write to memory per line read.  Behind caches
+// full of clean lines the two kinds of load take the same time, and inputs that
+// were written just before the launch and fit the memory-side cache are read
+// 8-10 % faster with ordinary loads.)  The loss is several times the gain, and
+// a launch cannot know what the caches hold, so the operands' size alone does
+// not choose ordinary loads.  What does:
 //  * a launch that reads the same bytes more than once -- the all-gather copy
 //    phase hands one source chunk to every other rank, seven copies of it --
 //    reads with ordinary loads, so that the later readers find the chunk in a
@@ -55,9 +54,25 @@ inline uint64_t vectorsOf(uint64_t count, int es) { return (count * (uint64_t)es
 //    cold); the batch entry points detect that (rereadHint);
 //  * FX_TEMPORAL_MAX_BYTES (environment, read once; default 0 = never) makes
 //    every launch that touches no more than that many bytes use ordinary loads,
-//    for a caller who knows that its operands are cache-resident;
-//  * FX_CACHE_POLICY = stream | keep | keep-loads | keep-stores forces one
-//    policy for every launch (measurements).
+//    for a caller who knows that its operands are cache-resident.
+// Stores.  A launch in which stores are at least half of the traffic (copies,
+// pack / unpack, the one-read-n-stores collectives) and which writes no more
+// than the memory-side cache holds (kCachedStoreMaxBytes) leaves its results
+// there -- write-back stores at agent scope, stg_keep -- for whoever reads them
+// next; everything else streams its results (nontemporal stores).  Measured
+// against nontemporal stores, same box, alternating: alltoallv pack of 19.6 MB
+// 6.2 against 7.4 us and unpack 6.2 against 7.6 (behind a 1 GiB fill 15.5
+// against 15.0 and 14.9 against 15.1), seven copies of 8 MiB 16.8 against
+// 18.7 us, an eight-rank all-reduce of 16 MiB per rank 46.1 against 50.1 us and
+// all-gather 26.4 against 27.7 (behind a fill both within 0.5 %).  Reductions
+// into one output gain 1-10 % by them when the same buffers are used over and
+// over -- the output is then never written to memory at all, which a benchmark
+// loop rewards and an application does not -- and lose 1-6 % behind a fill, so
+// they stream.  Above the limit cached stores lose 0.3-2.4 % (eight inputs of
+// 512 MiB: 741 against 736 us).  Plain stores without a scope (what a C++
+// assignment compiles to) are slower than either everywhere.
+// FX_CACHE_POLICY = stream | keep | keep-loads | keep-stores forces one policy
+// for every launch (measurements).
 struct CachePolicyConfig {
   uint64_t maxBytes;
   int forced;        // -1: by the rules above; otherwise the policy bits for every launch
@@ -77,11 +92,13 @@ inline CachePolicyConfig readCachePolicyConfig() {
   }
   return c;
 }
+constexpr uint64_t kCachedStoreMaxBytes = 256ull << 20;   // the memory-side cache
 // `hint`: policy bits the caller has a reason for (rereadHint).
-inline uint32_t cachePolicyFor(uint64_t bytesTouched, uint32_t hint = 0) {
+inline uint32_t cachePolicyFor(uint64_t bytesRead, uint64_t bytesWritten, uint32_t hint = 0) {
   static const CachePolicyConfig cfg = readCachePolicyConfig();
   if (cfg.forced >= 0) return (uint32_t)cfg.forced;
-  return hint | (bytesTouched <= cfg.maxBytes ? kKeepAllLoads : 0u);
+  return hint | (bytesRead + bytesWritten <= cfg.maxBytes ? kKeepAllLoads : 0u) |
+         (bytesWritten >= bytesRead && bytesWritten <= kCachedStoreMaxBytes ? kKeepStores : 0u);
 }
 // Bytes a reduction of `count` elements of `es` bytes touches: k inputs, nout outputs.
 inline uint64_t touchedBytes(uint64_t count, int es, int k, int nout) {
@@ -156,7 +173,7 @@ flagcxResult_t launchDirectU(void *out, const void *const *in, int k, uint64_t c
   a.out = out;
   a.count = count;
   a.k = kk;
-  a.keep = cachePolicyFor(touchedBytes(count, R::ES, kk, 1));
+  a.keep = cachePolicyFor(touchedBytes(count, R::ES, kk, 0), touchedBytes(count, R::ES, 0, 1));
   uint64_t ntiles = tilesFor(out, in, kk, count, R::ES, U);
   if (ntiles == 0) return flagcxSuccess;
   if (ntiles > 0x7ffffff0ull) return flagcxInvalidArgument;
@@ -211,7 +228,7 @@ flagcxResult_t launchSlicesInline(const fxSliceDesc *slices, size_t n, uint32_t 
     vecs += vectorsOf(slices[i].count, R::ES);
     elems += slices[i].count;
   }
-  const uint32_t keep = cachePolicyFor(touchedBytes(elems, R::ES, K, 1), hint);
+  const uint32_t keep = cachePolicyFor(touchedBytes(elems, R::ES, K, 0), touchedBytes(elems, R::ES, 0, 1), hint);
   if constexpr (LEAN) return launchSlicesInlineSized<R, K, UD, kSmallSliceTable>(slices, n, keep, s);
   if (n > (size_t)kSmallSliceTable) return launchSlicesInlineSized<R, K, UD, 0>(slices, n, keep, s);
   if constexpr (US != UD)
@@ -271,13 +288,14 @@ flagcxResult_t launchBcastMany(const BcastDescDev *d, size_t n, uint32_t keep, h
 }
 
 inline uint32_t bcastPolicy(const BcastDescDev *d, size_t n, int es, int k, uint64_t *vecsPerOutput) {
-  uint64_t vecs = 0, bytes = 0;
+  uint64_t vecs = 0, read = 0, written = 0;
   for (size_t i = 0; i < n; i++) {
     vecs += vectorsOf(d[i].count, es);
-    bytes += touchedBytes(d[i].count, es, k, (int)d[i].nout);
+    read += touchedBytes(d[i].count, es, k, 0);
+    written += touchedBytes(d[i].count, es, 0, (int)d[i].nout);
   }
   *vecsPerOutput = vecs;
-  return cachePolicyFor(bytes);
+  return cachePolicyFor(read, written);
 }
 
 template <class R, int K, bool LEAN>
@@ -307,7 +325,7 @@ flagcxResult_t launchBcastRuntimeU(void *const *out, int nout, const void *const
   a.count = count;
   a.k = k;
   a.nout = nout;
-  a.keep = cachePolicyFor(touchedBytes(count, R::ES, k, nout));
+  a.keep = cachePolicyFor(touchedBytes(count, R::ES, k, 0), touchedBytes(count, R::ES, 0, nout));
   if (count == 0) return flagcxSuccess;
   a.co = coAlignedHost(out[0], in, k, out + 1, nout - 1) ? 1 : 0;
   const uint64_t ntiles = planTiles((uint64_t)(uintptr_t)out[0], count, R::ES, U, handOutFor(a.co != 0, k)).tiles();
@@ -327,17 +345,18 @@ flagcxResult_t launchBcastRuntime(void *const *out, int nout, const void *const 
 
 template <class R, int U>
 flagcxResult_t launchChunksRuntimeU(ChunkedArgs *a, hipStream_t s) {
-  uint64_t total = 0, bytes = 0;
+  uint64_t total = 0, read = 0, written = 0;
   a->tileStart[0] = 0;
   for (int c = 0; c < a->nchunks; c++) {
     a->co[c] = chunkCoAligned(*a, c) ? 1 : 0;
     total += a->cnt[c] ? chunkPlan<R::ES, U>(*a, c).tiles() : 0;
     if (total > 0x7ffffff0ull) return flagcxInvalidArgument;
     a->tileStart[c + 1] = (uint32_t)total;
-    bytes += touchedBytes(a->cnt[c], R::ES, a->only[c] >= 0 ? 1 : a->k, a->outSel[c] >= 0 ? 1 : a->nout);
+    read += touchedBytes(a->cnt[c], R::ES, a->only[c] >= 0 ? 1 : a->k, 0);
+    written += touchedBytes(a->cnt[c], R::ES, 0, a->outSel[c] >= 0 ? 1 : a->nout);
   }
   if (total == 0) return flagcxSuccess;
-  a->keep = cachePolicyFor(bytes);
+  a->keep = cachePolicyFor(read, written);
   return launchKernel(reduceChunksRuntime<R, U>, (uint32_t)total, s, *a);
 }
 
@@ -362,7 +381,8 @@ flagcxResult_t launchAllToAllU(void *const *recv, const void *const *send, int n
   }
   a.blockElems = blockElems;
   a.n = n;
-  a.keep = cachePolicyFor(touchedBytes(blockElems * (uint64_t)n * (uint64_t)n, R::ES, 1, 1));
+  const uint64_t moved = touchedBytes(blockElems * (uint64_t)n * (uint64_t)n, R::ES, 1, 0);
+  a.keep = cachePolicyFor(moved, moved);
   const uint64_t V = (uint64_t)U * kBlock, nv = vectorsOf(blockElems, R::ES) + 1;   // + 1: a block off 16-byte alignment spans one vector more
   const uint64_t striped = blockElems * (uint64_t)R::ES >= kStripeMinBytes ? 2 : 0;   // shorter blocks have no regions
   const uint64_t per = (nv + V - 1) / V + striped, total = per * (uint64_t)n * (uint64_t)n;

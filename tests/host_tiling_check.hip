@@ -132,7 +132,14 @@ int main() {
         rereadHint(less.data(), less.size(), 1, 4) != 0 || rereadHint(lens.data(), lens.size(), 1, 1) != 0 ||
         rereadHint(ag.data(), 1, 1, 1) != 0 || rereadHint(ag.data(), ag.size(), 2, 1) != 0 ||
         rereadHint(many.data(), many.size(), 1, 1) != 0 || rereadHint(many.data(), kRereadMaxSlices, 1, 1) != kKeepAllLoads ||
-        touchedBytes(1000, 2, 8, 1) != 18000 || touchedBytes(3ull << 30, 8, 8, 8) != (3ull << 37)) {
+        touchedBytes(1000, 2, 8, 1) != 18000 || touchedBytes(3ull << 30, 8, 8, 8) != (3ull << 37) ||
+        // store-heavy launches whose results fit the memory-side cache leave them there; reductions into one output
+        // and larger results stream (no forced policy in this process)
+        (getenv("FX_CACHE_POLICY") == nullptr && getenv("FX_TEMPORAL_MAX_BYTES") == nullptr &&
+         (cachePolicyFor(256ull << 20, 256ull << 20) != kKeepStores || cachePolicyFor(256ull << 20, (256ull << 20) + 1) != 0 ||
+          cachePolicyFor((256ull << 20) + 1, 256ull << 20) != 0 || cachePolicyFor(8ull << 20, 1ull << 20) != 0 ||
+          cachePolicyFor(1ull << 20, 8ull << 20) != kKeepStores ||
+          cachePolicyFor(1, 1, kKeepAllLoads) != (kKeepAllLoads | kKeepStores)))) {
       printf("FAIL re-read detection\n");
       return 1;
     }
